@@ -1,0 +1,257 @@
+/*
+ * Public device API: the reference's names stamped over the templates of nvshmemi_device.h.
+ *   thread scope  nvshmem_*            reference src/include/device/nvshmem_defines.h:80-740
+ *   warp / block  nvshmemx_*_{warp,block}  reference src/include/device/nvshmemx_defines.h:35-451
+ *   collectives   reference src/include/device/nvshmem_coll_defines.cuh:17-116,
+ *                 src/include/device/nvshmemx_coll_defines.cuh:16-175
+ * "_warp" means one 64-lane wavefront here.  Device functions share their names with the host
+ * entry points; hipcc keeps the two apart by target.
+ */
+#ifndef NVSHMEM_AMD_DEVICE_API_H
+#define NVSHMEM_AMD_DEVICE_API_H
+
+#include "nvshmemi_device.h"
+
+#define NVSHMEMI_DEV static __device__ __forceinline__
+
+/* ---- identity and translation ---- */
+NVSHMEMI_DEV int nvshmem_my_pe(void) { return nvshmemi_amd_my_pe(); }
+NVSHMEMI_DEV int nvshmem_n_pes(void) { return nvshmemi_amd_n_pes(); }
+NVSHMEMI_DEV int nvshmem_team_my_pe(nvshmem_team_t) { return nvshmemi_amd_my_pe(); }
+NVSHMEMI_DEV int nvshmem_team_n_pes(nvshmem_team_t) { return nvshmemi_amd_n_pes(); }
+NVSHMEMI_DEV void *nvshmem_ptr(const void *ptr, int pe) { return nvshmemi_ptr(ptr, pe); }
+
+/* ---- ordering ---- */
+NVSHMEMI_DEV void nvshmem_quiet(void) { nvshmemi_quiet<NVSHMEMI_THREADGROUP_THREAD>(); }
+NVSHMEMI_DEV void nvshmem_fence(void) { nvshmemi_quiet<NVSHMEMI_THREADGROUP_THREAD>(); }
+NVSHMEMI_DEV void nvshmemx_quiet_warp(void) { nvshmemi_quiet<NVSHMEMI_THREADGROUP_WARP>(); }
+NVSHMEMI_DEV void nvshmemx_quiet_block(void) { nvshmemi_quiet<NVSHMEMI_THREADGROUP_BLOCK>(); }
+
+/* ---- barrier / sync over all PEs: one thread group per PE calls ---- */
+#define NVSHMEMI_STAMP_BARRIER(PFX, SFX, SC)                                                     \
+    NVSHMEMI_DEV void PFX##_barrier_all##SFX(void) { nvshmemi_barrier_threadgroup<SC>(); }       \
+    NVSHMEMI_DEV int PFX##_barrier##SFX(nvshmem_team_t) {                                        \
+        nvshmemi_barrier_threadgroup<SC>();                                                      \
+        return 0;                                                                                \
+    }                                                                                            \
+    NVSHMEMI_DEV void PFX##_sync_all##SFX(void) { nvshmemi_sync_threadgroup<SC>(); }             \
+    NVSHMEMI_DEV int PFX##_team_sync##SFX(nvshmem_team_t) {                                      \
+        nvshmemi_sync_threadgroup<SC>();                                                         \
+        return 0;                                                                                \
+    }
+NVSHMEMI_STAMP_BARRIER(nvshmem, , NVSHMEMI_THREADGROUP_THREAD)
+NVSHMEMI_STAMP_BARRIER(nvshmemx, _warp, NVSHMEMI_THREADGROUP_WARP)
+NVSHMEMI_STAMP_BARRIER(nvshmemx, _block, NVSHMEMI_THREADGROUP_BLOCK)
+#undef NVSHMEMI_STAMP_BARRIER
+
+/* ---- byte RMA ---- */
+#define NVSHMEMI_STAMP_MEM_RMA(PFX, SFX, SC)                                                      \
+    NVSHMEMI_DEV void PFX##_putmem##SFX(void *dest, const void *source, size_t bytes, int pe) {   \
+        nvshmemi_put<char, SC>((char *)dest, (const char *)source, bytes, pe);                    \
+    }                                                                                             \
+    NVSHMEMI_DEV void PFX##_getmem##SFX(void *dest, const void *source, size_t bytes, int pe) {   \
+        nvshmemi_get<char, SC>((char *)dest, (const char *)source, bytes, pe);                    \
+    }                                                                                             \
+    NVSHMEMI_DEV void PFX##_putmem_nbi##SFX(void *dest, const void *source, size_t bytes,         \
+                                            int pe) {                                             \
+        nvshmemi_put<char, SC>((char *)dest, (const char *)source, bytes, pe);                    \
+    }                                                                                             \
+    NVSHMEMI_DEV void PFX##_getmem_nbi##SFX(void *dest, const void *source, size_t bytes,         \
+                                            int pe) {                                             \
+        nvshmemi_get<char, SC>((char *)dest, (const char *)source, bytes, pe);                    \
+    }                                                                                             \
+    NVSHMEMI_DEV void PFX##_putmem_signal##SFX(void *dest, const void *source, size_t bytes,      \
+                                               uint64_t *sig_addr, uint64_t signal, int sig_op,   \
+                                               int pe) {                                          \
+        nvshmemi_put_signal<char, SC>((char *)dest, (const char *)source, bytes, sig_addr,        \
+                                      signal, sig_op, pe);                                        \
+    }                                                                                             \
+    NVSHMEMI_DEV void PFX##_putmem_signal_nbi##SFX(void *dest, const void *source, size_t bytes,  \
+                                                   uint64_t *sig_addr, uint64_t signal,           \
+                                                   int sig_op, int pe) {                          \
+        nvshmemi_put_signal<char, SC>((char *)dest, (const char *)source, bytes, sig_addr,        \
+                                      signal, sig_op, pe);                                        \
+    }
+NVSHMEMI_STAMP_MEM_RMA(nvshmem, , NVSHMEMI_THREADGROUP_THREAD)
+NVSHMEMI_STAMP_MEM_RMA(nvshmemx, _warp, NVSHMEMI_THREADGROUP_WARP)
+NVSHMEMI_STAMP_MEM_RMA(nvshmemx, _block, NVSHMEMI_THREADGROUP_BLOCK)
+#undef NVSHMEMI_STAMP_MEM_RMA
+
+/* ---- typed RMA: 25 types x 3 scopes ---- */
+#define NVSHMEMI_STAMP_TYPED_RMA_SCOPE(NAME, TYPE, PFX, SFX, SC)                                  \
+    NVSHMEMI_DEV void PFX##_##NAME##_put##SFX(TYPE *dest, const TYPE *source, size_t nelems,      \
+                                              int pe) {                                           \
+        nvshmemi_put<TYPE, SC>(dest, source, nelems, pe);                                         \
+    }                                                                                             \
+    NVSHMEMI_DEV void PFX##_##NAME##_get##SFX(TYPE *dest, const TYPE *source, size_t nelems,      \
+                                              int pe) {                                           \
+        nvshmemi_get<TYPE, SC>(dest, source, nelems, pe);                                         \
+    }                                                                                             \
+    NVSHMEMI_DEV void PFX##_##NAME##_put_nbi##SFX(TYPE *dest, const TYPE *source, size_t nelems,  \
+                                                  int pe) {                                       \
+        nvshmemi_put<TYPE, SC>(dest, source, nelems, pe);                                         \
+    }                                                                                             \
+    NVSHMEMI_DEV void PFX##_##NAME##_get_nbi##SFX(TYPE *dest, const TYPE *source, size_t nelems,  \
+                                                  int pe) {                                       \
+        nvshmemi_get<TYPE, SC>(dest, source, nelems, pe);                                         \
+    }                                                                                             \
+    NVSHMEMI_DEV void PFX##_##NAME##_iput##SFX(TYPE *dest, const TYPE *source, ptrdiff_t dst,     \
+                                               ptrdiff_t sst, size_t nelems, int pe) {            \
+        nvshmemi_iput<TYPE, SC>(dest, source, dst, sst, nelems, pe);                              \
+    }                                                                                             \
+    NVSHMEMI_DEV void PFX##_##NAME##_iget##SFX(TYPE *dest, const TYPE *source, ptrdiff_t dst,     \
+                                               ptrdiff_t sst, size_t nelems, int pe) {            \
+        nvshmemi_iget<TYPE, SC>(dest, source, dst, sst, nelems, pe);                              \
+    }                                                                                             \
+    NVSHMEMI_DEV void PFX##_##NAME##_put_signal##SFX(TYPE *dest, const TYPE *source,              \
+                                                     size_t nelems, uint64_t *sig_addr,           \
+                                                     uint64_t signal, int sig_op, int pe) {       \
+        nvshmemi_put_signal<TYPE, SC>(dest, source, nelems, sig_addr, signal, sig_op, pe);        \
+    }                                                                                             \
+    NVSHMEMI_DEV void PFX##_##NAME##_put_signal_nbi##SFX(TYPE *dest, const TYPE *source,          \
+                                                         size_t nelems, uint64_t *sig_addr,       \
+                                                         uint64_t signal, int sig_op, int pe) {   \
+        nvshmemi_put_signal<TYPE, SC>(dest, source, nelems, sig_addr, signal, sig_op, pe);        \
+    }
+#define NVSHMEMI_STAMP_TYPED_RMA(NAME, TYPE, TAG)                                                 \
+    NVSHMEMI_DEV void nvshmem_##NAME##_p(TYPE *dest, const TYPE value, int pe) {                  \
+        nvshmemi_p<TYPE>(dest, value, pe);                                                        \
+    }                                                                                             \
+    NVSHMEMI_DEV TYPE nvshmem_##NAME##_g(const TYPE *source, int pe) {                            \
+        return nvshmemi_g<TYPE>(source, pe);                                                      \
+    }                                                                                             \
+    NVSHMEMI_STAMP_TYPED_RMA_SCOPE(NAME, TYPE, nvshmem, , NVSHMEMI_THREADGROUP_THREAD)            \
+    NVSHMEMI_STAMP_TYPED_RMA_SCOPE(NAME, TYPE, nvshmemx, _warp, NVSHMEMI_THREADGROUP_WARP)        \
+    NVSHMEMI_STAMP_TYPED_RMA_SCOPE(NAME, TYPE, nvshmemx, _block, NVSHMEMI_THREADGROUP_BLOCK)
+NVSHMEMI_REPT_FOR_STANDARD_RMA_TYPES(NVSHMEMI_STAMP_TYPED_RMA)
+#undef NVSHMEMI_STAMP_TYPED_RMA
+#undef NVSHMEMI_STAMP_TYPED_RMA_SCOPE
+
+/* ---- sized RMA put8..put128: nelems elements of BITS/8 bytes ---- */
+#define NVSHMEMI_STAMP_SIZED_RMA_SCOPE(BITS, BYTES, PFX, SFX, SC)                                 \
+    NVSHMEMI_DEV void PFX##_put##BITS##SFX(void *dest, const void *source, size_t nelems,         \
+                                           int pe) {                                              \
+        nvshmemi_put<char, SC>((char *)dest, (const char *)source, nelems * BYTES, pe);           \
+    }                                                                                             \
+    NVSHMEMI_DEV void PFX##_get##BITS##SFX(void *dest, const void *source, size_t nelems,         \
+                                           int pe) {                                              \
+        nvshmemi_get<char, SC>((char *)dest, (const char *)source, nelems * BYTES, pe);           \
+    }                                                                                             \
+    NVSHMEMI_DEV void PFX##_put##BITS##_nbi##SFX(void *dest, const void *source, size_t nelems,   \
+                                                 int pe) {                                        \
+        nvshmemi_put<char, SC>((char *)dest, (const char *)source, nelems * BYTES, pe);           \
+    }                                                                                             \
+    NVSHMEMI_DEV void PFX##_get##BITS##_nbi##SFX(void *dest, const void *source, size_t nelems,   \
+                                                 int pe) {                                        \
+        nvshmemi_get<char, SC>((char *)dest, (const char *)source, nelems * BYTES, pe);           \
+    }                                                                                             \
+    NVSHMEMI_DEV void PFX##_put##BITS##_signal##SFX(void *dest, const void *source,               \
+                                                    size_t nelems, uint64_t *sig_addr,            \
+                                                    uint64_t signal, int sig_op, int pe) {        \
+        nvshmemi_put_signal<char, SC>((char *)dest, (const char *)source, nelems * BYTES,         \
+                                      sig_addr, signal, sig_op, pe);                              \
+    }                                                                                             \
+    NVSHMEMI_DEV void PFX##_put##BITS##_signal_nbi##SFX(void *dest, const void *source,           \
+                                                        size_t nelems, uint64_t *sig_addr,        \
+                                                        uint64_t signal, int sig_op, int pe) {    \
+        nvshmemi_put_signal<char, SC>((char *)dest, (const char *)source, nelems * BYTES,         \
+                                      sig_addr, signal, sig_op, pe);                              \
+    }
+#define NVSHMEMI_STAMP_SIZED_RMA(BITS, BYTES)                                                     \
+    NVSHMEMI_STAMP_SIZED_RMA_SCOPE(BITS, BYTES, nvshmem, , NVSHMEMI_THREADGROUP_THREAD)           \
+    NVSHMEMI_STAMP_SIZED_RMA_SCOPE(BITS, BYTES, nvshmemx, _warp, NVSHMEMI_THREADGROUP_WARP)       \
+    NVSHMEMI_STAMP_SIZED_RMA_SCOPE(BITS, BYTES, nvshmemx, _block, NVSHMEMI_THREADGROUP_BLOCK)
+NVSHMEMI_REPT_FOR_SIZES(NVSHMEMI_STAMP_SIZED_RMA)
+#undef NVSHMEMI_STAMP_SIZED_RMA
+#undef NVSHMEMI_STAMP_SIZED_RMA_SCOPE
+
+/* ---- signals ---- */
+NVSHMEMI_DEV void nvshmemx_signal_op(uint64_t *sig_addr, uint64_t signal, int sig_op, int pe) {
+    nvshmemi_signal_op_release(sig_addr, signal, sig_op, pe);
+}
+NVSHMEMI_DEV uint64_t nvshmem_signal_fetch(uint64_t *sig_addr) {
+    return nvshmemi_amd_poll(reinterpret_cast<const uint64_t *>(nvshmemi_amd_local(sig_addr)));
+}
+NVSHMEMI_DEV uint64_t nvshmem_signal_wait_until(uint64_t *sig_addr, int cmp, uint64_t cmp_val) {
+    return nvshmemi_wait_until<uint64_t>(sig_addr, cmp, cmp_val);
+}
+
+/* ---- typed wait / test (14 types) ---- */
+#define NVSHMEMI_STAMP_WAIT(NAME, TYPE)                                                           \
+    NVSHMEMI_DEV void nvshmem_##NAME##_wait_until(TYPE *ivar, int cmp, TYPE cmp_value) {          \
+        nvshmemi_wait_until<TYPE>(ivar, cmp, cmp_value);                                          \
+    }                                                                                             \
+    NVSHMEMI_DEV int nvshmem_##NAME##_test(TYPE *ivar, int cmp, TYPE cmp_value) {                 \
+        return nvshmemi_test<TYPE>(ivar, cmp, cmp_value);                                         \
+    }                                                                                             \
+    NVSHMEMI_DEV void nvshmem_##NAME##_wait_until_all(TYPE *ivars, size_t nelems,                 \
+                                                      const int *status, int cmp,                 \
+                                                      TYPE cmp_value) {                           \
+        for (size_t i = 0; i < nelems; ++i)                                                       \
+            if (!status || !status[i]) nvshmemi_wait_until<TYPE>(ivars + i, cmp, cmp_value);      \
+    }                                                                                             \
+    NVSHMEMI_DEV int nvshmem_##NAME##_test_all(TYPE *ivars, size_t nelems, const int *status,     \
+                                               int cmp, TYPE cmp_value) {                         \
+        for (size_t i = 0; i < nelems; ++i)                                                       \
+            if ((!status || !status[i]) && !nvshmemi_test<TYPE>(ivars + i, cmp, cmp_value))       \
+                return 0;                                                                         \
+        return 1;                                                                                 \
+    }
+NVSHMEMI_REPT_FOR_WAIT_TYPES(NVSHMEMI_STAMP_WAIT)
+#undef NVSHMEMI_STAMP_WAIT
+
+/* ---- collectives inside a kernel: one thread group per PE ---- */
+#define NVSHMEMI_STAMP_COLL_SCOPE(NAME, TYPE, PFX, SFX, SC)                                       \
+    NVSHMEMI_DEV int PFX##_##NAME##_alltoall##SFX(nvshmem_team_t team, TYPE *dest,                \
+                                                  const TYPE *src, size_t nelems) {               \
+        return nvshmemi_alltoall_threadgroup<TYPE, SC>(team, dest, src, nelems);                  \
+    }                                                                                             \
+    NVSHMEMI_DEV int PFX##_##NAME##_fcollect##SFX(nvshmem_team_t team, TYPE *dest,                \
+                                                  const TYPE *src, size_t nelems) {               \
+        return nvshmemi_fcollect_threadgroup<TYPE, SC>(team, dest, src, nelems);                  \
+    }
+#define NVSHMEMI_STAMP_COLL(NAME, TYPE, TAG)                                                      \
+    NVSHMEMI_STAMP_COLL_SCOPE(NAME, TYPE, nvshmem, , NVSHMEMI_THREADGROUP_THREAD)                 \
+    NVSHMEMI_STAMP_COLL_SCOPE(NAME, TYPE, nvshmemx, _warp, NVSHMEMI_THREADGROUP_WARP)             \
+    NVSHMEMI_STAMP_COLL_SCOPE(NAME, TYPE, nvshmemx, _block, NVSHMEMI_THREADGROUP_BLOCK)
+NVSHMEMI_REPT_FOR_STANDARD_RMA_TYPES(NVSHMEMI_STAMP_COLL)
+#undef NVSHMEMI_STAMP_COLL
+#undef NVSHMEMI_STAMP_COLL_SCOPE
+
+#define NVSHMEMI_STAMP_MEM_COLL(PFX, SFX, SC)                                                     \
+    NVSHMEMI_DEV int PFX##_alltoallmem##SFX(nvshmem_team_t team, void *dest, const void *src,     \
+                                            size_t nelems) {                                      \
+        return nvshmemi_alltoall_threadgroup<char, SC>(team, (char *)dest, (const char *)src,     \
+                                                       nelems);                                   \
+    }                                                                                             \
+    NVSHMEMI_DEV int PFX##_fcollectmem##SFX(nvshmem_team_t team, void *dest, const void *src,     \
+                                            size_t nelems) {                                      \
+        return nvshmemi_fcollect_threadgroup<char, SC>(team, (char *)dest, (const char *)src,     \
+                                                       nelems);                                   \
+    }
+NVSHMEMI_STAMP_MEM_COLL(nvshmem, , NVSHMEMI_THREADGROUP_THREAD)
+NVSHMEMI_STAMP_MEM_COLL(nvshmemx, _warp, NVSHMEMI_THREADGROUP_WARP)
+NVSHMEMI_STAMP_MEM_COLL(nvshmemx, _block, NVSHMEMI_THREADGROUP_BLOCK)
+#undef NVSHMEMI_STAMP_MEM_COLL
+
+#define NVSHMEMI_STAMP_REDUCE(NAME, TYPE, TAG, OP)                                                \
+    NVSHMEMI_DEV int nvshmem_##NAME##_##OP##_reduce(nvshmem_team_t team, TYPE *dest,              \
+                                                    const TYPE *src, size_t nreduce) {            \
+        return nvshmemi_reduce_threadgroup<TYPE, NVSHMEMI_OP_##OP, NVSHMEMI_THREADGROUP_THREAD>(  \
+            team, dest, src, nreduce);                                                            \
+    }                                                                                             \
+    NVSHMEMI_DEV int nvshmemx_##NAME##_##OP##_reduce_warp(nvshmem_team_t team, TYPE *dest,        \
+                                                          const TYPE *src, size_t nreduce) {      \
+        return nvshmemi_reduce_threadgroup<TYPE, NVSHMEMI_OP_##OP, NVSHMEMI_THREADGROUP_WARP>(    \
+            team, dest, src, nreduce);                                                            \
+    }                                                                                             \
+    NVSHMEMI_DEV int nvshmemx_##NAME##_##OP##_reduce_block(nvshmem_team_t team, TYPE *dest,       \
+                                                           const TYPE *src, size_t nreduce) {     \
+        return nvshmemi_reduce_threadgroup<TYPE, NVSHMEMI_OP_##OP, NVSHMEMI_THREADGROUP_BLOCK>(   \
+            team, dest, src, nreduce);                                                            \
+    }
+NVSHMEMI_REPT_FOR_ALL_REDUCE_TYPES_AND_OPS(NVSHMEMI_STAMP_REDUCE)
+#undef NVSHMEMI_STAMP_REDUCE
+
+#undef NVSHMEMI_DEV
+#endif

@@ -1,0 +1,540 @@
+/*
+ * Device-side building blocks of the data-movement path for gfx950 (wavefront64).
+ * Header-only: everything is inlined into the caller's kernel, as in the reference, whose device
+ * layer is src/include/non_abi/device/{common,threadgroup,wait,coll}.
+ *
+ * Logical PEs.  A kernel started through nvshmemx_collective_launch has gridDim.z == npes and a
+ * block acts as PE blockIdx.z.  Symmetric pointers in kernel arguments are canonical (PE 0 slice)
+ * addresses; API calls translate them: a remote operand goes to PE `pe`'s slice, a local operand
+ * that lies in slice 0 goes to the calling PE's slice, any other address is used as it is.
+ * Code that dereferences a symmetric pointer itself localises it with nvshmem_ptr(p, nvshmem_my_pe()).
+ */
+#ifndef NVSHMEM_AMD_DEVICE_INTERNAL_H
+#define NVSHMEM_AMD_DEVICE_INTERNAL_H
+
+#if !defined(__HIPCC__)
+#error "the NVSHMEM device API needs hipcc"
+#endif
+
+#include <hip/hip_runtime.h>
+#include <type_traits>
+#include "../nvshmem_host_api.h"
+#include "../nvshmem_types.h"
+
+/* One private copy per translation unit.  The unit registers a callback that copies the host
+ * library's state block into its copy; the library calls every registered callback whenever the
+ * state changes. */
+static __constant__ nvshmemi_device_state_t nvshmemi_device_state_d;
+
+namespace nvshmemi_amd {
+static int push_state(const nvshmemi_device_state_t *host_copy) {
+    return (int)hipMemcpyToSymbol(HIP_SYMBOL(nvshmemi_device_state_d), host_copy,
+                                  sizeof(nvshmemi_device_state_t), 0, hipMemcpyHostToDevice);
+}
+struct state_registrar {
+    state_registrar() { nvshmemi_amd_register_state_updater(&push_state); }
+    ~state_registrar() { nvshmemi_amd_unregister_state_updater(&push_state); }
+};
+static state_registrar state_registrar_instance;
+}  // namespace nvshmemi_amd
+
+#define NVSHMEMI_DEVICE_INLINE __device__ __forceinline__
+
+/* ------------------------------------------------------------------------------------------------
+ * Thread groups (reference threadgroup/nvshmemi_common_device_defines.cuh:32-120)
+ * ---------------------------------------------------------------------------------------------- */
+enum nvshmemi_threadgroup_t {
+    NVSHMEMI_THREADGROUP_THREAD = 0,
+    NVSHMEMI_THREADGROUP_WARP = 1,
+    NVSHMEMI_THREADGROUP_BLOCK = 2
+};
+
+NVSHMEMI_DEVICE_INLINE unsigned nvshmemi_amd_block_size() {
+    return blockDim.x * blockDim.y * blockDim.z;
+}
+NVSHMEMI_DEVICE_INLINE unsigned nvshmemi_amd_block_tid() {
+    return threadIdx.x + blockDim.x * (threadIdx.y + blockDim.y * threadIdx.z);
+}
+
+template <int SCOPE>
+NVSHMEMI_DEVICE_INLINE int nvshmemi_thread_id_in_threadgroup() {
+    if (SCOPE == NVSHMEMI_THREADGROUP_WARP) return (int)(nvshmemi_amd_block_tid() % NVSHMEMI_WARP_SIZE);
+    if (SCOPE == NVSHMEMI_THREADGROUP_BLOCK) return (int)nvshmemi_amd_block_tid();
+    return 0;
+}
+
+template <int SCOPE>
+NVSHMEMI_DEVICE_INLINE int nvshmemi_threadgroup_size() {
+    if (SCOPE == NVSHMEMI_THREADGROUP_WARP) {
+        unsigned b = nvshmemi_amd_block_size();
+        return (int)(b < NVSHMEMI_WARP_SIZE ? b : NVSHMEMI_WARP_SIZE);
+    }
+    if (SCOPE == NVSHMEMI_THREADGROUP_BLOCK) return (int)nvshmemi_amd_block_size();
+    return 1;
+}
+
+template <int SCOPE>
+NVSHMEMI_DEVICE_INLINE void nvshmemi_threadgroup_sync() {
+    if (SCOPE == NVSHMEMI_THREADGROUP_WARP) {
+        /* A wavefront runs in lock step; this only orders its memory operations. */
+        __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");
+        __builtin_amdgcn_wave_barrier();
+    } else if (SCOPE == NVSHMEMI_THREADGROUP_BLOCK) {
+        __syncthreads();
+    }
+}
+
+/* Wait until this wavefront's outstanding vector memory operations have completed
+ * (s_waitcnt vmcnt(0), gfx9 encoding: lgkmcnt and expcnt left at their maxima). */
+NVSHMEMI_DEVICE_INLINE void nvshmemi_amd_wait_vm() { __builtin_amdgcn_s_waitcnt(0x0F70); }
+
+/* ------------------------------------------------------------------------------------------------
+ * PE identity and address translation
+ * (reference nvshmemi_ptr, common/nvshmemi_common_device.cuh:578-590, and the inline
+ * `peer_base + (ptr - heap_base)` of every RMA call, e.g. :493-498)
+ * ---------------------------------------------------------------------------------------------- */
+NVSHMEMI_DEVICE_INLINE int nvshmemi_amd_my_pe() {
+    return (gridDim.z == (unsigned)nvshmemi_device_state_d.npes) ? (int)blockIdx.z
+                                                                 : nvshmemi_device_state_d.mype;
+}
+NVSHMEMI_DEVICE_INLINE int nvshmemi_amd_n_pes() { return nvshmemi_device_state_d.npes; }
+
+/* Address of PE `pe`'s copy of the symmetric object at `sym` (an address in any PE's slice). */
+NVSHMEMI_DEVICE_INLINE char *nvshmemi_amd_remote(const void *sym, int pe) {
+    const uint64_t off = (uint64_t)((const char *)sym - nvshmemi_device_state_d.heap_base) &
+                         (nvshmemi_device_state_d.heap_size - 1);
+    return nvshmemi_device_state_d.heap_base +
+           ((uint64_t)(unsigned)pe << nvshmemi_device_state_d.heap_shift) + off;
+}
+
+/* Local operand: a canonical address means "my copy"; anything else is taken literally. */
+NVSHMEMI_DEVICE_INLINE char *nvshmemi_amd_local(const void *p) {
+    const uint64_t off = (uint64_t)((const char *)p - nvshmemi_device_state_d.heap_base);
+    if (off < nvshmemi_device_state_d.heap_size)
+        return nvshmemi_device_state_d.heap_base +
+               ((uint64_t)(unsigned)nvshmemi_amd_my_pe() << nvshmemi_device_state_d.heap_shift) + off;
+    return (char *)p;
+}
+
+NVSHMEMI_DEVICE_INLINE void *nvshmemi_ptr(const void *ptr, int pe) {
+    const uint64_t off = (uint64_t)((const char *)ptr - nvshmemi_device_state_d.heap_base);
+    if (pe >= 0 && pe < nvshmemi_device_state_d.npes &&
+        off < ((uint64_t)(unsigned)nvshmemi_device_state_d.npes << nvshmemi_device_state_d.heap_shift))
+        return nvshmemi_amd_remote(ptr, pe);
+    return nullptr;
+}
+
+/* ------------------------------------------------------------------------------------------------
+ * Copy engine (reference nvshmemi_memcpy_threadgroup, common/nvshmemi_common_device.cuh:254-349)
+ *
+ * Byte-exact copy by the lanes of one thread group.  Where the reference picks the widest element
+ * both pointers are aligned to and cascades, this version always stores 16-byte vectors: a byte
+ * head brings dst to a 16-byte boundary, the body issues four independent dwordx4 loads per lane
+ * before the first store (gfx950 accepts unaligned vector loads, so a src that is not co-aligned
+ * only costs extra cache-line touches, not narrower instructions), and a byte tail finishes.
+ * ---------------------------------------------------------------------------------------------- */
+typedef unsigned int nvshmemi_v4u __attribute__((ext_vector_type(4)));
+typedef nvshmemi_v4u __attribute__((aligned(1))) nvshmemi_v4u_unaligned;
+
+#ifndef NVSHMEMI_AMD_COPY_UNROLL
+#define NVSHMEMI_AMD_COPY_UNROLL 4
+#endif
+
+template <bool SRC_ALIGNED>
+NVSHMEMI_DEVICE_INLINE nvshmemi_v4u nvshmemi_amd_load16(const char *p) {
+    if (SRC_ALIGNED) return *reinterpret_cast<const nvshmemi_v4u *>(p);
+    return *reinterpret_cast<const nvshmemi_v4u_unaligned *>(p);
+}
+
+template <bool SRC_ALIGNED>
+NVSHMEMI_DEVICE_INLINE void nvshmemi_amd_copy_vectors(char *__restrict__ dst,
+                                                     const char *__restrict__ src, size_t nvec,
+                                                     size_t tid, size_t nthr) {
+    constexpr int U = NVSHMEMI_AMD_COPY_UNROLL;
+    size_t i = tid;
+    for (; i + (U - 1) * nthr < nvec; i += U * nthr) {
+        nvshmemi_v4u v[U];
+#pragma unroll
+        for (int u = 0; u < U; ++u) v[u] = nvshmemi_amd_load16<SRC_ALIGNED>(src + 16 * (i + u * nthr));
+#pragma unroll
+        for (int u = 0; u < U; ++u) *reinterpret_cast<nvshmemi_v4u *>(dst + 16 * (i + u * nthr)) = v[u];
+    }
+    for (; i < nvec; i += nthr)
+        *reinterpret_cast<nvshmemi_v4u *>(dst + 16 * i) = nvshmemi_amd_load16<SRC_ALIGNED>(src + 16 * i);
+}
+
+template <int SCOPE>
+NVSHMEMI_DEVICE_INLINE void nvshmemi_memcpy_threadgroup(void *__restrict__ dst_v,
+                                                       const void *__restrict__ src_v, size_t len) {
+    char *dst = static_cast<char *>(dst_v);
+    const char *src = static_cast<const char *>(src_v);
+    const size_t tid = (size_t)nvshmemi_thread_id_in_threadgroup<SCOPE>();
+    const size_t nthr = (size_t)nvshmemi_threadgroup_size<SCOPE>();
+
+    size_t head = (size_t)(-(uintptr_t)dst & 15);
+    if (head > len) head = len;
+    for (size_t i = tid; i < head; i += nthr) dst[i] = src[i];
+    dst += head;
+    src += head;
+    len -= head;
+
+    const size_t nvec = len / 16;
+    if (nvec) {
+        if (((uintptr_t)src & 15) == 0)
+            nvshmemi_amd_copy_vectors<true>(dst, src, nvec, tid, nthr);
+        else
+            nvshmemi_amd_copy_vectors<false>(dst, src, nvec, tid, nthr);
+    }
+    const size_t done = nvec * 16;
+    for (size_t i = done + tid; i < len; i += nthr) dst[i] = src[i];
+}
+
+/* ------------------------------------------------------------------------------------------------
+ * put / get / p / g  (reference common/nvshmemi_common_device.cuh:396-505)
+ * The non-blocking forms are the same code on a load/store path, as in the reference (:410-427).
+ * ---------------------------------------------------------------------------------------------- */
+template <typename T, int SCOPE>
+NVSHMEMI_DEVICE_INLINE void nvshmemi_put(T *dest, const T *source, size_t nelems, int pe) {
+    nvshmemi_threadgroup_sync<SCOPE>();
+    nvshmemi_memcpy_threadgroup<SCOPE>(nvshmemi_amd_remote(dest, pe), nvshmemi_amd_local(source),
+                                       nelems * sizeof(T));
+    nvshmemi_threadgroup_sync<SCOPE>();
+}
+
+template <typename T, int SCOPE>
+NVSHMEMI_DEVICE_INLINE void nvshmemi_get(T *dest, const T *source, size_t nelems, int pe) {
+    nvshmemi_threadgroup_sync<SCOPE>();
+    nvshmemi_memcpy_threadgroup<SCOPE>(nvshmemi_amd_local(dest), nvshmemi_amd_remote(source, pe),
+                                       nelems * sizeof(T));
+    nvshmemi_threadgroup_sync<SCOPE>();
+}
+
+template <typename T>
+NVSHMEMI_DEVICE_INLINE void nvshmemi_p(T *dest, const T value, int pe) {
+    *reinterpret_cast<T *>(nvshmemi_amd_remote(dest, pe)) = value;
+}
+
+/* A remote word may be written by another PE while this kernel runs, so the read is an agent-scope
+ * atomic load of the element's bits (never kept in a register, never served from a stale line). */
+template <typename T>
+NVSHMEMI_DEVICE_INLINE T nvshmemi_g(const T *source, int pe) {
+    const char *p = nvshmemi_amd_remote(source, pe);
+    T out;
+    if constexpr (sizeof(T) == 1) {
+        uint8_t v = __hip_atomic_load((const uint8_t *)p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        __builtin_memcpy(&out, &v, 1);
+    } else if constexpr (sizeof(T) == 2) {
+        uint16_t v = __hip_atomic_load((const uint16_t *)p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        __builtin_memcpy(&out, &v, 2);
+    } else if constexpr (sizeof(T) == 4) {
+        uint32_t v = __hip_atomic_load((const uint32_t *)p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        __builtin_memcpy(&out, &v, 4);
+    } else {
+        static_assert(sizeof(T) == 8, "scalar get supports 1, 2, 4 and 8 byte elements");
+        uint64_t v = __hip_atomic_load((const uint64_t *)p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        __builtin_memcpy(&out, &v, 8);
+    }
+    return out;
+}
+
+/* Strided forms (reference src/include/device/nvshmem_defines.h:345-431): element i of the source
+ * at stride sst goes to element i*dst of the destination. */
+template <typename T, int SCOPE>
+NVSHMEMI_DEVICE_INLINE void nvshmemi_iput(T *dest, const T *source, ptrdiff_t dst, ptrdiff_t sst,
+                                          size_t nelems, int pe) {
+    nvshmemi_threadgroup_sync<SCOPE>();
+    T *d = reinterpret_cast<T *>(nvshmemi_amd_remote(dest, pe));
+    const T *s = reinterpret_cast<const T *>(nvshmemi_amd_local(source));
+    const size_t tid = (size_t)nvshmemi_thread_id_in_threadgroup<SCOPE>();
+    const size_t nthr = (size_t)nvshmemi_threadgroup_size<SCOPE>();
+    for (size_t i = tid; i < nelems; i += nthr) d[(ptrdiff_t)i * dst] = s[(ptrdiff_t)i * sst];
+    nvshmemi_threadgroup_sync<SCOPE>();
+}
+
+template <typename T, int SCOPE>
+NVSHMEMI_DEVICE_INLINE void nvshmemi_iget(T *dest, const T *source, ptrdiff_t dst, ptrdiff_t sst,
+                                          size_t nelems, int pe) {
+    nvshmemi_threadgroup_sync<SCOPE>();
+    T *d = reinterpret_cast<T *>(nvshmemi_amd_local(dest));
+    const T *s = reinterpret_cast<const T *>(nvshmemi_amd_remote(source, pe));
+    const size_t tid = (size_t)nvshmemi_thread_id_in_threadgroup<SCOPE>();
+    const size_t nthr = (size_t)nvshmemi_threadgroup_size<SCOPE>();
+    for (size_t i = tid; i < nelems; i += nthr) d[(ptrdiff_t)i * dst] = s[(ptrdiff_t)i * sst];
+    nvshmemi_threadgroup_sync<SCOPE>();
+}
+
+/* ------------------------------------------------------------------------------------------------
+ * quiet / fence  (reference common/nvshmemi_common_device.cuh:352-385): one GPU, so agent scope.
+ * ---------------------------------------------------------------------------------------------- */
+template <int SCOPE>
+NVSHMEMI_DEVICE_INLINE void nvshmemi_quiet() {
+    nvshmemi_amd_wait_vm();
+    nvshmemi_threadgroup_sync<SCOPE>();
+    if (nvshmemi_thread_id_in_threadgroup<SCOPE>() == 0)
+        __builtin_amdgcn_fence(__ATOMIC_SEQ_CST, "agent");
+    nvshmemi_threadgroup_sync<SCOPE>();
+}
+
+/* ------------------------------------------------------------------------------------------------
+ * signal / put_signal  (reference common/nvshmemi_common_device.cuh:507-561)
+ * ---------------------------------------------------------------------------------------------- */
+NVSHMEMI_DEVICE_INLINE void nvshmemi_signal_op(uint64_t *sig_addr, uint64_t signal, int sig_op,
+                                               int pe) {
+    uint64_t *p = reinterpret_cast<uint64_t *>(nvshmemi_amd_remote(sig_addr, pe));
+    if (sig_op == NVSHMEM_SIGNAL_SET)
+        __hip_atomic_store(p, signal, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    else
+        __hip_atomic_fetch_add(p, signal, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+
+/* A standalone signal publishes everything its caller wrote before it. */
+NVSHMEMI_DEVICE_INLINE void nvshmemi_signal_op_release(uint64_t *sig_addr, uint64_t signal,
+                                                       int sig_op, int pe) {
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "agent");
+    nvshmemi_signal_op(sig_addr, signal, sig_op, pe);
+}
+
+template <typename T, int SCOPE>
+NVSHMEMI_DEVICE_INLINE void nvshmemi_put_signal(T *dest, const T *source, size_t nelems,
+                                                uint64_t *sig_addr, uint64_t signal, int sig_op,
+                                                int pe) {
+    nvshmemi_threadgroup_sync<SCOPE>();
+    nvshmemi_memcpy_threadgroup<SCOPE>(nvshmemi_amd_remote(dest, pe), nvshmemi_amd_local(source),
+                                       nelems * sizeof(T));
+    /* Every wavefront's stores have reached the L2 before the group meets; the one lane that
+     * signals then releases at agent scope, which writes the L2 back for the other XCDs. */
+    nvshmemi_amd_wait_vm();
+    nvshmemi_threadgroup_sync<SCOPE>();
+    if (nvshmemi_thread_id_in_threadgroup<SCOPE>() == 0)
+        nvshmemi_signal_op_release(sig_addr, signal, sig_op, pe);
+    nvshmemi_threadgroup_sync<SCOPE>();
+}
+
+/* ------------------------------------------------------------------------------------------------
+ * wait / test  (reference wait/nvshmemi_wait_until_apis.cuh:37-155, nvshmemi_test
+ * common/nvshmemi_common_device.cuh:130-147)
+ * ---------------------------------------------------------------------------------------------- */
+template <typename T>
+NVSHMEMI_DEVICE_INLINE bool nvshmemi_amd_compare(T found, int cmp, T expected) {
+    switch (cmp) {
+        case NVSHMEM_CMP_EQ: return found == expected;
+        case NVSHMEM_CMP_NE: return found != expected;
+        case NVSHMEM_CMP_GT: return found > expected;
+        case NVSHMEM_CMP_LE: return found <= expected;
+        case NVSHMEM_CMP_LT: return found < expected;
+        case NVSHMEM_CMP_GE: return found >= expected;
+        default: return true; /* an unknown comparator never blocks */
+    }
+}
+
+template <typename T>
+NVSHMEMI_DEVICE_INLINE T nvshmemi_amd_poll(const T *addr) {
+    return __hip_atomic_load(addr, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+
+NVSHMEMI_DEVICE_INLINE void nvshmemi_amd_record_timeout(const void *addr, uint64_t found,
+                                                        uint64_t expected) {
+    uint64_t *rec = reinterpret_cast<uint64_t *>(
+        nvshmemi_amd_remote(nvshmemi_device_state_d.timeout_record, nvshmemi_amd_my_pe()));
+    rec[1] = (uint64_t)(uintptr_t)addr;
+    rec[2] = found;
+    rec[3] = expected;
+    __hip_atomic_store(rec, (uint64_t)1, __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_AGENT);
+}
+
+/* Spin until `*ivar cmp value`; `ivar` is a local operand.  Returns the value that ended the wait.
+ * The final acquire makes data published before the signal visible to the caller; the reference's
+ * typed waits fence the same way (__threadfence via nvshmemi_transfer_syncapi_update_mem). */
+template <typename T>
+NVSHMEMI_DEVICE_INLINE T nvshmemi_wait_until(T *ivar, int cmp, T value) {
+    const T *addr = reinterpret_cast<const T *>(nvshmemi_amd_local(ivar));
+    const uint64_t limit = nvshmemi_device_state_d.spin_limit;
+    uint64_t polls = 0;
+    T found = nvshmemi_amd_poll(addr);
+    while (!nvshmemi_amd_compare(found, cmp, value)) {
+        if (limit && ++polls > limit) {
+            nvshmemi_amd_record_timeout(addr, (uint64_t)found, (uint64_t)value);
+            break;
+        }
+        __builtin_amdgcn_s_sleep(1);
+        found = nvshmemi_amd_poll(addr);
+    }
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "agent");
+    return found;
+}
+
+template <typename T>
+NVSHMEMI_DEVICE_INLINE int nvshmemi_test(T *ivar, int cmp, T value) {
+    const T *addr = reinterpret_cast<const T *>(nvshmemi_amd_local(ivar));
+    if (nvshmemi_amd_compare(nvshmemi_amd_poll(addr), cmp, value)) {
+        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "agent");
+        return 1;
+    }
+    return 0;
+}
+
+/* ------------------------------------------------------------------------------------------------
+ * barrier / sync  (reference coll/barrier.cuh:24-251, coll/utils.cuh:38-51)
+ *
+ * One thread group per PE takes part.  Flat exchange (the reference's dissemination with radix =
+ * team size, its choice for block scope on a load/store path, barrier.cuh:195-225): PE me stores
+ * its new epoch into word [me] of every PE's flag row, then waits until all npes words of its own
+ * row have reached that epoch.  Epochs only grow, so rows are never reset.
+ * ---------------------------------------------------------------------------------------------- */
+template <int SCOPE>
+NVSHMEMI_DEVICE_INLINE void nvshmemi_sync_threadgroup() {
+    const int me = nvshmemi_amd_my_pe();
+    const int npes = nvshmemi_device_state_d.npes;
+    const int tid = nvshmemi_thread_id_in_threadgroup<SCOPE>();
+    const int nthr = nvshmemi_threadgroup_size<SCOPE>();
+    uint64_t *epoch_p =
+        reinterpret_cast<uint64_t *>(nvshmemi_amd_remote(nvshmemi_device_state_d.sync_epoch, me));
+    nvshmemi_threadgroup_sync<SCOPE>();
+    const uint64_t epoch = *reinterpret_cast<volatile uint64_t *>(epoch_p) + 1;
+    nvshmemi_threadgroup_sync<SCOPE>();
+    if (tid == 0) *reinterpret_cast<volatile uint64_t *>(epoch_p) = epoch;
+    for (int pe = tid; pe < npes; pe += nthr) {
+        uint64_t *flag =
+            reinterpret_cast<uint64_t *>(nvshmemi_amd_remote(nvshmemi_device_state_d.sync_flags, pe)) + me;
+        __hip_atomic_store(flag, epoch, __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_AGENT);
+    }
+    uint64_t *row = reinterpret_cast<uint64_t *>(nvshmemi_amd_remote(nvshmemi_device_state_d.sync_flags, me));
+    for (int pe = tid; pe < npes; pe += nthr) nvshmemi_wait_until<uint64_t>(row + pe, NVSHMEM_CMP_GE, epoch);
+    nvshmemi_threadgroup_sync<SCOPE>();
+}
+
+template <int SCOPE>
+NVSHMEMI_DEVICE_INLINE void nvshmemi_barrier_threadgroup() {
+    nvshmemi_quiet<SCOPE>();
+    nvshmemi_sync_threadgroup<SCOPE>();
+}
+
+/* ------------------------------------------------------------------------------------------------
+ * Reduction operator (reference perform_gpu_rdxn, coll/reduce.cuh:49-105): computed in the element
+ * type; 16-bit floats add/multiply in fp32 and round to nearest-even once per step, which equals
+ * the correctly rounded 16-bit operation.  min/max keep the reference's operand rule
+ * `(a < b) ? a : b` / `(a > b) ? a : b`, which fixes the result for NaN and signed zeros.
+ * Signed integer sum/prod wrap (computed unsigned).
+ * ---------------------------------------------------------------------------------------------- */
+template <typename T> struct nvshmemi_amd_arith { typedef T type; };
+template <> struct nvshmemi_amd_arith<__hip_bfloat16> { typedef float type; };
+template <> struct nvshmemi_amd_arith<__half> { typedef float type; };
+template <> struct nvshmemi_amd_arith<signed char> { typedef unsigned char type; };
+template <> struct nvshmemi_amd_arith<char> { typedef unsigned char type; };
+template <> struct nvshmemi_amd_arith<short> { typedef unsigned short type; };
+template <> struct nvshmemi_amd_arith<int> { typedef unsigned int type; };
+template <> struct nvshmemi_amd_arith<long> { typedef unsigned long type; };
+template <> struct nvshmemi_amd_arith<long long> { typedef unsigned long long type; };
+
+template <typename T> NVSHMEMI_DEVICE_INLINE float nvshmemi_amd_to_float(T v) { return (float)v; }
+template <> NVSHMEMI_DEVICE_INLINE float nvshmemi_amd_to_float(__hip_bfloat16 v) { return __bfloat162float(v); }
+template <> NVSHMEMI_DEVICE_INLINE float nvshmemi_amd_to_float(__half v) { return __half2float(v); }
+template <typename T> NVSHMEMI_DEVICE_INLINE T nvshmemi_amd_from_float(float v) { return (T)v; }
+template <> NVSHMEMI_DEVICE_INLINE __hip_bfloat16 nvshmemi_amd_from_float(float v) { return __float2bfloat16(v); }
+template <> NVSHMEMI_DEVICE_INLINE __half nvshmemi_amd_from_float(float v) { return __float2half_rn(v); }
+
+template <typename T> struct nvshmemi_amd_is_half { static constexpr bool value = false; };
+template <> struct nvshmemi_amd_is_half<__hip_bfloat16> { static constexpr bool value = true; };
+template <> struct nvshmemi_amd_is_half<__half> { static constexpr bool value = true; };
+
+template <typename T, int OP>
+NVSHMEMI_DEVICE_INLINE T nvshmemi_amd_reduce_op(T a, T b) {
+    typedef typename nvshmemi_amd_arith<T>::type A;
+    if constexpr (nvshmemi_amd_is_half<T>::value) {
+        const float fa = nvshmemi_amd_to_float(a), fb = nvshmemi_amd_to_float(b);
+        if constexpr (OP == NVSHMEMI_OP_sum) return nvshmemi_amd_from_float<T>(fa + fb);
+        if constexpr (OP == NVSHMEMI_OP_prod) return nvshmemi_amd_from_float<T>(fa * fb);
+        if constexpr (OP == NVSHMEMI_OP_min) return (fa < fb) ? a : b;
+        if constexpr (OP == NVSHMEMI_OP_max) return (fa > fb) ? a : b;
+        return a;
+    } else {
+        if constexpr (OP == NVSHMEMI_OP_sum) return (T)((A)a + (A)b);
+        if constexpr (OP == NVSHMEMI_OP_prod) return (T)((A)a * (A)b);
+        if constexpr (OP == NVSHMEMI_OP_min) return (a < b) ? a : b;
+        if constexpr (OP == NVSHMEMI_OP_max) return (a > b) ? a : b;
+        if constexpr (std::is_integral<T>::value) {
+            if constexpr (OP == NVSHMEMI_OP_and) return (T)(a & b);
+            if constexpr (OP == NVSHMEMI_OP_or) return (T)(a | b);
+            if constexpr (OP == NVSHMEMI_OP_xor) return (T)(a ^ b);
+        }
+        return a;
+    }
+}
+
+/* Fold of one element over the PEs in the fixed order of the reference's gather-then-fold path
+ * (coll/reduce.cuh:1297-1303): acc = op(x0, x1); acc = op(x_i, acc) for i = 2..n-1. */
+template <typename T, int OP>
+NVSHMEMI_DEVICE_INLINE T nvshmemi_amd_fold_step(int i, T acc, T x) {
+    return (i == 1) ? nvshmemi_amd_reduce_op<T, OP>(acc, x) : nvshmemi_amd_reduce_op<T, OP>(x, acc);
+}
+
+/* ------------------------------------------------------------------------------------------------
+ * Collectives called from inside a user kernel, one thread group per PE
+ * (reference coll/reduce.cuh:1158-1196 get-based reduce, coll/fcollect.cuh:331-344,
+ * coll/alltoall.cuh:122-143).  Each ends with barrier semantics.
+ * ---------------------------------------------------------------------------------------------- */
+/* Reduce: PE `me` owns the element range [me*chunk, (me+1)*chunk): it folds that range from every
+ * PE's source and stores the result into every PE's dest.  Each element is read by exactly one lane
+ * before that lane overwrites it, so source == dest is safe, and every source byte is read once. */
+template <typename T, int OP, int SCOPE>
+NVSHMEMI_DEVICE_INLINE int nvshmemi_reduce_threadgroup(nvshmem_team_t team, T *dest, const T *source,
+                                                       size_t nreduce) {
+    (void)team;
+    const int me = nvshmemi_amd_my_pe();
+    const int npes = nvshmemi_device_state_d.npes;
+    const size_t tid = (size_t)nvshmemi_thread_id_in_threadgroup<SCOPE>();
+    const size_t nthr = (size_t)nvshmemi_threadgroup_size<SCOPE>();
+    /* every PE's source is complete and visible before anyone reads it */
+    nvshmemi_barrier_threadgroup<SCOPE>();
+    const size_t chunk = (nreduce + (size_t)npes - 1) / (size_t)npes;
+    size_t lo = (size_t)me * chunk;
+    if (lo > nreduce) lo = nreduce;
+    size_t hi = lo + chunk;
+    if (hi > nreduce) hi = nreduce;
+    const T *src0 = reinterpret_cast<const T *>(nvshmemi_amd_remote(source, 0));
+    T *dst0 = reinterpret_cast<T *>(nvshmemi_amd_remote(dest, 0));
+    const size_t pe_stride = (size_t)(nvshmemi_device_state_d.heap_size / sizeof(T));
+    for (size_t i = lo + tid; i < hi; i += nthr) {
+        T acc = src0[i];
+        for (int pe = 1; pe < npes; ++pe)
+            acc = nvshmemi_amd_fold_step<T, OP>(pe, acc, src0[(size_t)pe * pe_stride + i]);
+        for (int pe = 0; pe < npes; ++pe) dst0[(size_t)pe * pe_stride + i] = acc;
+    }
+    nvshmemi_barrier_threadgroup<SCOPE>();
+    return 0;
+}
+
+template <typename T, int SCOPE>
+NVSHMEMI_DEVICE_INLINE int nvshmemi_fcollect_threadgroup(nvshmem_team_t team, T *dest,
+                                                         const T *source, size_t nelems) {
+    (void)team;
+    const int me = nvshmemi_amd_my_pe();
+    const int npes = nvshmemi_device_state_d.npes;
+    nvshmemi_threadgroup_sync<SCOPE>();
+    for (int ii = 0; ii < npes; ++ii) {
+        const int peer = (me + ii) % npes;
+        nvshmemi_memcpy_threadgroup<SCOPE>(nvshmemi_amd_remote(dest + (size_t)me * nelems, peer),
+                                           nvshmemi_amd_local(source), nelems * sizeof(T));
+    }
+    nvshmemi_barrier_threadgroup<SCOPE>();
+    return 0;
+}
+
+template <typename T, int SCOPE>
+NVSHMEMI_DEVICE_INLINE int nvshmemi_alltoall_threadgroup(nvshmem_team_t team, T *dest,
+                                                         const T *source, size_t nelems) {
+    (void)team;
+    const int me = nvshmemi_amd_my_pe();
+    const int npes = nvshmemi_device_state_d.npes;
+    nvshmemi_threadgroup_sync<SCOPE>();
+    for (int ii = 0; ii < npes; ++ii) {
+        const int peer = (me + ii) % npes;
+        nvshmemi_memcpy_threadgroup<SCOPE>(nvshmemi_amd_remote(dest + (size_t)me * nelems, peer),
+                                           nvshmemi_amd_local(source + (size_t)peer * nelems),
+                                           nelems * sizeof(T));
+    }
+    nvshmemi_barrier_threadgroup<SCOPE>();
+    return 0;
+}
+
+#endif

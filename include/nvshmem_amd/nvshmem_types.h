@@ -1,0 +1,165 @@
+/*
+ * Type lists and the device state block.
+ *
+ * The X-macro lists restate the type matrices of the reference API
+ * (reference src/include/device_host/nvshmem_common.cuh:48-73 RMA types, :135-147 sizes,
+ * :156-170 wait types, :172-210 reduce types).  Each entry is X(api_name, c_type, kernel_tag):
+ * kernel_tag names the one kernel instantiation several same-width C types share
+ * (i8..i64, u8..u64, f16, bf16, f32, f64), so `long`, `long long` and `int64_t` run the same code.
+ */
+#ifndef NVSHMEM_AMD_TYPES_H
+#define NVSHMEM_AMD_TYPES_H
+
+#include "nvshmem_constants.h"
+
+#if defined(__HIPCC__)
+#include <hip/hip_runtime.h>
+#include <hip/hip_bf16.h>
+#include <hip/hip_fp16.h>
+typedef __hip_bfloat16 nvshmem_bfloat16_t;
+typedef __half nvshmem_half_t;
+#else
+/* Storage-only views for C and host C++ callers: the ABI passes pointers to 2-byte elements. */
+typedef struct { uint16_t bits; } nvshmem_bfloat16_t;
+typedef struct { uint16_t bits; } nvshmem_half_t;
+#endif
+
+/* 25 standard RMA types. */
+#define NVSHMEMI_REPT_FOR_STANDARD_RMA_TYPES(X) \
+    X(bfloat16, nvshmem_bfloat16_t, bf16)       \
+    X(half, nvshmem_half_t, f16)                \
+    X(float, float, f32)                        \
+    X(double, double, f64)                      \
+    X(char, char, i8)                           \
+    X(short, short, i16)                        \
+    X(schar, signed char, i8)                   \
+    X(int, int, i32)                            \
+    X(long, long, i64)                          \
+    X(longlong, long long, i64)                 \
+    X(uchar, unsigned char, u8)                 \
+    X(ushort, unsigned short, u16)              \
+    X(uint, unsigned int, u32)                  \
+    X(ulong, unsigned long, u64)                \
+    X(ulonglong, unsigned long long, u64)       \
+    X(int8, int8_t, i8)                         \
+    X(int16, int16_t, i16)                      \
+    X(int32, int32_t, i32)                      \
+    X(int64, int64_t, i64)                      \
+    X(uint8, uint8_t, u8)                       \
+    X(uint16, uint16_t, u16)                    \
+    X(uint32, uint32_t, u32)                    \
+    X(uint64, uint64_t, u64)                    \
+    X(size, size_t, u64)                        \
+    X(ptrdiff, ptrdiff_t, i64)
+
+/* put8/16/32/64/128: element width in bits and bytes. */
+#define NVSHMEMI_REPT_FOR_SIZES(X) X(8, 1) X(16, 2) X(32, 4) X(64, 8) X(128, 16)
+
+/* 14 wait/test types. */
+#define NVSHMEMI_REPT_FOR_WAIT_TYPES(X) \
+    X(short, short)                     \
+    X(int, int)                         \
+    X(long, long)                       \
+    X(longlong, long long)              \
+    X(ushort, unsigned short)           \
+    X(uint, unsigned int)               \
+    X(ulong, unsigned long)             \
+    X(ulonglong, unsigned long long)    \
+    X(int32, int32_t)                   \
+    X(int64, int64_t)                   \
+    X(uint32, uint32_t)                 \
+    X(uint64, uint64_t)                 \
+    X(size, size_t)                     \
+    X(ptrdiff, ptrdiff_t)
+
+/* and / or / xor. */
+#define NVSHMEMI_REPT_FOR_BITWISE_REDUCE_TYPES(X, OP) \
+    X(uchar, unsigned char, u8, OP)                   \
+    X(ushort, unsigned short, u16, OP)                \
+    X(uint, unsigned int, u32, OP)                    \
+    X(ulong, unsigned long, u64, OP)                  \
+    X(ulonglong, unsigned long long, u64, OP)         \
+    X(int8, int8_t, i8, OP)                           \
+    X(int16, int16_t, i16, OP)                        \
+    X(int32, int32_t, i32, OP)                        \
+    X(int64, int64_t, i64, OP)                        \
+    X(uint8, uint8_t, u8, OP)                         \
+    X(uint16, uint16_t, u16, OP)                      \
+    X(uint32, uint32_t, u32, OP)                      \
+    X(uint64, uint64_t, u64, OP)                      \
+    X(size, size_t, u64, OP)
+
+/* min / max / sum / prod: the bitwise list plus the signed and floating types. */
+#define NVSHMEMI_REPT_FOR_STANDARD_REDUCE_TYPES(X, OP) \
+    NVSHMEMI_REPT_FOR_BITWISE_REDUCE_TYPES(X, OP)      \
+    X(char, char, i8, OP)                              \
+    X(schar, signed char, i8, OP)                      \
+    X(short, short, i16, OP)                           \
+    X(int, int, i32, OP)                               \
+    X(long, long, i64, OP)                             \
+    X(longlong, long long, i64, OP)                    \
+    X(bfloat16, nvshmem_bfloat16_t, bf16, OP)          \
+    X(half, nvshmem_half_t, f16, OP)                   \
+    X(float, float, f32, OP)                           \
+    X(double, double, f64, OP)
+
+/* Every (type, op) pair of the reduce API, in one list: X(api_name, c_type, kernel_tag, op). */
+#define NVSHMEMI_REPT_FOR_ALL_REDUCE_TYPES_AND_OPS(X) \
+    NVSHMEMI_REPT_FOR_BITWISE_REDUCE_TYPES(X, and)    \
+    NVSHMEMI_REPT_FOR_BITWISE_REDUCE_TYPES(X, or)     \
+    NVSHMEMI_REPT_FOR_BITWISE_REDUCE_TYPES(X, xor)    \
+    NVSHMEMI_REPT_FOR_STANDARD_REDUCE_TYPES(X, max)   \
+    NVSHMEMI_REPT_FOR_STANDARD_REDUCE_TYPES(X, min)   \
+    NVSHMEMI_REPT_FOR_STANDARD_REDUCE_TYPES(X, sum)   \
+    NVSHMEMI_REPT_FOR_STANDARD_REDUCE_TYPES(X, prod)
+
+/* Reduction operator ids shared by host launchers, device code and the test oracle
+ * (same set as the reference's rdxn_ops_t, src/include/device_host/nvshmem_common.cuh:471-489). */
+typedef enum {
+    NVSHMEMI_OP_and = 0,
+    NVSHMEMI_OP_or = 1,
+    NVSHMEMI_OP_xor = 2,
+    NVSHMEMI_OP_min = 3,
+    NVSHMEMI_OP_max = 4,
+    NVSHMEMI_OP_sum = 5,
+    NVSHMEMI_OP_prod = 6
+} nvshmemi_amd_op_t;
+
+/* Element kinds of the shared kernel instantiations. */
+typedef enum {
+    NVSHMEMI_DT_i8 = 0,
+    NVSHMEMI_DT_i16,
+    NVSHMEMI_DT_i32,
+    NVSHMEMI_DT_i64,
+    NVSHMEMI_DT_u8,
+    NVSHMEMI_DT_u16,
+    NVSHMEMI_DT_u32,
+    NVSHMEMI_DT_u64,
+    NVSHMEMI_DT_f16,
+    NVSHMEMI_DT_bf16,
+    NVSHMEMI_DT_f32,
+    NVSHMEMI_DT_f64,
+    NVSHMEMI_DT_COUNT
+} nvshmemi_amd_dtype_t;
+
+/*
+ * State block read by device code (counterpart of the reference's nvshmemi_device_host_state_t,
+ * src/include/device_host/nvshmem_types.h:452-509).  All logical PEs live in one allocation:
+ * PE p owns [heap_base + p*heap_size, heap_base + (p+1)*heap_size), heap_size is a power of two,
+ * so the reference's peer_heap_base_p2p[] table collapses to a shift.  Symmetric addresses handed
+ * to users are addresses inside PE 0's slice ("canonical" addresses).
+ */
+typedef struct nvshmemi_device_state {
+    uint32_t version;     /* (1 << 16) + sizeof(struct) */
+    int32_t mype;         /* PE a kernel acts as when its grid is not PE-multiplexed */
+    int32_t npes;
+    uint32_t heap_shift;  /* log2(heap_size) */
+    char *heap_base;      /* start of PE 0's slice */
+    uint64_t heap_size;   /* bytes per PE */
+    uint64_t *sync_flags; /* canonical address: NVSHMEMI_AMD_MAX_PES arrival words per PE */
+    uint64_t *sync_epoch; /* canonical address: that PE's barrier epoch */
+    uint64_t spin_limit;  /* 0 = wait forever; else a bounded wait gives up after this many polls */
+    uint64_t *timeout_record; /* canonical address: 4 words {flag, addr, found, expected} */
+} nvshmemi_device_state_t;
+
+#endif

@@ -1,0 +1,128 @@
+/*
+ * C ABI of libnvshmem_amd_perftest.so: kernels written against the public device API (nvshmem.h /
+ * nvshmemx.h only, a separate code object from the runtime) and the host drivers that start them.
+ * They are this build's counterpart of the reference's device-initiated benchmarks and examples,
+ * the only in-tree callers of the device API there:
+ *   perftest/device/pt-to-pt/shmem_put_bw.cu, shmem_get_bw.cu          -> ring_rma
+ *   perftest/device/pt-to-pt/shmem_put_signal_ping_pong_latency.cu     -> put_signal_pingpong
+ *   examples/put-block.cu                                              -> ring_rma (its known answer)
+ *   examples/ring-reduce.cu                                            -> ring_reduce
+ *   perftest/device/coll/{reduction,fcollect,alltoall,barrier}_latency.cu -> device_* entry points
+ *   examples/moe_shuffle.cu                                            -> moe_* entry points
+ * All pointers are canonical symmetric addresses from nvshmem_malloc unless noted.  Every entry
+ * point returns 0 on success or an nvshmemx_status; work is enqueued on `stream` (a hipStream_t
+ * passed as void *, NULL = null stream) and is not waited for.
+ */
+#ifndef NVSHMEM_PERFTEST_H
+#define NVSHMEM_PERFTEST_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+enum { NVSHMEM_PERFTEST_SCOPE_THREAD = 0, NVSHMEM_PERFTEST_SCOPE_WARP = 1,
+       NVSHMEM_PERFTEST_SCOPE_BLOCK = 2 };
+
+/*
+ * Every PE p moves `bytes` bytes between its `src` and PE (p+1)%npes: put (is_get = 0) writes the
+ * peer's `dest`, get reads the peer's `src` into the local `dest`.  blocks_per_pe blocks of
+ * `threads` threads per PE; block b moves the slice [b*bytes/B, (b+1)*bytes/B) (the last block also
+ * takes the remainder; with bytes < B only block 0 works), as shmem_put_bw.cu:26-31 does.  With
+ * warp scope each wavefront of a block moves an equal part of the block's slice, with thread scope
+ * each thread does.  `iters` back-to-back launches.
+ */
+int nvshmem_perftest_ring_rma(void *dest, const void *src, size_t bytes, int blocks_per_pe,
+                              int threads, int scope, int is_get, int iters, void *stream);
+
+/* PE p writes value_base + p into word [p] of PE (p+1)%npes's `words` with nvshmem_uint64_p, then
+ * (after a barrier) reads word [q] of every PE q's `words`... with nvshmem_uint64_g into
+ * out[q] of its own `out`.  words and out hold npes uint64 each. */
+int nvshmem_perftest_p_g(uint64_t *words, uint64_t *out, uint64_t value_base, void *stream);
+
+/* Each of `threads` threads of one block per PE applies nvshmemx_signal_op(sig, value, sig_op,
+ * (p+1)%npes) `reps` times. */
+int nvshmem_perftest_signal_op(uint64_t *sig, uint64_t value, int sig_op, int threads, int reps,
+                               void *stream);
+
+/* One thread per PE waits with nvshmem_signal_wait_until(sig, cmp, cmp_value) and stores the value
+ * the wait returned into its own out[0].  Nobody signals: use it with a preset signal word or with
+ * a small spin limit (nvshmemx_amd_set_spin_limit) to exercise the bounded wait. */
+int nvshmem_perftest_signal_wait(uint64_t *sig, int cmp, uint64_t cmp_value, uint64_t *out,
+                                 void *stream);
+
+/* PE 0 and PE 1 bounce a `bytes` payload `iters` times with nvshmemx_putmem_signal_block and
+ * nvshmem_signal_wait_until (shmem_put_signal_ping_pong_latency.cu:29-49).  After it `data` on
+ * both PEs holds the payload PE 0 started with and sig == iters on both.  npes must be >= 2. */
+int nvshmem_perftest_put_signal_pingpong(void *data, uint64_t *sig, size_t bytes, int iters,
+                                         int threads, void *stream);
+
+/* Ring allreduce of int32 built from put_signal_nbi + signal_wait_until, the algorithm of
+ * examples/ring-reduce.cu:88-144: reduce phase around the ring, then broadcast phase.  nreduce must
+ * be a multiple of blocks*chunk_elems.  signal holds `blocks` words (zero before the call; the
+ * kernel zeroes them again).  Known answer of the example: src[i]=i on all PEs => dst[i]=i*npes. */
+int nvshmem_perftest_ring_reduce(int32_t *dst, const int32_t *src, size_t nreduce,
+                                 uint64_t *signal, size_t chunk_elems, int blocks, int threads,
+                                 void *stream);
+
+/* In-kernel collectives, one thread group per PE (grid 1 x 1 x npes).  dtype/op use the numbering
+ * of nvshmemi_amd_dtype_t / nvshmemi_amd_op_t; supported pairs: (i32,sum) (i64,xor) (f32,sum)
+ * (f32,max) (bf16,sum) (bf16,max) (u64,and) (f64,prod) (i16,min).  Returns NOT_SUPPORTED else. */
+int nvshmem_perftest_device_reduce(int dtype, int op, void *dest, const void *src, size_t nreduce,
+                                   int scope, int threads, void *stream);
+int nvshmem_perftest_device_fcollect(void *dest, const void *src, size_t bytes, int scope,
+                                     int threads, void *stream);
+int nvshmem_perftest_device_alltoall(void *dest, const void *src, size_t bytes, int scope,
+                                     int threads, void *stream);
+/* `rounds` barriers; before round r each PE stores r into its `counter`, after the barrier it reads
+ * every PE's counter and adds to its own errors[0] the number that are < r.  counter and errors
+ * hold one uint64 each. */
+int nvshmem_perftest_device_barrier(uint64_t *counter, uint64_t *errors, int rounds, int scope,
+                                    int threads, void *stream);
+
+/*
+ * MoE token shuffle (config: npes PEs, `tokens` rows of `row_bytes` per PE, `topk` copies per
+ * token).  Routing tables are device arrays in symmetric memory, one copy per PE, filled by the
+ * caller:  dest_pe[t*topk+k] (int32) and dest_row[t*topk+k] (int64) say where copy k of token t
+ * lands; expected[src] (uint64, npes words) is the number of rows this PE receives from PE src.
+ *   dispatch: recv@dest_pe[dest_row] = send[t]   via nvshmemx_putmem_signal_nbi_block with
+ *             NVSHMEM_SIGNAL_ADD of 1 on sig[src] at the destination; then every PE waits until
+ *             sig[src] >= expected[src] for all src (nvshmem_signal_wait_until, CMP_GE).
+ *   combine:  out[t*topk+k] = recv@dest_pe[dest_row]  via nvshmemx_getmem_nbi_block.
+ * sig holds npes words per PE and must be zero before dispatch.  recv holds recv_cap_rows rows on
+ * every PE; a routing entry outside [0, npes) x [0, recv_cap_rows) is skipped.  blocks_per_pe
+ * blocks of `threads` threads per PE; dispatch is a cooperative launch (it waits on other PEs).
+ * The plain entry points move one row per wavefront and publish one signal update per block and
+ * destination; the _ex forms choose the scope (NVSHMEM_PERFTEST_SCOPE_WARP or _BLOCK) and, with
+ * bit 8 set in `scope` (dispatch only), signal after every row.
+ */
+int nvshmem_perftest_moe_dispatch(void *recv, size_t recv_cap_rows, const void *send,
+                                  const int32_t *dest_pe, const int64_t *dest_row,
+                                  const uint64_t *expected, uint64_t *sig, int tokens, int topk,
+                                  size_t row_bytes, int blocks_per_pe, int threads, void *stream);
+int nvshmem_perftest_moe_dispatch_ex(void *recv, size_t recv_cap_rows, const void *send,
+                                     const int32_t *dest_pe, const int64_t *dest_row,
+                                     const uint64_t *expected, uint64_t *sig, int tokens, int topk,
+                                     size_t row_bytes, int blocks_per_pe, int threads, int scope,
+                                     void *stream);
+int nvshmem_perftest_moe_combine(void *out, const void *recv, size_t recv_cap_rows,
+                                 const int32_t *dest_pe, const int64_t *dest_row, int tokens,
+                                 int topk, size_t row_bytes, int blocks_per_pe, int threads,
+                                 void *stream);
+int nvshmem_perftest_moe_combine_ex(void *out, const void *recv, size_t recv_cap_rows,
+                                    const int32_t *dest_pe, const int64_t *dest_row, int tokens,
+                                    int topk, size_t row_bytes, int blocks_per_pe, int threads,
+                                    int scope, void *stream);
+/* Per-expert counts exchange + prefix sum on the device (examples/moe_shuffle.cu:204-234):
+ * counts holds num_experts int64 per PE (rows this PE sends to each expert); on return
+ * seg_base[e*npes + src] (int64, num_experts*npes words per PE, every PE gets the full table) is the
+ * first receive row of segment (expert e, source src) and recv_rows[0] the rows this PE receives. */
+int nvshmem_perftest_moe_exchange_offsets(const int64_t *counts, int64_t *seg_base,
+                                          int64_t *recv_rows, int num_experts, void *stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif

@@ -1,0 +1,87 @@
+"""Builds the in-tree native libraries with hipcc / gcc (gfx950 only).
+
+  nvshmem_amd/lib/libnvshmem_amd.so           host runtime + host-launched collectives (C ABI)
+  nvshmem_amd/lib/libnvshmem_amd_perftest.so  kernels that call the device API + their C ABI drivers
+  oracle/liboracle.so                         CPU oracle (test infrastructure only)
+
+Run as ``python -m nvshmem_amd.build``.  hipcc cross-compiles without a GPU.
+"""
+import os
+import shutil
+import subprocess
+import sys
+from concurrent.futures import ThreadPoolExecutor
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+CSRC = os.path.join(ROOT, "nvshmem_amd", "csrc")
+LIBDIR = os.path.join(ROOT, "nvshmem_amd", "lib")
+OBJDIR = os.path.join(ROOT, "build", "obj")
+INCLUDE = os.path.join(ROOT, "include")
+
+HIPCC = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
+HIP_FLAGS = [
+    "--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-Wall", "-Wno-unused-function",
+    "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
+    "-I" + INCLUDE, "-I" + CSRC,
+]
+
+RUNTIME_SOURCES = ["mspace.cpp", "runtime.hip", "collectives.hip"]
+PERFTEST_SOURCES = ["perftest/rma_kernels.hip", "perftest/coll_kernels.hip",
+                    "perftest/moe_shuffle.hip"]
+
+
+def _run(cmd):
+    proc = subprocess.run(cmd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)
+    out = "\n".join(l for l in proc.stdout.splitlines()
+                    if "packed-fp32-ops" not in l)  # host pass does not know the GPU feature
+    if proc.returncode != 0:
+        raise RuntimeError("command failed: %s\n%s" % (" ".join(cmd), out))
+    if out.strip():
+        sys.stderr.write(out + "\n")
+
+
+def _compile(src):
+    obj = os.path.join(OBJDIR, src.replace("/", "_") + ".o")
+    cmd = [HIPCC] + HIP_FLAGS + ["-c", os.path.join(CSRC, src), "-o", obj]
+    if src.endswith(".cpp"):
+        cmd.insert(1, "-x")
+        cmd.insert(2, "hip")
+    _run(cmd)
+    return obj
+
+
+def _link(objs, out, extra=()):
+    _run([HIPCC, "--offload-arch=gfx950", "-shared", "-fPIC", "-o", out] + objs + list(extra))
+
+
+def build_native(jobs=8):
+    os.makedirs(LIBDIR, exist_ok=True)
+    os.makedirs(OBJDIR, exist_ok=True)
+    sources = RUNTIME_SOURCES + [s for s in PERFTEST_SOURCES
+                                 if os.path.exists(os.path.join(CSRC, s))]
+    with ThreadPoolExecutor(max_workers=jobs) as pool:
+        objs = dict(zip(sources, pool.map(_compile, sources)))
+    runtime = os.path.join(LIBDIR, "libnvshmem_amd.so")
+    _link([objs[s] for s in RUNTIME_SOURCES], runtime)
+    perf = [objs[s] for s in PERFTEST_SOURCES if s in objs]
+    if perf:
+        _link(perf, os.path.join(LIBDIR, "libnvshmem_amd_perftest.so"),
+              ["-L" + LIBDIR, "-lnvshmem_amd", "-Wl,-rpath,$ORIGIN"])
+    return runtime
+
+
+def build_oracle():
+    """The oracle is a checker for tests and the bench's CPU baseline; nothing shipped links it."""
+    odir = os.path.join(ROOT, "oracle")
+    _run(["make", "-C", odir, "-B", "-s"])
+    return os.path.join(odir, "liboracle.so")
+
+
+def build_all():
+    build_native()
+    build_oracle()
+
+
+if __name__ == "__main__":
+    build_all()
+    print("built:", ", ".join(sorted(os.listdir(LIBDIR))))

@@ -1,0 +1,143 @@
+// In-kernel collectives through the public device API, one thread group per PE.
+// Counterparts in the reference tree: perftest/device/coll/reduction_latency.cu:23-44,
+// fcollect_latency.cu, alltoall_latency.cu, barrier_latency.cu (which time these calls from block 0
+// of one kernel per PE and never check the result).
+#include <hip/hip_runtime.h>
+
+#include "nvshmem_perftest.h"
+#include "nvshmemx.h"
+#include "perftest_common.hpp"
+
+namespace {
+
+enum { kReduce = 0, kFcollect = 1, kAlltoall = 2 };
+
+#define SCOPED_CALL(SCOPE, NAME, ...)                                               \
+    do {                                                                            \
+        if (SCOPE == NVSHMEM_PERFTEST_SCOPE_BLOCK) nvshmemx_##NAME##_block(__VA_ARGS__); \
+        else if (SCOPE == NVSHMEM_PERFTEST_SCOPE_WARP) {                            \
+            if (threadIdx.x < NVSHMEMI_WARP_SIZE) nvshmemx_##NAME##_warp(__VA_ARGS__); \
+        } else {                                                                    \
+            if (threadIdx.x == 0) nvshmem_##NAME(__VA_ARGS__);                      \
+        }                                                                           \
+    } while (0)
+
+#define DEFINE_REDUCE_KERNEL(TNAME, TYPE, OP)                                                    \
+    template <int SCOPE>                                                                         \
+    __global__ void reduce_##TNAME##_##OP##_kernel(TYPE *dest, const TYPE *src, size_t n) {      \
+        SCOPED_CALL(SCOPE, TNAME##_##OP##_reduce, NVSHMEM_TEAM_WORLD, dest, src, n);             \
+    }
+DEFINE_REDUCE_KERNEL(int32, int32_t, sum)
+DEFINE_REDUCE_KERNEL(int64, int64_t, xor)
+DEFINE_REDUCE_KERNEL(float, float, sum)
+DEFINE_REDUCE_KERNEL(float, float, max)
+DEFINE_REDUCE_KERNEL(bfloat16, nvshmem_bfloat16_t, sum)
+DEFINE_REDUCE_KERNEL(bfloat16, nvshmem_bfloat16_t, max)
+DEFINE_REDUCE_KERNEL(uint64, uint64_t, and)
+DEFINE_REDUCE_KERNEL(double, double, prod)
+DEFINE_REDUCE_KERNEL(int16, int16_t, min)
+
+template <int SCOPE>
+__global__ void fcollect_kernel(char *dest, const char *src, size_t bytes) {
+    SCOPED_CALL(SCOPE, fcollectmem, NVSHMEM_TEAM_WORLD, dest, src, bytes);
+}
+template <int SCOPE>
+__global__ void alltoall_kernel(char *dest, const char *src, size_t bytes) {
+    SCOPED_CALL(SCOPE, alltoallmem, NVSHMEM_TEAM_WORLD, dest, src, bytes);
+}
+
+template <int SCOPE>
+__global__ void barrier_kernel(uint64_t *counter, uint64_t *errors, int rounds) {
+    const int me = nvshmem_my_pe(), np = nvshmem_n_pes();
+    uint64_t *my_counter = (uint64_t *)nvshmem_ptr(counter, me);
+    uint64_t bad = 0;
+    for (int r = 1; r <= rounds; ++r) {
+        if (threadIdx.x == 0) *my_counter = (uint64_t)r;
+        SCOPED_CALL(SCOPE, barrier_all);
+        if (threadIdx.x == 0)
+            for (int q = 0; q < np; ++q) bad += nvshmem_uint64_g(counter, q) < (uint64_t)r;
+        // nobody may start round r+1 (and overwrite its counter) while others still check round r
+        SCOPED_CALL(SCOPE, barrier_all);
+    }
+    if (threadIdx.x == 0) *(uint64_t *)nvshmem_ptr(errors, me) += bad;
+}
+
+template <typename... Args>
+int launch_scoped(int scope, void (*kb)(Args...), void (*kw)(Args...), void (*kt)(Args...),
+                  int threads, void *stream, Args... a) {
+    void *args[] = {(void *)&a...};
+    const void *fn = scope == NVSHMEM_PERFTEST_SCOPE_BLOCK  ? (const void *)kb
+                     : scope == NVSHMEM_PERFTEST_SCOPE_WARP ? (const void *)kw
+                                                            : (const void *)kt;
+    return nvshmemx_collective_launch(fn, dim3(1), dim3(threads), args, 0, (hipStream_t)stream);
+}
+
+#define LAUNCH_REDUCE(TNAME, TYPE, OP)                                                           \
+    return launch_scoped<TYPE *, const TYPE *, size_t>(                                          \
+        scope, reduce_##TNAME##_##OP##_kernel<NVSHMEM_PERFTEST_SCOPE_BLOCK>,                     \
+        reduce_##TNAME##_##OP##_kernel<NVSHMEM_PERFTEST_SCOPE_WARP>,                             \
+        reduce_##TNAME##_##OP##_kernel<NVSHMEM_PERFTEST_SCOPE_THREAD>, threads, stream,          \
+        (TYPE *)dest, (const TYPE *)src, nreduce)
+
+}  // namespace
+
+extern "C" {
+
+int nvshmem_perftest_device_reduce(int dtype, int op, void *dest, const void *src, size_t nreduce,
+                                   int scope, int threads, void *stream) {
+    static const size_t esize[NVSHMEMI_DT_COUNT] = {1, 2, 4, 8, 1, 2, 4, 8, 2, 2, 4, 8};
+    if (!perftest::ready() || dtype < 0 || dtype >= NVSHMEMI_DT_COUNT || scope < 0 || scope > 2 ||
+        !perftest::check_launch(1, threads) || !perftest::check_range(dest, nreduce * esize[dtype]) ||
+        !perftest::check_range(src, nreduce * esize[dtype]))
+        return NVSHMEMX_ERROR_INVALID_VALUE;
+    const int key = dtype * 16 + op;
+    switch (key) {
+        case NVSHMEMI_DT_i32 * 16 + NVSHMEMI_OP_sum: LAUNCH_REDUCE(int32, int32_t, sum);
+        case NVSHMEMI_DT_i64 * 16 + NVSHMEMI_OP_xor: LAUNCH_REDUCE(int64, int64_t, xor);
+        case NVSHMEMI_DT_f32 * 16 + NVSHMEMI_OP_sum: LAUNCH_REDUCE(float, float, sum);
+        case NVSHMEMI_DT_f32 * 16 + NVSHMEMI_OP_max: LAUNCH_REDUCE(float, float, max);
+        case NVSHMEMI_DT_bf16 * 16 + NVSHMEMI_OP_sum: LAUNCH_REDUCE(bfloat16, nvshmem_bfloat16_t, sum);
+        case NVSHMEMI_DT_bf16 * 16 + NVSHMEMI_OP_max: LAUNCH_REDUCE(bfloat16, nvshmem_bfloat16_t, max);
+        case NVSHMEMI_DT_u64 * 16 + NVSHMEMI_OP_and: LAUNCH_REDUCE(uint64, uint64_t, and);
+        case NVSHMEMI_DT_f64 * 16 + NVSHMEMI_OP_prod: LAUNCH_REDUCE(double, double, prod);
+        case NVSHMEMI_DT_i16 * 16 + NVSHMEMI_OP_min: LAUNCH_REDUCE(int16, int16_t, min);
+        default: return NVSHMEMX_ERROR_NOT_SUPPORTED;
+    }
+}
+
+int nvshmem_perftest_device_fcollect(void *dest, const void *src, size_t bytes, int scope,
+                                     int threads, void *stream) {
+    if (!perftest::ready() || scope < 0 || scope > 2 || !perftest::check_launch(1, threads) ||
+        !perftest::check_range(dest, bytes * (size_t)nvshmem_n_pes()) ||
+        !perftest::check_range(src, bytes))
+        return NVSHMEMX_ERROR_INVALID_VALUE;
+    return launch_scoped<char *, const char *, size_t>(
+        scope, fcollect_kernel<NVSHMEM_PERFTEST_SCOPE_BLOCK>, fcollect_kernel<NVSHMEM_PERFTEST_SCOPE_WARP>,
+        fcollect_kernel<NVSHMEM_PERFTEST_SCOPE_THREAD>, threads, stream, (char *)dest,
+        (const char *)src, bytes);
+}
+
+int nvshmem_perftest_device_alltoall(void *dest, const void *src, size_t bytes, int scope,
+                                     int threads, void *stream) {
+    const size_t total = bytes * (size_t)nvshmem_n_pes();
+    if (!perftest::ready() || scope < 0 || scope > 2 || !perftest::check_launch(1, threads) ||
+        !perftest::check_range(dest, total) || !perftest::check_range(src, total))
+        return NVSHMEMX_ERROR_INVALID_VALUE;
+    return launch_scoped<char *, const char *, size_t>(
+        scope, alltoall_kernel<NVSHMEM_PERFTEST_SCOPE_BLOCK>, alltoall_kernel<NVSHMEM_PERFTEST_SCOPE_WARP>,
+        alltoall_kernel<NVSHMEM_PERFTEST_SCOPE_THREAD>, threads, stream, (char *)dest,
+        (const char *)src, bytes);
+}
+
+int nvshmem_perftest_device_barrier(uint64_t *counter, uint64_t *errors, int rounds, int scope,
+                                    int threads, void *stream) {
+    if (!perftest::ready() || scope < 0 || scope > 2 || !perftest::check_launch(1, threads) ||
+        !perftest::check_range(counter, sizeof(uint64_t)) ||
+        !perftest::check_range(errors, sizeof(uint64_t)))
+        return NVSHMEMX_ERROR_INVALID_VALUE;
+    return launch_scoped<uint64_t *, uint64_t *, int>(
+        scope, barrier_kernel<NVSHMEM_PERFTEST_SCOPE_BLOCK>, barrier_kernel<NVSHMEM_PERFTEST_SCOPE_WARP>,
+        barrier_kernel<NVSHMEM_PERFTEST_SCOPE_THREAD>, threads, stream, counter, errors, rounds);
+}
+
+}  // extern "C"

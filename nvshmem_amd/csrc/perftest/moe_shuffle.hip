@@ -1,0 +1,256 @@
+// MoE token shuffle on logical PEs: dispatch rows to the PEs that own their experts with
+// put + signal, wait for the expected row counts, and combine (gather the rows back).
+//
+// Workload model: examples/moe_shuffle.cu in the reference tree (offset exchange :204-234, one row
+// per thread group pushed to `expert / experts_per_pe` :240-289); the signalling idiom is the
+// put_signal_nbi + signal_wait_until(GE) pair of examples/ring-reduce.cu:111-127.
+//
+// A row of 14336 bytes is 896 16-byte vectors: a wavefront moves it with 14 vectors per lane, so
+// the default scope is one row per wavefront with no block-wide synchronisation in the loop.
+#include <hip/hip_runtime.h>
+
+#include "nvshmem_perftest.h"
+#include "nvshmemx.h"
+#include "perftest_common.hpp"
+
+namespace {
+
+constexpr int kMaxPes = NVSHMEMI_AMD_MAX_PES;
+
+// A routing entry that points outside the receive buffer is skipped instead of written.
+__device__ __forceinline__ bool row_ok(int pe, int64_t row, int np, size_t cap_rows) {
+    return (unsigned)pe < (unsigned)np && (uint64_t)row < (uint64_t)cap_rows;
+}
+
+// Dispatch.  Rows are dealt round-robin to the thread groups of the PE's blocks.  Each group tallies
+// what it sent to every destination; once all its puts are complete it adds the tallies to the
+// destinations' signal words (one release + npes atomic adds per block instead of one per row).
+template <bool WARP_SCOPED>
+__global__ void moe_dispatch_kernel(char *recv, const char *send, const int32_t *dest_pe,
+                                    const int64_t *dest_row, const uint64_t *expected,
+                                    uint64_t *sig, int tokens, int topk, size_t row_bytes,
+                                    size_t recv_cap_rows) {
+    __shared__ unsigned tally[kMaxPes];
+    const int me = nvshmem_my_pe(), np = nvshmem_n_pes();
+    const int32_t *my_dest_pe = (const int32_t *)nvshmem_ptr(dest_pe, me);
+    const int64_t *my_dest_row = (const int64_t *)nvshmem_ptr(dest_row, me);
+    const size_t rows = (size_t)tokens * (size_t)topk;
+    for (int i = threadIdx.x; i < np; i += blockDim.x) tally[i] = 0;
+    __syncthreads();
+
+    if (WARP_SCOPED) {
+        const size_t waves_per_block = blockDim.x / NVSHMEMI_WARP_SIZE;
+        const size_t wave = blockIdx.x * waves_per_block + threadIdx.x / NVSHMEMI_WARP_SIZE;
+        const size_t nwaves = (size_t)gridDim.x * waves_per_block;
+        const bool lane0 = (threadIdx.x % NVSHMEMI_WARP_SIZE) == 0;
+        for (size_t r = wave; r < rows; r += nwaves) {
+            const int pe = my_dest_pe[r];
+            if (!row_ok(pe, my_dest_row[r], np, recv_cap_rows)) continue;
+            nvshmemx_putmem_nbi_warp(recv + (size_t)my_dest_row[r] * row_bytes,
+                                     send + (r / (size_t)topk) * row_bytes, row_bytes, pe);
+            if (lane0) atomicAdd(&tally[pe], 1u);
+        }
+    } else {
+        for (size_t r = blockIdx.x; r < rows; r += gridDim.x) {
+            const int pe = my_dest_pe[r];
+            if (!row_ok(pe, my_dest_row[r], np, recv_cap_rows)) continue;
+            nvshmemx_putmem_nbi_block(recv + (size_t)my_dest_row[r] * row_bytes,
+                                      send + (r / (size_t)topk) * row_bytes, row_bytes, pe);
+            if (threadIdx.x == 0) tally[pe] += 1u;
+        }
+    }
+    // all rows of this block are written; publish the counts
+    nvshmemx_quiet_block();
+    for (int pe = threadIdx.x; pe < np; pe += blockDim.x)
+        if (tally[pe]) nvshmemx_signal_op(sig + me, (uint64_t)tally[pe], NVSHMEM_SIGNAL_ADD, pe);
+
+    // receiver side: block 0 of every PE waits until each source has delivered what it announced
+    if (blockIdx.x == 0) {
+        const uint64_t *my_expected = (const uint64_t *)nvshmem_ptr(expected, me);
+        for (int src = threadIdx.x; src < np; src += blockDim.x)
+            nvshmem_signal_wait_until(sig + src, NVSHMEM_CMP_GE, my_expected[src]);
+    }
+}
+
+// Per-row signalling: the API-literal form, one nvshmemx_putmem_signal_nbi per row.
+template <bool WARP_SCOPED>
+__global__ void moe_dispatch_rowsignal_kernel(char *recv, const char *send, const int32_t *dest_pe,
+                                              const int64_t *dest_row, const uint64_t *expected,
+                                              uint64_t *sig, int tokens, int topk,
+                                              size_t row_bytes, size_t recv_cap_rows) {
+    const int me = nvshmem_my_pe(), np = nvshmem_n_pes();
+    const int32_t *my_dest_pe = (const int32_t *)nvshmem_ptr(dest_pe, me);
+    const int64_t *my_dest_row = (const int64_t *)nvshmem_ptr(dest_row, me);
+    const size_t rows = (size_t)tokens * (size_t)topk;
+    if (WARP_SCOPED) {
+        const size_t waves_per_block = blockDim.x / NVSHMEMI_WARP_SIZE;
+        const size_t wave = blockIdx.x * waves_per_block + threadIdx.x / NVSHMEMI_WARP_SIZE;
+        const size_t nwaves = (size_t)gridDim.x * waves_per_block;
+        for (size_t r = wave; r < rows; r += nwaves)
+            if (row_ok(my_dest_pe[r], my_dest_row[r], np, recv_cap_rows))
+            nvshmemx_putmem_signal_nbi_warp(recv + (size_t)my_dest_row[r] * row_bytes,
+                                            send + (r / (size_t)topk) * row_bytes, row_bytes,
+                                            sig + me, 1, NVSHMEM_SIGNAL_ADD, my_dest_pe[r]);
+    } else {
+        for (size_t r = blockIdx.x; r < rows; r += gridDim.x)
+            if (row_ok(my_dest_pe[r], my_dest_row[r], np, recv_cap_rows))
+            nvshmemx_putmem_signal_nbi_block(recv + (size_t)my_dest_row[r] * row_bytes,
+                                             send + (r / (size_t)topk) * row_bytes, row_bytes,
+                                             sig + me, 1, NVSHMEM_SIGNAL_ADD, my_dest_pe[r]);
+    }
+    if (blockIdx.x == 0) {
+        const uint64_t *my_expected = (const uint64_t *)nvshmem_ptr(expected, me);
+        for (int src = threadIdx.x; src < np; src += blockDim.x)
+            nvshmem_signal_wait_until(sig + src, NVSHMEM_CMP_GE, my_expected[src]);
+    }
+}
+
+template <bool WARP_SCOPED>
+__global__ void moe_combine_kernel(char *out, const char *recv, const int32_t *dest_pe,
+                                   const int64_t *dest_row, int tokens, int topk,
+                                   size_t row_bytes, size_t recv_cap_rows) {
+    const int me = nvshmem_my_pe();
+    const int np = nvshmem_n_pes();
+    const int32_t *my_dest_pe = (const int32_t *)nvshmem_ptr(dest_pe, me);
+    const int64_t *my_dest_row = (const int64_t *)nvshmem_ptr(dest_row, me);
+    const size_t rows = (size_t)tokens * (size_t)topk;
+    if (WARP_SCOPED) {
+        const size_t waves_per_block = blockDim.x / NVSHMEMI_WARP_SIZE;
+        const size_t wave = blockIdx.x * waves_per_block + threadIdx.x / NVSHMEMI_WARP_SIZE;
+        const size_t nwaves = (size_t)gridDim.x * waves_per_block;
+        for (size_t r = wave; r < rows; r += nwaves)
+            if (row_ok(my_dest_pe[r], my_dest_row[r], np, recv_cap_rows))
+            nvshmemx_getmem_nbi_warp(out + r * row_bytes, recv + (size_t)my_dest_row[r] * row_bytes,
+                                     row_bytes, my_dest_pe[r]);
+    } else {
+        for (size_t r = blockIdx.x; r < rows; r += gridDim.x)
+            if (row_ok(my_dest_pe[r], my_dest_row[r], np, recv_cap_rows))
+            nvshmemx_getmem_nbi_block(out + r * row_bytes, recv + (size_t)my_dest_row[r] * row_bytes,
+                                      row_bytes, my_dest_pe[r]);
+    }
+}
+
+// counts exchange + prefix sums: every PE fetches all PEs' per-expert counts with scalar gets and
+// lays out the receive segments of every destination PE in (expert, source PE) order.
+__global__ void moe_exchange_offsets_kernel(const int64_t *counts, int64_t *seg_base,
+                                            int64_t *recv_rows, int num_experts) {
+    extern __shared__ int64_t table[];  // [expert][src]
+    const int me = nvshmem_my_pe(), np = nvshmem_n_pes();
+    const int epp = num_experts / np;
+    for (int i = threadIdx.x; i < num_experts * np; i += blockDim.x)
+        table[i] = nvshmem_int64_g(counts + i / np, i % np);
+    __syncthreads();
+    int64_t *my_seg = (int64_t *)nvshmem_ptr(seg_base, me);
+    for (int d = threadIdx.x; d < np; d += blockDim.x) {
+        int64_t run = 0;
+        for (int i = d * epp * np; i < (d + 1) * epp * np; ++i) {
+            my_seg[i] = run;
+            run += table[i];
+        }
+        if (d == me) ((int64_t *)nvshmem_ptr(recv_rows, me))[0] = run;
+    }
+}
+
+bool moe_args_ok(const void *table_pe, const void *table_row, int tokens, int topk,
+                 size_t row_bytes, int blocks, int threads, bool warp) {
+    if (!perftest::ready() || tokens < 1 || topk < 1 || row_bytes == 0 ||
+        !perftest::check_launch(blocks, threads))
+        return false;
+    if (warp && (threads % NVSHMEMI_WARP_SIZE)) {
+        fprintf(stderr, "nvshmem_perftest: warp-scoped shuffle needs a multiple of 64 threads\n");
+        return false;
+    }
+    const size_t rows = (size_t)tokens * (size_t)topk;
+    return perftest::check_range(table_pe, rows * sizeof(int32_t)) &&
+           perftest::check_range(table_row, rows * sizeof(int64_t));
+}
+
+}  // namespace
+
+extern "C" {
+
+// scope: NVSHMEM_PERFTEST_SCOPE_WARP (row per wavefront) or _BLOCK (row per block);
+// bit 8 set (scope | 256) selects per-row signalling instead of per-block tallies.
+int nvshmem_perftest_moe_dispatch_ex(void *recv, size_t recv_cap_rows, const void *send, const int32_t *dest_pe,
+                                     const int64_t *dest_row, const uint64_t *expected,
+                                     uint64_t *sig, int tokens, int topk, size_t row_bytes,
+                                     int blocks_per_pe, int threads, int scope, void *stream) {
+    const bool per_row = (scope & 256) != 0;
+    const bool warp = (scope & 255) == NVSHMEM_PERFTEST_SCOPE_WARP;
+    if (!warp && (scope & 255) != NVSHMEM_PERFTEST_SCOPE_BLOCK) return NVSHMEMX_ERROR_INVALID_VALUE;
+    if (!moe_args_ok(dest_pe, dest_row, tokens, topk, row_bytes, blocks_per_pe, threads, warp))
+        return NVSHMEMX_ERROR_INVALID_VALUE;
+    const size_t words = sizeof(uint64_t) * (size_t)nvshmem_n_pes();
+    if (!perftest::check_range(expected, words) || !perftest::check_range(sig, words) ||
+        !perftest::check_range(send, (size_t)tokens * row_bytes) ||
+        !perftest::check_range(recv, recv_cap_rows * row_bytes))
+        return NVSHMEMX_ERROR_INVALID_VALUE;
+    char *r = (char *)recv;
+    const char *s = (const char *)send;
+    void *args[] = {&r, &s, &dest_pe, &dest_row, &expected, &sig, &tokens, &topk, &row_bytes,
+                    &recv_cap_rows};
+    const void *fn;
+    if (per_row)
+        fn = warp ? (const void *)moe_dispatch_rowsignal_kernel<true>
+                  : (const void *)moe_dispatch_rowsignal_kernel<false>;
+    else
+        fn = warp ? (const void *)moe_dispatch_kernel<true> : (const void *)moe_dispatch_kernel<false>;
+    return nvshmemx_collective_launch(fn, dim3(blocks_per_pe), dim3(threads), args, 0,
+                                      (hipStream_t)stream);
+}
+
+int nvshmem_perftest_moe_dispatch(void *recv, size_t recv_cap_rows, const void *send, const int32_t *dest_pe,
+                                  const int64_t *dest_row, const uint64_t *expected, uint64_t *sig,
+                                  int tokens, int topk, size_t row_bytes, int blocks_per_pe,
+                                  int threads, void *stream) {
+    return nvshmem_perftest_moe_dispatch_ex(recv, recv_cap_rows, send, dest_pe, dest_row, expected, sig, tokens,
+                                            topk, row_bytes, blocks_per_pe, threads,
+                                            NVSHMEM_PERFTEST_SCOPE_WARP, stream);
+}
+
+int nvshmem_perftest_moe_combine_ex(void *out, const void *recv, size_t recv_cap_rows, const int32_t *dest_pe,
+                                    const int64_t *dest_row, int tokens, int topk,
+                                    size_t row_bytes, int blocks_per_pe, int threads, int scope,
+                                    void *stream) {
+    const bool warp = scope == NVSHMEM_PERFTEST_SCOPE_WARP;
+    if (!warp && scope != NVSHMEM_PERFTEST_SCOPE_BLOCK) return NVSHMEMX_ERROR_INVALID_VALUE;
+    if (!moe_args_ok(dest_pe, dest_row, tokens, topk, row_bytes, blocks_per_pe, threads, warp) ||
+        !perftest::check_range(out, (size_t)tokens * (size_t)topk * row_bytes) ||
+        !perftest::check_range(recv, recv_cap_rows * row_bytes))
+        return NVSHMEMX_ERROR_INVALID_VALUE;
+    const dim3 grid((unsigned)blocks_per_pe, 1, (unsigned)nvshmem_n_pes());
+    if (warp)
+        hipLaunchKernelGGL(moe_combine_kernel<true>, grid, dim3(threads), 0, (hipStream_t)stream,
+                           (char *)out, (const char *)recv, dest_pe, dest_row, tokens, topk, row_bytes,
+                           recv_cap_rows);
+    else
+        hipLaunchKernelGGL(moe_combine_kernel<false>, grid, dim3(threads), 0, (hipStream_t)stream,
+                           (char *)out, (const char *)recv, dest_pe, dest_row, tokens, topk, row_bytes,
+                           recv_cap_rows);
+    return perftest::launch_status("moe_combine");
+}
+
+int nvshmem_perftest_moe_combine(void *out, const void *recv, size_t recv_cap_rows, const int32_t *dest_pe,
+                                 const int64_t *dest_row, int tokens, int topk, size_t row_bytes,
+                                 int blocks_per_pe, int threads, void *stream) {
+    return nvshmem_perftest_moe_combine_ex(out, recv, recv_cap_rows, dest_pe, dest_row, tokens, topk, row_bytes,
+                                           blocks_per_pe, threads, NVSHMEM_PERFTEST_SCOPE_WARP,
+                                           stream);
+}
+
+int nvshmem_perftest_moe_exchange_offsets(const int64_t *counts, int64_t *seg_base,
+                                          int64_t *recv_rows, int num_experts, void *stream) {
+    const int np = nvshmem_n_pes();
+    if (!perftest::ready() || num_experts < np || num_experts % np ||
+        (size_t)num_experts * np * sizeof(int64_t) > 64 * 1024 ||
+        !perftest::check_range(counts, sizeof(int64_t) * (size_t)num_experts) ||
+        !perftest::check_range(seg_base, sizeof(int64_t) * (size_t)num_experts * np) ||
+        !perftest::check_range(recv_rows, sizeof(int64_t)))
+        return NVSHMEMX_ERROR_INVALID_VALUE;
+    hipLaunchKernelGGL(moe_exchange_offsets_kernel, dim3(1, 1, (unsigned)np), dim3(256),
+                       (size_t)num_experts * np * sizeof(int64_t), (hipStream_t)stream, counts,
+                       seg_base, recv_rows, num_experts);
+    return perftest::launch_status("moe_exchange_offsets");
+}
+
+}  // extern "C"

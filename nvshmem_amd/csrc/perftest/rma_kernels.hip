@@ -1,0 +1,230 @@
+// Point-to-point kernels written against the public device API: ring put/get in the three scopes,
+// scalar p/g, signal operations, bounded waits, put_signal ping-pong and the ring allreduce built
+// from put_signal + signal_wait_until.
+//
+// Counterparts in the reference tree: perftest/device/pt-to-pt/shmem_put_bw.cu:21-60,
+// perftest/device/pt-to-pt/shmem_put_signal_ping_pong_latency.cu:29-49, examples/put-block.cu:30-60,
+// examples/ring-reduce.cu:88-144.
+#include <hip/hip_runtime.h>
+
+#include "nvshmem_perftest.h"
+#include "nvshmemx.h"
+#include "perftest_common.hpp"
+
+namespace {
+
+// Slice [off, off+len) of a `bytes` long message owned by part `idx` of `parts`.
+__device__ __forceinline__ bool slice_of(size_t bytes, size_t parts, size_t idx, size_t *off,
+                                         size_t *len) {
+    if (bytes < parts) {
+        *off = 0;
+        *len = bytes;
+        return idx == 0;
+    }
+    const size_t per = bytes / parts;
+    *off = idx * per;
+    *len = (idx == parts - 1) ? bytes - *off : per;
+    return true;
+}
+
+template <int SCOPE, bool GET>
+__global__ void ring_rma_kernel(char *dest, const char *src, size_t bytes) {
+    const int peer = (nvshmem_my_pe() + 1) % nvshmem_n_pes();
+    size_t off, len;
+    if (!slice_of(bytes, gridDim.x, blockIdx.x, &off, &len)) return;
+    if (SCOPE == NVSHMEM_PERFTEST_SCOPE_BLOCK) {
+        if (GET) nvshmemx_getmem_block(dest + off, src + off, len, peer);
+        else nvshmemx_putmem_block(dest + off, src + off, len, peer);
+    } else if (SCOPE == NVSHMEM_PERFTEST_SCOPE_WARP) {
+        const size_t waves = (blockDim.x + NVSHMEMI_WARP_SIZE - 1) / NVSHMEMI_WARP_SIZE;
+        size_t woff, wlen;
+        if (!slice_of(len, waves, threadIdx.x / NVSHMEMI_WARP_SIZE, &woff, &wlen)) return;
+        if (GET) nvshmemx_getmem_warp(dest + off + woff, src + off + woff, wlen, peer);
+        else nvshmemx_putmem_warp(dest + off + woff, src + off + woff, wlen, peer);
+    } else {
+        size_t toff, tlen;
+        if (!slice_of(len, blockDim.x, threadIdx.x, &toff, &tlen)) return;
+        if (GET) nvshmem_getmem(dest + off + toff, src + off + toff, tlen, peer);
+        else nvshmem_putmem(dest + off + toff, src + off + toff, tlen, peer);
+    }
+}
+
+__global__ void p_g_kernel(uint64_t *words, uint64_t *out, uint64_t value_base) {
+    const int me = nvshmem_my_pe(), np = nvshmem_n_pes();
+    nvshmem_uint64_p(words + me, value_base + (uint64_t)me, (me + 1) % np);
+    nvshmem_barrier_all();
+    uint64_t *mine = (uint64_t *)nvshmem_ptr(out, me);
+    for (int q = 0; q < np; ++q) mine[q] = nvshmem_uint64_g(words + (q + np - 1) % np, q);
+}
+
+__global__ void signal_op_kernel(uint64_t *sig, uint64_t value, int sig_op, int reps) {
+    const int peer = (nvshmem_my_pe() + 1) % nvshmem_n_pes();
+    for (int r = 0; r < reps; ++r) nvshmemx_signal_op(sig, value, sig_op, peer);
+}
+
+__global__ void signal_wait_kernel(uint64_t *sig, int cmp, uint64_t cmp_value, uint64_t *out) {
+    const uint64_t got = nvshmem_signal_wait_until(sig, cmp, cmp_value);
+    ((uint64_t *)nvshmem_ptr(out, nvshmem_my_pe()))[0] = got;
+}
+
+__global__ void pingpong_kernel(char *data, uint64_t *sig, size_t bytes, int iters) {
+    const int me = nvshmem_my_pe();
+    if (me > 1) return;
+    for (int i = 1; i <= iters; ++i) {
+        if (me == 0) {
+            nvshmemx_putmem_signal_block(data, data, bytes, sig, (uint64_t)i, NVSHMEM_SIGNAL_SET, 1);
+            if (threadIdx.x == 0) nvshmem_signal_wait_until(sig, NVSHMEM_CMP_EQ, (uint64_t)i);
+            __syncthreads();
+        } else {
+            if (threadIdx.x == 0) nvshmem_signal_wait_until(sig, NVSHMEM_CMP_EQ, (uint64_t)i);
+            __syncthreads();
+            nvshmemx_putmem_signal_block(data, data, bytes, sig, (uint64_t)i, NVSHMEM_SIGNAL_SET, 0);
+        }
+    }
+}
+
+// Ring allreduce: the partial sum travels PE 0 -> 1 -> ... -> n-1 chunk by chunk (reduce phase),
+// then the finished chunks travel n-1 -> 0 -> ... -> n-2 (broadcast phase).  A signal word per
+// block counts the chunks that have arrived.
+__global__ void ring_reduce_kernel(int32_t *dst, const int32_t *src, size_t nreduce,
+                                   uint64_t *signal, size_t chunk_elems) {
+    const int me = nvshmem_my_pe(), np = nvshmem_n_pes();
+    const int peer = (me + 1) % np;
+    const size_t per_block = nreduce / gridDim.x;
+    const size_t chunks = per_block / chunk_elems;
+    dst += (size_t)blockIdx.x * per_block;
+    src += (size_t)blockIdx.x * per_block;
+    signal += blockIdx.x;
+    int32_t *my_dst = (int32_t *)nvshmem_ptr(dst, me);
+    const int32_t *my_src = (const int32_t *)nvshmem_ptr(src, me);
+
+    for (size_t c = 0; c < chunks; ++c) {
+        const size_t at = c * chunk_elems;
+        if (me != 0) {
+            if (threadIdx.x == 0) nvshmem_signal_wait_until(signal, NVSHMEM_CMP_GE, c + 1);
+            __syncthreads();
+            for (size_t i = threadIdx.x; i < chunk_elems; i += blockDim.x)
+                my_dst[at + i] = (int32_t)((uint32_t)my_dst[at + i] + (uint32_t)my_src[at + i]);
+            __syncthreads();
+        }
+        nvshmemx_int32_put_signal_nbi_block(dst + at, (me == 0) ? src + at : dst + at, chunk_elems,
+                                            signal, 1, NVSHMEM_SIGNAL_ADD, peer);
+    }
+    for (size_t c = 0; c < chunks; ++c) {
+        const size_t at = c * chunk_elems;
+        if (me < np - 1) {
+            if (threadIdx.x == 0)
+                nvshmem_signal_wait_until(signal, NVSHMEM_CMP_GE, (me == 0) ? c + 1 : chunks + c + 1);
+            __syncthreads();
+        }
+        if (me < np - 2)
+            nvshmemx_int32_put_signal_nbi_block(dst + at, dst + at, chunk_elems, signal, 1,
+                                                NVSHMEM_SIGNAL_ADD, peer);
+    }
+    __syncthreads();
+    if (threadIdx.x == 0) *(uint64_t *)nvshmem_ptr(signal, me) = 0;  // ready for the next run
+}
+
+template <int SCOPE>
+int launch_ring(bool is_get, char *dest, const char *src, size_t bytes, int blocks, int threads,
+                hipStream_t stream) {
+    const dim3 grid((unsigned)blocks, 1, (unsigned)nvshmem_n_pes());
+    if (is_get)
+        hipLaunchKernelGGL((ring_rma_kernel<SCOPE, true>), grid, dim3(threads), 0, stream, dest, src, bytes);
+    else
+        hipLaunchKernelGGL((ring_rma_kernel<SCOPE, false>), grid, dim3(threads), 0, stream, dest, src, bytes);
+    return perftest::launch_status("ring_rma");
+}
+
+}  // namespace
+
+extern "C" {
+
+int nvshmem_perftest_ring_rma(void *dest, const void *src, size_t bytes, int blocks_per_pe,
+                              int threads, int scope, int is_get, int iters, void *stream) {
+    if (!perftest::ready() || !perftest::check_launch(blocks_per_pe, threads) ||
+        !perftest::check_range(dest, bytes) || !perftest::check_range(src, bytes))
+        return NVSHMEMX_ERROR_INVALID_VALUE;
+    if (bytes == 0) return 0;
+    int rc = 0;
+    for (int i = 0; i < iters && rc == 0; ++i) {
+        switch (scope) {
+            case NVSHMEM_PERFTEST_SCOPE_BLOCK:
+                rc = launch_ring<NVSHMEM_PERFTEST_SCOPE_BLOCK>(is_get, (char *)dest, (const char *)src,
+                                                               bytes, blocks_per_pe, threads,
+                                                               (hipStream_t)stream);
+                break;
+            case NVSHMEM_PERFTEST_SCOPE_WARP:
+                rc = launch_ring<NVSHMEM_PERFTEST_SCOPE_WARP>(is_get, (char *)dest, (const char *)src,
+                                                              bytes, blocks_per_pe, threads,
+                                                              (hipStream_t)stream);
+                break;
+            case NVSHMEM_PERFTEST_SCOPE_THREAD:
+                rc = launch_ring<NVSHMEM_PERFTEST_SCOPE_THREAD>(is_get, (char *)dest, (const char *)src,
+                                                                bytes, blocks_per_pe, threads,
+                                                                (hipStream_t)stream);
+                break;
+            default:
+                return NVSHMEMX_ERROR_INVALID_VALUE;
+        }
+    }
+    return rc;
+}
+
+int nvshmem_perftest_p_g(uint64_t *words, uint64_t *out, uint64_t value_base, void *stream) {
+    const size_t row = sizeof(uint64_t) * (size_t)nvshmem_n_pes();
+    if (!perftest::ready() || !perftest::check_range(words, row) || !perftest::check_range(out, row))
+        return NVSHMEMX_ERROR_INVALID_VALUE;
+    void *args[] = {&words, &out, &value_base};
+    return nvshmemx_collective_launch((const void *)p_g_kernel, dim3(1), dim3(1), args, 0,
+                                      (hipStream_t)stream);
+}
+
+int nvshmem_perftest_signal_op(uint64_t *sig, uint64_t value, int sig_op, int threads, int reps,
+                               void *stream) {
+    if (!perftest::ready() || !perftest::check_launch(1, threads) ||
+        !perftest::check_range(sig, sizeof(uint64_t)))
+        return NVSHMEMX_ERROR_INVALID_VALUE;
+    if (sig_op != NVSHMEM_SIGNAL_SET && sig_op != NVSHMEM_SIGNAL_ADD)
+        return NVSHMEMX_ERROR_INVALID_VALUE;
+    hipLaunchKernelGGL(signal_op_kernel, dim3(1, 1, (unsigned)nvshmem_n_pes()), dim3(threads), 0,
+                       (hipStream_t)stream, sig, value, sig_op, reps);
+    return perftest::launch_status("signal_op");
+}
+
+int nvshmem_perftest_signal_wait(uint64_t *sig, int cmp, uint64_t cmp_value, uint64_t *out,
+                                 void *stream) {
+    if (!perftest::ready() || !perftest::check_range(sig, sizeof(uint64_t)) ||
+        !perftest::check_range(out, sizeof(uint64_t)))
+        return NVSHMEMX_ERROR_INVALID_VALUE;
+    hipLaunchKernelGGL(signal_wait_kernel, dim3(1, 1, (unsigned)nvshmem_n_pes()), dim3(1), 0,
+                       (hipStream_t)stream, sig, cmp, cmp_value, out);
+    return perftest::launch_status("signal_wait");
+}
+
+int nvshmem_perftest_put_signal_pingpong(void *data, uint64_t *sig, size_t bytes, int iters,
+                                         int threads, void *stream) {
+    if (!perftest::ready() || nvshmem_n_pes() < 2 || !perftest::check_launch(1, threads) ||
+        !perftest::check_range(data, bytes) || !perftest::check_range(sig, sizeof(uint64_t)))
+        return NVSHMEMX_ERROR_INVALID_VALUE;
+    char *d = (char *)data;
+    void *args[] = {&d, &sig, &bytes, &iters};
+    return nvshmemx_collective_launch((const void *)pingpong_kernel, dim3(1), dim3(threads), args,
+                                      0, (hipStream_t)stream);
+}
+
+int nvshmem_perftest_ring_reduce(int32_t *dst, const int32_t *src, size_t nreduce,
+                                 uint64_t *signal, size_t chunk_elems, int blocks, int threads,
+                                 void *stream) {
+    if (!perftest::ready() || !perftest::check_launch(blocks, threads) || chunk_elems == 0 ||
+        nreduce % ((size_t)blocks * chunk_elems) != 0 ||
+        !perftest::check_range(dst, nreduce * sizeof(int32_t)) ||
+        !perftest::check_range(src, nreduce * sizeof(int32_t)) ||
+        !perftest::check_range(signal, sizeof(uint64_t) * (size_t)blocks))
+        return NVSHMEMX_ERROR_INVALID_VALUE;
+    void *args[] = {&dst, &src, &nreduce, &signal, &chunk_elems};
+    return nvshmemx_collective_launch((const void *)ring_reduce_kernel, dim3(blocks), dim3(threads),
+                                      args, 0, (hipStream_t)stream);
+}
+
+}  // extern "C"

@@ -1,0 +1,68 @@
+// Process-wide state of the logical-PE runtime, shared by the host translation units of
+// libnvshmem_amd.so.
+#pragma once
+
+#include <hip/hip_runtime.h>
+
+#include <cstdarg>
+#include <cstdint>
+#include <memory>
+#include <mutex>
+#include <set>
+#include <string>
+
+#include "mspace.hpp"
+#include "nvshmem_amd/nvshmem_host_api.h"
+
+namespace nvshmem_amd {
+
+struct Runtime {
+    std::recursive_mutex mu;
+    bool initialized = false;
+    int device = 0;
+    int npes = 0;
+    int num_cus = 0;
+    uint32_t heap_shift = 0;
+    uint64_t heap_size = 0;  // bytes per PE, power of two
+    char *base = nullptr;    // start of PE 0's slice
+    std::unique_ptr<SymmetricSpace> space;
+    nvshmemi_device_state_t dev{};
+    std::set<nvshmemi_amd_state_updater_t> updaters;  // one per translation unit with a state block
+    bool symbols_stale = false;
+
+    static Runtime &get();
+
+    // Offset of a symmetric address inside its PE slice; false when p is outside the heap.
+    bool offset_of(const void *p, uint64_t *off) const {
+        const uint64_t d = (uint64_t)((const char *)p - base);
+        if (!initialized || p == nullptr || (const char *)p < base ||
+            d >= ((uint64_t)npes << heap_shift))
+            return false;
+        *off = d & (heap_size - 1);
+        return true;
+    }
+    char *slice(int pe) const { return base + ((uint64_t)pe << heap_shift); }
+};
+
+// Records a message for nvshmemx_amd_last_error() and prints it to stderr.
+void set_error(const char *fmt, ...) __attribute__((format(printf, 1, 2)));
+void clear_error();
+
+// Pushes the state block to every registered translation unit when it changed.
+void refresh_symbols(Runtime &rt, bool force);
+
+// Common argument check of the collectives and RMA calls: [p, p+bytes) must lie inside one PE
+// slice.  Returns the offset through *off.
+bool check_symmetric_range(Runtime &rt, const char *what, const void *p, uint64_t bytes,
+                           uint64_t *off);
+
+#define NVSHMEM_AMD_HIP_CHECK(expr)                                                        \
+    do {                                                                                   \
+        hipError_t e_ = (expr);                                                            \
+        if (e_ != hipSuccess) {                                                            \
+            ::nvshmem_amd::set_error("%s failed: %s (%s:%d)", #expr, hipGetErrorString(e_), \
+                                     __FILE__, __LINE__);                                  \
+        }                                                                                  \
+    } while (0)
+
+}  // namespace nvshmem_amd
