@@ -1,0 +1,192 @@
+"""GPU parity of signals, waits, scalar p/g and the in-kernel barrier (a5-a7) through the C ABI,
+plus the reference's put_signal workloads (ping-pong, ring allreduce) with their known answers."""
+import ctypes as C
+
+import numpy as np
+import pytest
+
+import nvshmem_amd as N
+import oracle_lib as O
+from gpu_util import note, runtime
+from nvshmem_amd import hip
+
+pytestmark = pytest.mark.gpu
+NPES = 8
+
+
+@pytest.fixture(scope="module")
+def rt():
+    with runtime(NPES, 1 << 28) as r:
+        yield r
+
+
+def _words(rt, sym, n=1):
+    return rt.download_all(sym, (n,), np.uint64)
+
+
+def test_signal_add_accumulates_exactly_and_set_overwrites(rt):
+    perf = rt.perftest()
+    sig = rt.calloc(8, 8)
+    L = O.lib()
+    note("signal_op ADD")
+    assert perf.nvshmem_perftest_signal_op(sig, 3, N.SIGNAL_ADD, 256, 10, None) == 0
+    rt.sync()
+    want = 0
+    for _ in range(256 * 10):
+        want = L.oracle_signal_op(want, 3, N.SIGNAL_ADD)
+    assert (_words(rt, sig)[:, 0] == want).all() and want == 7680
+    note("signal_op SET")
+    assert perf.nvshmem_perftest_signal_op(sig, 41, N.SIGNAL_SET, 64, 2, None) == 0
+    rt.sync()
+    assert (_words(rt, sig)[:, 0] == L.oracle_signal_op(want, 41, N.SIGNAL_SET)).all()
+    assert perf.nvshmem_perftest_signal_op(sig, 1, 7, 64, 1, None) != 0     # unknown operator
+    rt.free(sig)
+
+
+def test_host_signal_op_and_wait_on_stream(rt):
+    sig = rt.calloc(8, 8)
+    s = hip.Stream()
+    note("signal_op_on_stream / signal_wait_until_on_stream")
+    rt.lib.nvshmemx_signal_op_on_stream(sig, 5, N.SIGNAL_SET, 3, s.ptr)
+    rt.lib.nvshmemx_signal_op_on_stream(sig, 2, N.SIGNAL_ADD, 3, s.ptr)
+    rt.lib.nvshmemx_signal_op_on_stream(sig, 2, N.SIGNAL_ADD, 3, s.ptr)
+    # the wait is stream-ordered behind the updates: it is satisfied when it starts
+    rt.lib.nvshmemx_signal_wait_until_on_stream(rt.ptr(sig, 3), N.CMP["EQ"], 9, s.ptr)
+    s.synchronize()
+    w = _words(rt, sig)[:, 0]
+    assert w[3] == 9 and w.sum() == 9
+    assert rt.read_timeout(0)[0] == 0
+    # put + signal from the host: data lands before the signal
+    a = rt.malloc(4096); b = rt.calloc(4096, 1)
+    data = O.fill_all("bytes", NPES, 4096, 21)
+    rt.upload_all(a, data)
+    rt.lib.nvshmemx_putmem_signal_on_stream(b, a, 4096, sig, 100, N.SIGNAL_SET, 6, s.ptr)
+    s.synchronize()
+    assert np.array_equal(rt.download(b, 6, (4096,), np.uint8), data[0])
+    assert _words(rt, sig)[6, 0] == 100
+    rt.lib.nvshmemx_signal_op_on_stream(sig, 1, 4, 0, s.ptr)
+    assert b"neither SET" in rt.lib.nvshmemx_amd_last_error()
+    s.destroy()
+    rt.free(sig); rt.free(a); rt.free(b)
+
+
+@pytest.mark.parametrize("cmp_name", ["EQ", "NE", "GT", "LE", "LT", "GE"])
+def test_signal_wait_until_returns_the_satisfying_value(rt, cmp_name):
+    perf = rt.perftest()
+    L = O.lib()
+    sig = rt.calloc(8, 8); out = rt.calloc(8, 8)
+    # a preset value per PE that satisfies the comparison against 100 (checked with the oracle)
+    preset = {"EQ": 100, "NE": 7, "GT": 101, "LE": 100, "LT": 3, "GE": 2**63}[cmp_name]
+    assert L.oracle_compare_u64(preset, N.CMP[cmp_name], 100)
+    for pe in range(NPES):
+        rt.upload(sig, pe, np.array([preset + (0 if cmp_name == "EQ" else pe)], np.uint64))
+    note("signal_wait_until cmp=%s" % cmp_name)
+    assert perf.nvshmem_perftest_signal_wait(sig, N.CMP[cmp_name], 100, out, None) == 0
+    rt.sync()
+    got = _words(rt, out)[:, 0]
+    for pe in range(NPES):
+        assert got[pe] == preset + (0 if cmp_name == "EQ" else pe)
+        assert rt.read_timeout(pe)[0] == 0
+    rt.free(sig); rt.free(out)
+
+
+def test_bounded_wait_gives_up_and_records_the_timeout(rt):
+    # nobody ever signals: with a tiny poll limit the kernel must still finish, and the record says
+    # which word was waited on, what was found and what was expected
+    perf = rt.perftest()
+    sig = rt.calloc(8, 8); out = rt.calloc(8, 8)
+    rt.lib.nvshmemx_amd_set_spin_limit(200)
+    try:
+        note("bounded wait: spin limit 200, condition never true")
+        assert perf.nvshmem_perftest_signal_wait(sig, N.CMP["GE"], 5, out, None) == 0
+        rt.sync()
+        for pe in range(NPES):
+            flag, rec = rt.read_timeout(pe)
+            assert flag == 1
+            assert rec[1] == rt.ptr(sig, pe) and rec[2] == 0 and rec[3] == 5
+            assert rt.read_timeout(pe)[0] == 0         # reading clears the record
+    finally:
+        rt.lib.nvshmemx_amd_set_spin_limit(1 << 24)
+    rt.free(sig); rt.free(out)
+
+
+def test_scalar_p_and_g(rt):
+    perf = rt.perftest()
+    words = rt.calloc(NPES, 8); out = rt.calloc(NPES, 8)
+    note("uint64 p/g")
+    assert perf.nvshmem_perftest_p_g(words, out, 1000, None) == 0
+    rt.sync()
+    w = rt.download_all(words, (NPES,), np.uint64)
+    o = rt.download_all(out, (NPES,), np.uint64)
+    for q in range(NPES):
+        writer = (q - 1) % NPES
+        assert w[q, writer] == 1000 + writer and w[q].sum() == 1000 + writer
+        assert (o[:, q] == 1000 + writer).all()      # every PE read PE q's word with g
+    rt.free(words); rt.free(out)
+
+
+@pytest.mark.parametrize("scope,threads", [(N.SCOPE_THREAD, 1), (N.SCOPE_WARP, 64), (N.SCOPE_BLOCK, 256)])
+def test_device_barrier_holds_every_pe(rt, scope, threads):
+    perf = rt.perftest()
+    counter = rt.calloc(1, 8); errors = rt.calloc(1, 8)
+    note("barrier_all x200 scope=%d" % scope)
+    assert perf.nvshmem_perftest_device_barrier(counter, errors, 200, scope, threads, None) == 0
+    rt.sync()
+    assert (_words(rt, errors)[:, 0] == 0).all()
+    assert (_words(rt, counter)[:, 0] == 200).all()
+    assert all(rt.read_timeout(pe)[0] == 0 for pe in range(NPES))
+    rt.free(counter); rt.free(errors)
+
+
+def test_put_signal_pingpong(rt):
+    perf = rt.perftest()
+    for nbytes in (8, 1000, 65536):
+        data = rt.malloc(nbytes); sig = rt.calloc(1, 8)
+        payload = O.fill_all("bytes", NPES, nbytes, 30)
+        rt.upload_all(data, payload)
+        note("put_signal ping-pong bytes=%d" % nbytes)
+        assert perf.nvshmem_perftest_put_signal_pingpong(data, sig, nbytes, 50, 256, None) == 0
+        rt.sync()
+        got = rt.download_all(data, (nbytes,), np.uint8)
+        assert np.array_equal(got[0], payload[0]) and np.array_equal(got[1], payload[0])
+        assert np.array_equal(got[2:], payload[2:])          # bystanders untouched
+        s = _words(rt, sig)[:, 0]
+        assert s[0] == 50 and s[1] == 50 and (s[2:] == 0).all()
+        assert all(rt.read_timeout(pe)[0] == 0 for pe in range(NPES))
+        rt.free(data); rt.free(sig)
+
+
+def test_ring_allreduce_from_put_signal_known_answer_and_oracle(rt):
+    perf = rt.perftest()
+    blocks, chunk, chunks = 4, 1024, 3
+    n = blocks * chunk * chunks
+    dst = rt.calloc(n, 4); src = rt.malloc(n * 4); sig = rt.calloc(blocks, 8)
+    # known answer of examples/ring-reduce.cu:209,242-248: src[i] = i on every PE -> dst[i] = i*npes
+    rt.upload_all(src, np.tile(np.arange(n, dtype=np.int32), (NPES, 1)))
+    note("ring_reduce known answer")
+    assert perf.nvshmem_perftest_ring_reduce(dst, src, n, sig, chunk, blocks, 256, None) == 0
+    rt.sync()
+    got = rt.download_all(dst, (n,), np.int32)
+    assert (got == np.arange(n, dtype=np.int32) * NPES).all()
+    assert (_words(rt, sig, blocks) == 0).all()               # signals reset for the next run
+    # seeded data against the oracle (integer sum: any order gives the same bits)
+    data = O.fill_all("i32", NPES, n, 1)
+    rt.upload_all(src, data)
+    rt.fill(dst, 0, n * 4)
+    note("ring_reduce seeded")
+    assert perf.nvshmem_perftest_ring_reduce(dst, src, n, sig, chunk, blocks, 256, None) == 0
+    rt.sync()
+    got = rt.download_all(dst, (n,), np.int32)
+    assert (got == O.reduce("i32", "sum", data)).all()
+    assert all(rt.read_timeout(pe)[0] == 0 for pe in range(NPES))
+    assert perf.nvshmem_perftest_ring_reduce(dst, src, n + 1, sig, chunk, blocks, 256, None) != 0
+    rt.free(dst); rt.free(src); rt.free(sig)
+
+
+def test_collective_launch_refuses_grids_that_cannot_be_co_resident(rt):
+    perf = rt.perftest()
+    dst = rt.calloc(1 << 20, 4); src = rt.calloc(1 << 20, 4); sig = rt.calloc(65535, 8)
+    rc = perf.nvshmem_perftest_ring_reduce(dst, src, 65535 * 16, sig, 16, 65535, 1024, None)
+    assert rc == 6      # NVSHMEMX_ERROR_COLLECTIVE_LAUNCH_FAILED
+    assert b"co-resident" in rt.lib.nvshmemx_amd_last_error()
+    rt.free(dst); rt.free(src); rt.free(sig)
