@@ -181,10 +181,10 @@ NVSHMEMI_HOST_ONLY int nvshmemx_amd_collective_launch_query_gridsize(const void 
 typedef int (*nvshmemi_amd_state_updater_t)(const struct nvshmemi_device_state *host_copy);
 NVSHMEMI_HOST_ONLY void nvshmemi_amd_register_state_updater(nvshmemi_amd_state_updater_t fn);
 NVSHMEMI_HOST_ONLY void nvshmemi_amd_unregister_state_updater(nvshmemi_amd_state_updater_t fn);
-/* Pushes the current state to every registered unit now.  Library entry points do this on their own;
- * a program that loads a code object after nvshmem_init and starts its kernels with a plain launch
- * calls it first (the reference's nvshmemx_cumodule_init plays this role,
- * src/include/host/nvshmemx_api.h:86-90). */
+/* Pushes the current state to the units that registered since the last push (cheap when there are
+ * none).  Library entry points do this on their own; code that loads a code object after
+ * nvshmem_init and starts its kernels with a plain launch calls it before the first launch (the
+ * reference's nvshmemx_cumodule_init plays this role, src/include/host/nvshmemx_api.h:74). */
 NVSHMEMI_HOST_ONLY int nvshmemx_amd_module_init(void);
 
 /* Bounded device waits (counterpart of the reference's NVSHMEM_TIMEOUT_DEVICE_POLLING build,

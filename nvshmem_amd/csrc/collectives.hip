@@ -292,8 +292,11 @@ int reduce_on_stream(int dtype, int op, nvshmem_team_t team, void *dest, const v
     if (nreduce == 0) return 0;
     const size_t es = kDtypeSize[dtype];
     uint64_t doff = 0, soff = 0;
-    if (nreduce > rt.heap_size / es ||
-        !check_symmetric_range(rt, "reduce dest", dest, nreduce * es, &doff) ||
+    if (nreduce > rt.heap_size / es) {
+        set_error("reduce: %zu elements of %zu bytes leave the PE's heap slice", nreduce, es);
+        return NVSHMEMX_ERROR_INVALID_VALUE;
+    }
+    if (!check_symmetric_range(rt, "reduce dest", dest, nreduce * es, &doff) ||
         !check_symmetric_range(rt, "reduce source", src, nreduce * es, &soff))
         return NVSHMEMX_ERROR_INVALID_VALUE;
     if ((doff % es) || (soff % es)) {

@@ -10,8 +10,11 @@
 
 namespace perftest {
 
+// Also makes sure this library's device state blocks are populated: it may have been loaded after
+// nvshmem_init, and its kernels are started with plain launches.
 inline bool ready() {
-    if (nvshmemx_init_status() == NVSHMEM_STATUS_IS_INITIALIZED) return true;
+    if (nvshmemx_init_status() == NVSHMEM_STATUS_IS_INITIALIZED)
+        return nvshmemx_amd_module_init() == NVSHMEMX_SUCCESS;
     fprintf(stderr, "nvshmem_perftest: nvshmem is not initialised\n");
     return false;
 }

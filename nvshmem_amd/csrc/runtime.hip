@@ -116,7 +116,7 @@ int nvshmemx_amd_module_init(void) {
     Runtime &rt = Runtime::get();
     std::lock_guard<std::recursive_mutex> lock(rt.mu);
     if (!rt.initialized) return NVSHMEMX_ERROR_INVALID_VALUE;
-    refresh_symbols(rt, true);
+    refresh_symbols(rt, false);  // a no-op unless a unit registered since the last push
     return NVSHMEMX_SUCCESS;
 }
 
@@ -190,7 +190,7 @@ int nvshmemx_amd_init(int npes, size_t symmetric_size) {
     rt.dev.sync_flags = (uint64_t *)(uintptr_t)flags;
     rt.dev.sync_epoch = (uint64_t *)(uintptr_t)epoch;
     rt.dev.timeout_record = (uint64_t *)(uintptr_t)trec;
-    rt.dev.spin_limit = env_size("NVSHMEM_AMD_SPIN_LIMIT", 1ull << 24);
+    rt.dev.spin_limit = env_size("NVSHMEM_AMD_SPIN_LIMIT", 1ull << 22);
     NVSHMEM_AMD_HIP_CHECK(hipDeviceSynchronize());
     refresh_symbols(rt, true);
     return NVSHMEMX_SUCCESS;
@@ -299,6 +299,7 @@ void *nvshmem_calloc(size_t count, size_t size) {
     Runtime &rt = Runtime::get();
     std::lock_guard<std::recursive_mutex> lock(rt.mu);
     if (!require_init(rt, "nvshmem_calloc") || size == 0 || count == 0) return nullptr;
+    refresh_symbols(rt, false);
     if (count > SIZE_MAX / size) return heap_fail(rt, "nvshmem_calloc", SIZE_MAX);
     const size_t bytes = count * size;
     const uint64_t a = rt.space->allocate(bytes);
@@ -314,6 +315,7 @@ void *nvshmem_align(size_t alignment, size_t size) {
     Runtime &rt = Runtime::get();
     std::lock_guard<std::recursive_mutex> lock(rt.mu);
     if (!require_init(rt, "nvshmem_align") || size == 0) return nullptr;
+    refresh_symbols(rt, false);
     if (alignment == 0 || (alignment & (alignment - 1)) || alignment % sizeof(void *)) {
         set_error("nvshmem_align: alignment %zu is not a power of two multiple of %zu", alignment,
                   sizeof(void *));

@@ -76,7 +76,7 @@ def test_signal_wait_until_returns_the_satisfying_value(rt, cmp_name):
     L = O.lib()
     sig = rt.calloc(8, 8); out = rt.calloc(8, 8)
     # a preset value per PE that satisfies the comparison against 100 (checked with the oracle)
-    preset = {"EQ": 100, "NE": 7, "GT": 101, "LE": 100, "LT": 3, "GE": 2**63}[cmp_name]
+    preset = {"EQ": 100, "NE": 7, "GT": 101, "LE": 93, "LT": 3, "GE": 2**63}[cmp_name]
     assert L.oracle_compare_u64(preset, N.CMP[cmp_name], 100)
     for pe in range(NPES):
         rt.upload(sig, pe, np.array([preset + (0 if cmp_name == "EQ" else pe)], np.uint64))
@@ -106,7 +106,7 @@ def test_bounded_wait_gives_up_and_records_the_timeout(rt):
             assert rec[1] == rt.ptr(sig, pe) and rec[2] == 0 and rec[3] == 5
             assert rt.read_timeout(pe)[0] == 0         # reading clears the record
     finally:
-        rt.lib.nvshmemx_amd_set_spin_limit(1 << 24)
+        rt.lib.nvshmemx_amd_set_spin_limit(1 << 22)
     rt.free(sig); rt.free(out)
 
 
