@@ -139,11 +139,26 @@ typedef nvshmemi_v4u __attribute__((aligned(1))) nvshmemi_v4u_unaligned;
 #ifndef NVSHMEMI_AMD_COPY_UNROLL
 #define NVSHMEMI_AMD_COPY_UNROLL 4
 #endif
+/* bit 0: non-temporal loads, bit 1: non-temporal stores in the vector body */
+#ifndef NVSHMEMI_AMD_COPY_NT
+#define NVSHMEMI_AMD_COPY_NT 3
+#endif
 
 template <bool SRC_ALIGNED>
 NVSHMEMI_DEVICE_INLINE nvshmemi_v4u nvshmemi_amd_load16(const char *p) {
     if (SRC_ALIGNED) return *reinterpret_cast<const nvshmemi_v4u *>(p);
     return *reinterpret_cast<const nvshmemi_v4u_unaligned *>(p);
+}
+
+template <bool SRC_ALIGNED>
+NVSHMEMI_DEVICE_INLINE nvshmemi_v4u nvshmemi_amd_stream_load16(const char *p) {
+    if ((NVSHMEMI_AMD_COPY_NT & 1) && SRC_ALIGNED)
+        return __builtin_nontemporal_load(reinterpret_cast<const nvshmemi_v4u *>(p));
+    return nvshmemi_amd_load16<SRC_ALIGNED>(p);
+}
+NVSHMEMI_DEVICE_INLINE void nvshmemi_amd_stream_store16(char *p, nvshmemi_v4u v) {
+    if (NVSHMEMI_AMD_COPY_NT & 2) __builtin_nontemporal_store(v, reinterpret_cast<nvshmemi_v4u *>(p));
+    else *reinterpret_cast<nvshmemi_v4u *>(p) = v;
 }
 
 template <bool SRC_ALIGNED>
@@ -155,12 +170,12 @@ NVSHMEMI_DEVICE_INLINE void nvshmemi_amd_copy_vectors(char *__restrict__ dst,
     for (; i + (U - 1) * nthr < nvec; i += U * nthr) {
         nvshmemi_v4u v[U];
 #pragma unroll
-        for (int u = 0; u < U; ++u) v[u] = nvshmemi_amd_load16<SRC_ALIGNED>(src + 16 * (i + u * nthr));
+        for (int u = 0; u < U; ++u) v[u] = nvshmemi_amd_stream_load16<SRC_ALIGNED>(src + 16 * (i + u * nthr));
 #pragma unroll
-        for (int u = 0; u < U; ++u) *reinterpret_cast<nvshmemi_v4u *>(dst + 16 * (i + u * nthr)) = v[u];
+        for (int u = 0; u < U; ++u) nvshmemi_amd_stream_store16(dst + 16 * (i + u * nthr), v[u]);
     }
     for (; i < nvec; i += nthr)
-        *reinterpret_cast<nvshmemi_v4u *>(dst + 16 * i) = nvshmemi_amd_load16<SRC_ALIGNED>(src + 16 * i);
+        nvshmemi_amd_stream_store16(dst + 16 * i, nvshmemi_amd_stream_load16<SRC_ALIGNED>(src + 16 * i));
 }
 
 template <int SCOPE>
@@ -180,10 +195,19 @@ NVSHMEMI_DEVICE_INLINE void nvshmemi_memcpy_threadgroup(void *__restrict__ dst_v
 
     const size_t nvec = len / 16;
     if (nvec) {
+        /* Long copies: the first lanes move the vectors in front of the next 1 KiB boundary of dst, so
+         * that every wavefront access of the body is one aligned 1 KiB piece (HBM serves those
+         * measurably faster than pieces that straddle the boundary). */
+        size_t pre = 0;
+        if (nvec >= 256) {
+            pre = (size_t)((-(uintptr_t)dst >> 4) & 63);
+            if (((uintptr_t)src & 15) == 0) nvshmemi_amd_copy_vectors<true>(dst, src, pre, tid, nthr);
+            else nvshmemi_amd_copy_vectors<false>(dst, src, pre, tid, nthr);
+        }
         if (((uintptr_t)src & 15) == 0)
-            nvshmemi_amd_copy_vectors<true>(dst, src, nvec, tid, nthr);
+            nvshmemi_amd_copy_vectors<true>(dst + 16 * pre, src + 16 * pre, nvec - pre, tid, nthr);
         else
-            nvshmemi_amd_copy_vectors<false>(dst, src, nvec, tid, nthr);
+            nvshmemi_amd_copy_vectors<false>(dst + 16 * pre, src + 16 * pre, nvec - pre, tid, nthr);
     }
     const size_t done = nvec * 16;
     for (size_t i = done + tid; i < len; i += nthr) dst[i] = src[i];

@@ -4,7 +4,7 @@ import os
 import re
 
 ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
-LIBDIR = os.path.join(ROOT, "nvshmem_amd", "lib")
+LIBDIR = os.environ.get("NVSHMEM_AMD_LIBDIR") or os.path.join(ROOT, "nvshmem_amd", "lib")
 INCLUDE = os.path.join(ROOT, "include")
 
 

@@ -19,44 +19,66 @@
 namespace nvshmem_amd {
 namespace {
 
-constexpr int kThreads = 256;
+// Tunables (compile time).  Defaults are the values measured best on MI355X.
+#ifndef NVSHMEM_AMD_COLL_THREADS
+#define NVSHMEM_AMD_COLL_THREADS 256
+#endif
+#ifndef NVSHMEM_AMD_COPY_TILE_UNROLL
+#define NVSHMEM_AMD_COPY_TILE_UNROLL 2
+#endif
+#ifndef NVSHMEM_AMD_COLL_NT /* bit 0: non-temporal loads, bit 1: non-temporal stores */
+#define NVSHMEM_AMD_COLL_NT 3
+#endif
+
+constexpr int kThreads = NVSHMEM_AMD_COLL_THREADS;
+
+__device__ __forceinline__ nvshmemi_v4u stream_load(const char *p) {
+    if (NVSHMEM_AMD_COLL_NT & 1) return __builtin_nontemporal_load(reinterpret_cast<const nvshmemi_v4u *>(p));
+    return *reinterpret_cast<const nvshmemi_v4u *>(p);
+}
+__device__ __forceinline__ void stream_store(char *p, nvshmemi_v4u v) {
+    if (NVSHMEM_AMD_COLL_NT & 2) __builtin_nontemporal_store(v, reinterpret_cast<nvshmemi_v4u *>(p));
+    else *reinterpret_cast<nvshmemi_v4u *>(p) = v;
+}
 
 // ---------------------------------------------------------------------------------------------
 // Segment copy: fcollect and alltoall are sets of contiguous (source, destination) segments.
-// grid.y indexes the segment, grid.x the 32 KiB tile inside it.  The destination is written with
-// aligned 16-byte vectors only: block 0 of a segment copies the byte head in front of the first
-// aligned destination vector and the byte tail behind the last one.
+// grid.y indexes the segment, grid.x the tile inside it (kThreads x unroll 16-byte vectors).  The
+// destination is written with aligned vectors only: block 0 of a segment copies the byte head in
+// front of the first aligned destination vector and the byte tail behind the last one.  Blocks
+// are short-lived on purpose: the blocks in flight at any time then cover a narrow, moving window
+// of addresses, which HBM serves faster than many long independent streams.
 // ---------------------------------------------------------------------------------------------
-constexpr int kCopyUnroll = 8;
+constexpr int kCopyUnroll = NVSHMEM_AMD_COPY_TILE_UNROLL;
 constexpr size_t kTileVectors = (size_t)kThreads * kCopyUnroll;
 
 enum { kModeFcollect = 0, kModeAlltoall = 1 };
 
+// Copies the vectors v0 + t + u*kThreads (u < unroll) that fall inside [0, nvec); indices in front of
+// the segment wrap to huge unsigned values and are skipped the same way as those behind it.
 template <bool SRC_ALIGNED, bool REPLICATE>
 __device__ __forceinline__ void copy_tile(char *__restrict__ dst, const char *__restrict__ src,
-                                          size_t nvec, uint64_t rep_stride, int nrep) {
-    // nvec <= kTileVectors vectors, thread t takes t, t+256, ...
+                                          uint64_t v0, uint64_t nvec, uint64_t rep_stride, int nrep) {
     nvshmemi_v4u v[kCopyUnroll];
-    const size_t t = threadIdx.x;
 #pragma unroll
     for (int u = 0; u < kCopyUnroll; ++u) {
-        const size_t i = t + (size_t)u * kThreads;
-        if (i < nvec) v[u] = nvshmemi_amd_load16<SRC_ALIGNED>(src + 16 * i);
+        const uint64_t i = v0 + threadIdx.x + (uint64_t)u * kThreads;
+        if (i < nvec) v[u] = SRC_ALIGNED ? stream_load(src + 16 * i) : nvshmemi_amd_load16<false>(src + 16 * i);
     }
     if (REPLICATE) {
         for (int r = 0; r < nrep; ++r) {
             char *d = dst + (uint64_t)r * rep_stride;
 #pragma unroll
             for (int u = 0; u < kCopyUnroll; ++u) {
-                const size_t i = t + (size_t)u * kThreads;
-                if (i < nvec) *reinterpret_cast<nvshmemi_v4u *>(d + 16 * i) = v[u];
+                const uint64_t i = v0 + threadIdx.x + (uint64_t)u * kThreads;
+                if (i < nvec) stream_store(d + 16 * i, v[u]);
             }
         }
     } else {
 #pragma unroll
         for (int u = 0; u < kCopyUnroll; ++u) {
-            const size_t i = t + (size_t)u * kThreads;
-            if (i < nvec) *reinterpret_cast<nvshmemi_v4u *>(dst + 16 * i) = v[u];
+            const uint64_t i = v0 + threadIdx.x + (uint64_t)u * kThreads;
+            if (i < nvec) stream_store(dst + 16 * i, v[u]);
         }
     }
 }
@@ -97,96 +119,83 @@ __global__ __launch_bounds__(kThreads) void segment_copy_kernel(char *base, uint
             dst[r * rep_stride + pos] = src[pos];
         }
     }
-    const uint64_t first = (uint64_t)blockIdx.x * kTileVectors;
-    if (first >= nvec_total) return;
-    const uint64_t left = nvec_total - first;
-    const size_t nvec = left < kTileVectors ? (size_t)left : kTileVectors;
-    const char *s = src + head + first * 16;
-    char *d = dst + head + first * 16;
+    // tiles are cut on absolute 1 KiB boundaries of the destination: `lead` vector slots of tile 0
+    // lie in front of the segment
+    const uint64_t lead = ((uint64_t)(uintptr_t)(dst + head) >> 4) & 63;
+    const uint64_t v0 = (uint64_t)blockIdx.x * kTileVectors - lead;
+    if ((int64_t)v0 >= (int64_t)nvec_total) return;
+    const char *s = src + head;
+    char *d = dst + head;
     const bool aligned = (((uintptr_t)s) & 15) == 0;
     if (MODE == kModeFcollect) {
-        if (aligned) copy_tile<true, true>(d, s, nvec, rep_stride, nrep);
-        else copy_tile<false, true>(d, s, nvec, rep_stride, nrep);
+        if (aligned) copy_tile<true, true>(d, s, v0, nvec_total, rep_stride, nrep);
+        else copy_tile<false, true>(d, s, v0, nvec_total, rep_stride, nrep);
     } else {
-        if (aligned) copy_tile<true, false>(d, s, nvec, rep_stride, 1);
-        else copy_tile<false, false>(d, s, nvec, rep_stride, 1);
+        if (aligned) copy_tile<true, false>(d, s, v0, nvec_total, rep_stride, 1);
+        else copy_tile<false, false>(d, s, v0, nvec_total, rep_stride, 1);
     }
 }
 
 // ---------------------------------------------------------------------------------------------
-// Fused reduce.  A lane owns 16-byte vectors of the element range; for each it loads that vector
-// from every PE's source (groups of four PEs in flight, two vectors per lane), folds in PE order,
-// and stores the result into every PE's destination.  An element is read by exactly one lane
-// before that lane writes it, so dest == src (in place) needs no staging.
+// Fused reduce, LDS staged.  A block owns a tile of `lanes` 16-byte vectors of the element range
+// (lanes = 64 when the team has at most 16 PEs, so one wavefront streams 1 KiB of one PE's source).
+// Thread (pe, i) loads vector i of the tile from PE pe's source into LDS - one load per thread, like
+// a plain copy, which HBM serves measurably faster than one lane gathering the same vector from
+// every PE.  After a barrier the tile's elements are folded out of LDS in PE order 0..n-1, one
+// element per thread, and thread (pe, i) stores result vector i into PE pe's destination.
+// An element is read (by the loads of this block) before this block writes it and no other block
+// touches it, so dest == src (in place) needs no further staging.
 // ---------------------------------------------------------------------------------------------
-constexpr int kReduceUnroll = 2;
-constexpr int kPeGroup = 4;
-
-template <typename T>
-struct alignas(16) Pack {
-    static constexpr int N = 16 / sizeof(T);
-    T e[N];
-};
-
-template <typename T, int OP>
-__global__ __launch_bounds__(kThreads) void reduce_vector_kernel(char *base, uint32_t shift, int npes,
-                                                                 uint64_t dst_off, uint64_t src_off,
-                                                                 uint64_t nelems) {
-    typedef Pack<T> P;
-    const uint64_t nvec = nelems / P::N;
-    const uint64_t gsz = (uint64_t)gridDim.x * kThreads;
-    const uint64_t gid = (uint64_t)blockIdx.x * kThreads + threadIdx.x;
+// NPES > 0 fixes the team size at compile time (fold fully unrolled, one wavefront per PE);
+// NPES == 0 takes both from the arguments.
+template <typename T, int OP, int NPES>
+__global__ __launch_bounds__(NPES ? NPES * 64 : 1024) void reduce_vector_kernel(char *base, uint32_t shift, int npes_arg,
+                                                             uint32_t lane_shift_arg, uint64_t dst_off,
+                                                             uint64_t src_off, uint64_t nelems) {
+    extern __shared__ __attribute__((aligned(16))) char lds[];
+    constexpr int VEC = 16 / sizeof(T);
+    const int npes = NPES ? NPES : npes_arg;
+    const uint32_t lane_shift = NPES ? 6u : lane_shift_arg;
+    const unsigned lanes = 1u << lane_shift;
+    const unsigned pe = threadIdx.x >> lane_shift, i = threadIdx.x & (lanes - 1);
+    const uint64_t nvec = nelems / VEC;
+    // tiles are cut on absolute (16 * lanes)-byte boundaries of the destination, so a wavefront's
+    // access is one aligned 1 KiB piece whatever the buffer's own alignment: `lead` vector slots of
+    // the first tile lie in front of the buffer
+    const uint64_t lead = ((uint64_t)(uintptr_t)(base + dst_off) >> 4) & (lanes - 1);
+    const uint64_t ntiles = (nvec + lead + lanes - 1) >> lane_shift;
     const uint64_t pe_stride = 1ull << shift;
-    const char *src0 = base + src_off;
-    char *dst0 = base + dst_off;
+    nvshmemi_v4u *stage = reinterpret_cast<nvshmemi_v4u *>(lds);           // [npes][lanes]
+    nvshmemi_v4u *result = stage + ((size_t)npes << lane_shift);           // [lanes]
+    const T *stage_e = reinterpret_cast<const T *>(stage);
+    T *result_e = reinterpret_cast<T *>(result);
+    const unsigned tile_elems = lanes * VEC;
 
-    for (uint64_t v0 = gid; v0 < nvec; v0 += gsz * kReduceUnroll) {
-        P acc[kReduceUnroll];
-        for (int g = 0; g < npes; g += kPeGroup) {
-            P x[kPeGroup][kReduceUnroll];
+    for (uint64_t tile = blockIdx.x; tile < ntiles; tile += gridDim.x) {
+        const uint64_t v = (tile << lane_shift) + i - lead;  // wraps to a huge value in front of the buffer
+        if (v < nvec) stage[threadIdx.x] = stream_load(base + (uint64_t)pe * pe_stride + src_off + 16 * v);
+        __syncthreads();
+        for (unsigned e = threadIdx.x; e < tile_elems; e += blockDim.x) {
+            T acc = stage_e[e];
 #pragma unroll
-            for (int j = 0; j < kPeGroup; ++j) {
-#pragma unroll
-                for (int u = 0; u < kReduceUnroll; ++u) {
-                    const uint64_t v = v0 + (uint64_t)u * gsz;
-                    if (g + j < npes && v < nvec)
-                        x[j][u] = *reinterpret_cast<const P *>(src0 + (uint64_t)(g + j) * pe_stride + 16 * v);
-                }
-            }
-#pragma unroll
-            for (int j = 0; j < kPeGroup; ++j) {
-                const int pe = g + j;
-                if (pe >= npes) break;
-#pragma unroll
-                for (int u = 0; u < kReduceUnroll; ++u) {
-                    if (pe == 0) {
-                        acc[u] = x[j][u];
-                    } else {
-#pragma unroll
-                        for (int k = 0; k < P::N; ++k)
-                            acc[u].e[k] = nvshmemi_amd_fold_step<T, OP>(pe, acc[u].e[k], x[j][u].e[k]);
-                    }
-                }
-            }
+            for (int p = 1; p < npes; ++p)
+                acc = nvshmemi_amd_fold_step<T, OP>(p, acc, stage_e[(size_t)p * tile_elems + e]);
+            result_e[e] = acc;
         }
-        for (int pe = 0; pe < npes; ++pe) {
-#pragma unroll
-            for (int u = 0; u < kReduceUnroll; ++u) {
-                const uint64_t v = v0 + (uint64_t)u * gsz;
-                if (v < nvec) *reinterpret_cast<P *>(dst0 + (uint64_t)pe * pe_stride + 16 * v) = acc[u];
-            }
-        }
+        __syncthreads();
+        if (v < nvec) stream_store(base + (uint64_t)pe * pe_stride + dst_off + 16 * v, result[i]);
     }
     // elements behind the last full vector
-    const uint64_t done = nvec * P::N;
+    const uint64_t done = nvec * VEC;
+    const uint64_t gid = (uint64_t)blockIdx.x * blockDim.x + threadIdx.x;
     if (gid < nelems - done) {
-        const uint64_t i = done + gid;
-        const T *s = reinterpret_cast<const T *>(src0);
-        T *d = reinterpret_cast<T *>(dst0);
+        const uint64_t k = done + gid;
+        const T *s = reinterpret_cast<const T *>(base + src_off);
+        T *d = reinterpret_cast<T *>(base + dst_off);
         const uint64_t es = pe_stride / sizeof(T);
-        T acc = s[i];
-        for (int pe = 1; pe < npes; ++pe) acc = nvshmemi_amd_fold_step<T, OP>(pe, acc, s[(uint64_t)pe * es + i]);
-        for (int pe = 0; pe < npes; ++pe) d[(uint64_t)pe * es + i] = acc;
+        T acc = s[k];
+        for (int p = 1; p < npes; ++p) acc = nvshmemi_amd_fold_step<T, OP>(p, acc, s[(uint64_t)p * es + k]);
+        for (int p = 0; p < npes; ++p) d[(uint64_t)p * es + k] = acc;
     }
 }
 
@@ -210,18 +219,33 @@ template <typename T, int OP>
 void launch_reduce(Runtime &rt, uint64_t dst_off, uint64_t src_off, uint64_t nelems,
                    hipStream_t stream) {
     const bool vector_ok = ((dst_off | src_off) & 15) == 0;
-    const uint64_t per_thread = vector_ok ? (uint64_t)(16 / sizeof(T)) * kReduceUnroll : 1;
-    uint64_t blocks = (nelems + per_thread * kThreads - 1) / (per_thread * kThreads);
-    // enough resident work to cover HBM latency; more blocks than this only add launch cost
-    const uint64_t cap = (uint64_t)rt.num_cus * 32;
-    if (blocks > cap) blocks = cap;
-    if (blocks == 0) blocks = 1;
-    if (vector_ok)
-        hipLaunchKernelGGL((reduce_vector_kernel<T, OP>), dim3((unsigned)blocks), dim3(kThreads), 0,
-                           stream, rt.base, rt.heap_shift, rt.npes, dst_off, src_off, nelems);
-    else
+    if (vector_ok) {
+        // lanes per PE: a full wavefront when the block still fits 1024 threads
+        uint32_t lane_shift = 6;
+        while (((uint32_t)rt.npes << lane_shift) > 1024) --lane_shift;  // npes <= 64 -> >= 16 lanes
+        const unsigned threads = (unsigned)rt.npes << lane_shift;
+        const uint64_t nvec = nelems / (16 / sizeof(T));
+        uint64_t blocks = (nvec + (2u << lane_shift) - 1) >> lane_shift;  // +1 tile for the lead-in
+        if (blocks > 0x7fffffffull) blocks = 0x7fffffffull;  // the tile loop covers the rest
+        if (blocks == 0) blocks = 1;                          // only tail elements
+        const size_t lds = ((size_t)rt.npes + 1) * 16 << lane_shift;
+#define NVSHMEM_AMD_LAUNCH_REDUCE(N)                                                              \
+    hipLaunchKernelGGL((reduce_vector_kernel<T, OP, N>), dim3((unsigned)blocks), dim3(threads),   \
+                       lds, stream, rt.base, rt.heap_shift, rt.npes, lane_shift, dst_off,         \
+                       src_off, nelems)
+        switch (rt.npes) {
+            case 8: NVSHMEM_AMD_LAUNCH_REDUCE(8); break;
+            case 16: NVSHMEM_AMD_LAUNCH_REDUCE(16); break;
+            default: NVSHMEM_AMD_LAUNCH_REDUCE(0); break;
+        }
+#undef NVSHMEM_AMD_LAUNCH_REDUCE
+    } else {
+        uint64_t blocks = (nelems + kThreads - 1) / kThreads;
+        const uint64_t cap = (uint64_t)rt.num_cus * 64;
+        if (blocks > cap) blocks = cap;
         hipLaunchKernelGGL((reduce_scalar_kernel<T, OP>), dim3((unsigned)blocks), dim3(kThreads), 0,
                            stream, rt.base, rt.heap_shift, rt.npes, dst_off, src_off, nelems);
+    }
 }
 
 typedef void (*reduce_launcher_t)(Runtime &, uint64_t, uint64_t, uint64_t, hipStream_t);
@@ -335,7 +359,7 @@ static int segment_collective(int mode, const char *what, nvshmem_team_t team, v
         set_error("%s: dest and source overlap", what);
         return NVSHMEMX_ERROR_INVALID_VALUE;
     }
-    const uint64_t tiles = (seg_bytes / 16 + kTileVectors - 1) / kTileVectors + 1;
+    const uint64_t tiles = (seg_bytes / 16 + 64 + kTileVectors - 1) / kTileVectors + 1;
     const unsigned segs = mode == kModeFcollect ? (unsigned)n : (unsigned)(n * n);
     if (tiles > 0x7fffffffull) {
         set_error("%s: message too large", what);

@@ -169,16 +169,18 @@ int nvshmemx_amd_init(int npes, size_t symmetric_size) {
     rt.heap_shift = shift;
     rt.heap_size = 1ull << shift;
     rt.base = (char *)mem;
-    rt.space.reset(new SymmetricSpace((uint64_t)(uintptr_t)rt.base, rt.heap_size));
+    // The runtime's own symmetric words (barrier row, epoch, timeout record) live in the last
+    // granules of every slice, outside the allocator's space, so that user allocations start at the
+    // slice base: large buffers then sit on the 1 KiB boundaries the streaming kernels like.
+    const uint64_t internal_bytes = 4 * NVSHMEMI_MALLOC_ALIGNMENT;
+    rt.space.reset(new SymmetricSpace((uint64_t)(uintptr_t)rt.base, rt.heap_size - internal_bytes));
     rt.initialized = true;
-
-    // The runtime's own symmetric objects come first in every slice.
-    const uint64_t flags = rt.space->allocate(NVSHMEMI_AMD_MAX_PES * sizeof(uint64_t));
-    const uint64_t epoch = rt.space->allocate(sizeof(uint64_t));
-    const uint64_t trec = rt.space->allocate(4 * sizeof(uint64_t));
-    const uint64_t internal_end = trec + NVSHMEMI_MALLOC_ALIGNMENT - (uint64_t)(uintptr_t)rt.base;
+    const uint64_t internal = (uint64_t)(uintptr_t)rt.base + rt.heap_size - internal_bytes;
+    const uint64_t flags = internal;
+    const uint64_t epoch = internal + NVSHMEMI_AMD_MAX_PES * sizeof(uint64_t);
+    const uint64_t trec = epoch + NVSHMEMI_MALLOC_ALIGNMENT;
     for (int pe = 0; pe < npes; ++pe)
-        NVSHMEM_AMD_HIP_CHECK(hipMemset(rt.slice(pe), 0, internal_end));
+        NVSHMEM_AMD_HIP_CHECK(hipMemset(rt.slice(pe) + rt.heap_size - internal_bytes, 0, internal_bytes));
 
     memset(&rt.dev, 0, sizeof rt.dev);
     rt.dev.version = (1u << 16) + (uint32_t)sizeof(nvshmemi_device_state_t);
