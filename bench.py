@@ -1,0 +1,268 @@
+#!/usr/bin/env python3
+"""Benchmark of the NVSHMEM data-movement hot path on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W]
+
+Prints ONE JSON line.  The headline workload is put_block at the largest size of the put/get
+sweep: every one of 8 logical PEs moves 256 MiB to its right neighbour with
+nvshmemx_putmem_block; a "step" is one such exchange (one kernel launch carrying all PEs).
+`value` is algorithmic bytes (payload read once + written once, all PEs) per second, inputs
+already resident in HBM.  sum_reduce (fp32, 8 PEs x 2^26 elements) and alltoall (fp32, 16 PEs x 2^22
+elements) are measured the same way and reported under "workloads".  The CPU oracle is timed on
+a bounded sample of each workload on this host's cores as a reported baseline.
+"""
+import argparse
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+sys.path.insert(0, os.path.join(ROOT, "tests"))
+
+HBM_PEAK_GBS = 8000.0   # MI355X published HBM3E peak
+METRIC = "achieved GB/s and % of HBM peak: put_block, sum_reduce, alltoall (1 GPU)"
+
+# HBM bytes per launch measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE (scaled by the plain
+# copy calibration kernel; summaries under profiles/): read + write, equal to the algorithmic bytes.
+MEASURED_TRAFFIC_BYTES = {
+    "put_block": (2048 + 2048) << 20,    # profiles/ring_rma_kernel_put_block_8pe_256MiB.txt
+    "sum_reduce": (2048 + 2048) << 20,   # profiles/reduce_vector_kernel_float_sum_8pe_64Mi.txt
+    "alltoall": (256 + 256) << 20,       # profiles/segment_copy_kernel_alltoall_16pe_4Mi_fp32.txt
+}
+
+# put_block launch shape: each block moves a contiguous 16 KiB slice (short-lived blocks keep the
+# set of addresses in flight narrow, which is what HBM serves fastest)
+PUT_BYTES = 1 << 28
+PUT_BLOCKS_PER_PE = 16384
+PUT_THREADS = 512
+
+
+def _time_steps(fn, steps, warmup, hip):
+    """(wall ms per step, event ms per step): K launches bracketed by device synchronisation."""
+    for _ in range(warmup):
+        fn()
+    hip.synchronize()
+    e0, e1 = hip.Event(), hip.Event()
+    t0 = time.perf_counter()
+    e0.record()
+    for _ in range(steps):
+        fn()
+    e1.record()
+    hip.synchronize()
+    wall = (time.perf_counter() - t0) * 1e3 / steps
+    ev = e0.elapsed_ms(e1) / steps
+    e0.destroy(); e1.destroy()
+    return wall, ev
+
+
+def _cpu_time(fn, budget_s, max_passes):
+    """Best wall time of fn over passes that fit the budget."""
+    best, spent, passes = None, 0.0, 0
+    while passes < max_passes and (spent < budget_s or passes == 0):
+        t0 = time.perf_counter()
+        fn()
+        dt = time.perf_counter() - t0
+        best = dt if best is None else min(best, dt)
+        spent += dt
+        passes += 1
+    return best, passes
+
+
+def bench_put_block(N, O, hip, np, steps, warmup, cpu_budget):
+    npes, S = 8, PUT_BYTES
+    with _runtime(N, npes, 2 * S + (64 << 20)) as rt:
+        perf = rt.perftest()
+        src = rt.malloc(S); dst = rt.malloc(S)
+        data = O.fill_all("bytes", npes, S, 2)
+        rt.upload_all(src, data)
+        rt.fill(dst, 0, S)
+
+        def step():
+            rc = perf.nvshmem_perftest_ring_rma(dst, src, S, PUT_BLOCKS_PER_PE, PUT_THREADS,
+                                                N.SCOPE_BLOCK, 0, 1, None)
+            if rc != 0:
+                raise RuntimeError("ring_rma failed: %d" % rc)
+        wall, ev = _time_steps(step, steps, warmup, hip)
+        # parity spot check on the timed output: PE 3 must hold PE 2's payload
+        got = rt.download(dst, 3, (S,), np.uint8)
+        ok = bool(np.array_equal(got, data[2]))
+        rt.free(src); rt.free(dst)
+    alg = 2 * npes * S
+    # CPU oracle: the same exchange with memcpy, single thread, on a 64 MiB-per-PE sample
+    sample = 1 << 26
+    host_src = data[:, :sample].copy()
+    best, passes = _cpu_time(lambda: O.ring_put(host_src), cpu_budget, 40)
+    cpu = {"value": round(2 * npes * sample / best / 1e9, 2), "unit": "GB/s", "cores": 1,
+           "kind": "port", "sample": "oracle_ring_put, 8 PEs x 64 MiB, best of %d passes" % passes}
+    return {
+        "name": "put_block", "dtype": "u8", "verified": ok, "algorithmic_bytes": alg,
+        "wall_ms": wall, "kernel_ms": ev,
+        "config": {"workload": "put_block: nvshmemx_putmem_block ring, 8 logical PEs x 256 MiB "
+                               "(largest size of the put/get sweep)",
+                   "npes": npes, "bytes_per_pe": S, "blocks_per_pe": PUT_BLOCKS_PER_PE,
+                   "threads_per_block": PUT_THREADS,
+                   "payload_only_GBs": round(npes * S / ev / 1e6, 1)},
+        "kernel": "ring_rma_kernel<BLOCK, put> (nvshmemi_memcpy_threadgroup)",
+        "cpu_baseline": cpu,
+    }
+
+
+def bench_sum_reduce(N, O, hip, np, steps, warmup, cpu_budget):
+    npes, n = 8, 1 << 26
+    with _runtime(N, npes, 2 * n * 4 + (64 << 20)) as rt:
+        src = rt.malloc(n * 4); dst = rt.malloc(n * 4)
+        data = O.fill_all("f32", npes, n, 3)
+        rt.upload_all(src, data)
+        from nvshmem_amd import _lib
+        fn = _lib.typed_coll(rt.lib, "nvshmemx_float_sum_reduce_on_stream", True)
+
+        def step():
+            rc = fn(N.TEAM_WORLD, dst, src, n, None)
+            if rc != 0:
+                raise RuntimeError("reduce failed: %d %s" % (rc, rt.last_error()))
+        wall, ev = _time_steps(step, steps, warmup, hip)
+        sample = 1 << 22
+        want = O.reduce("f32", "sum", data[:, :sample])
+        got = rt.download(dst, 5, (sample,), np.float32)
+        ok = bool(np.array_equal(got.view(np.uint32), want.view(np.uint32)))
+        rt.free(src); rt.free(dst)
+    alg = 2 * npes * n * 4
+    cores = min(16, O.lib().oracle_get_threads())
+    O.lib().oracle_set_threads(cores)
+    cs = 1 << 24
+    host = np.ascontiguousarray(data[:, :cs])
+    best, passes = _cpu_time(lambda: O.reduce("f32", "sum", host), cpu_budget, 40)
+    # the CPU oracle produces one PE's result; the algorithmic formula counts npes destinations, so
+    # the CPU figure is quoted on what it actually moves: npes reads + 1 write per element
+    cpu = {"value": round((npes + 1) * cs * 4 / best / 1e9, 2), "unit": "GB/s", "cores": cores,
+           "kind": "port",
+           "sample": "oracle_reduce f32 sum, 8 PEs x 2^24 elements (8 reads + 1 write per element), "
+                     "best of %d passes" % passes}
+    return {
+        "name": "sum_reduce", "dtype": "f32", "verified": ok, "algorithmic_bytes": alg,
+        "wall_ms": wall, "kernel_ms": ev,
+        "config": {"workload": "sum_reduce: nvshmemx_float_sum_reduce_on_stream, 8 logical PEs x 2^26 "
+                               "fp32 (256 MiB per PE), fixed PE order", "npes": npes, "nreduce": n},
+        "kernel": "reduce_vector_kernel<float, sum, 8>",
+        "cpu_baseline": cpu,
+    }
+
+
+def bench_alltoall(N, O, hip, np, steps, warmup, cpu_budget):
+    npes, n = 16, 1 << 22
+    with _runtime(N, npes, 2 * n * 4 + (16 << 20)) as rt:
+        src = rt.malloc(n * 4); dst = rt.malloc(n * 4)
+        data = O.fill_all("u64", npes, n // 2, 6).view(np.uint8).reshape(npes, -1)
+        rt.upload_all(src, data)
+        from nvshmem_amd import _lib
+        fn = _lib.typed_coll(rt.lib, "nvshmemx_float_alltoall_on_stream", True)
+
+        def step():
+            rc = fn(N.TEAM_WORLD, dst, src, n // npes, None)
+            if rc != 0:
+                raise RuntimeError("alltoall failed: %d %s" % (rc, rt.last_error()))
+        wall, ev = _time_steps(step, steps, warmup, hip)
+        got = rt.download_all(dst, (n * 4,), np.uint8)
+        want = O.alltoall(data)
+        ok = bool(np.array_equal(got, want))
+        rt.free(src); rt.free(dst)
+    alg = 2 * npes * n * 4
+    cores = min(16, O.lib().oracle_get_threads())
+    O.lib().oracle_set_threads(cores)
+    best, passes = _cpu_time(lambda: O.alltoall(data), cpu_budget, 40)
+    cpu = {"value": round(alg / best / 1e9, 2), "unit": "GB/s", "cores": cores, "kind": "port",
+           "sample": "oracle_alltoall, 16 PEs x 2^22 fp32 (the full workload), best of %d passes" % passes}
+    return {
+        "name": "alltoall", "dtype": "u8", "verified": ok, "algorithmic_bytes": alg,
+        "wall_ms": wall, "kernel_ms": ev,
+        "config": {"workload": "alltoall: nvshmemx_float_alltoall_on_stream, 16 logical PEs x 2^22 fp32, "
+                               "block 2^18 elements per destination", "npes": npes, "nelems": n // npes},
+        "kernel": "segment_copy_kernel<alltoall>",
+        "cpu_baseline": cpu,
+    }
+
+
+class _runtime:
+    def __init__(self, N, npes, size):
+        self.N, self.npes, self.size = N, npes, size
+
+    def __enter__(self):
+        self.rt = self.N.Runtime(npes=self.npes, symmetric_size=self.size)
+        return self.rt
+
+    def __exit__(self, *exc):
+        self.rt.finalize()
+
+
+def _summarise(r):
+    gbs = r["algorithmic_bytes"] / r["wall_ms"] / 1e6
+    kernel_gbs = r["algorithmic_bytes"] / r["kernel_ms"] / 1e6
+    return {
+        "GBs": round(gbs, 1), "frac_of_hbm_peak": round(gbs / HBM_PEAK_GBS, 4),
+        "ms_per_step": round(r["wall_ms"], 5), "kernel_ms": round(r["kernel_ms"], 5),
+        "kernel_GBs": round(kernel_gbs, 1), "algorithmic_bytes": r["algorithmic_bytes"],
+        "traffic": MEASURED_TRAFFIC_BYTES[r["name"]],
+        "dtype": r["dtype"], "verified": r["verified"], "config": r["config"], "kernel": r["kernel"],
+        "cpu_baseline": r["cpu_baseline"],
+    }
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=50)
+    ap.add_argument("--warmup", type=int, default=10)
+    ap.add_argument("--cpu-seconds", type=float, default=6.0,
+                    help="CPU oracle timing budget per workload")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        print("bench.py: this build runs all logical PEs on ONE GPU; --gpus %d is not supported "
+              "(no inter-GPU path exists)" % args.gpus, file=sys.stderr)
+        return 2
+
+    import numpy as np
+    import nvshmem_amd as N          # raises if the HIP libraries are not built
+    from nvshmem_amd import hip
+    import oracle_lib as O           # the checker / CPU baseline only
+
+    if hip.device_count() < 1:
+        print("bench.py: no GPU visible", file=sys.stderr)
+        return 3
+
+    put = bench_put_block(N, O, hip, np, args.steps, args.warmup, args.cpu_seconds)
+    red = bench_sum_reduce(N, O, hip, np, args.steps, args.warmup, args.cpu_seconds)
+    a2a = bench_alltoall(N, O, hip, np, args.steps, args.warmup, args.cpu_seconds)
+
+    head = put
+    value = head["algorithmic_bytes"] / head["wall_ms"] / 1e6
+    achieved = head["algorithmic_bytes"] / head["kernel_ms"] / 1e6
+    line = {
+        "metric": METRIC,
+        "value": round(value, 1),
+        "unit": "GB/s",
+        "n_gpus": 1,
+        "steps": args.steps,
+        "warmup": args.warmup,
+        "ms_per_step": round(head["wall_ms"], 5),
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": head["dtype"],
+        "data": "synthetic",
+        "config": head["config"],
+        "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS,
+                     "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBS, 4),
+                     "traffic": MEASURED_TRAFFIC_BYTES[head["name"]], "kernel": head["kernel"]},
+        "cpu_baseline": head["cpu_baseline"],
+        "verified": bool(put["verified"] and red["verified"] and a2a["verified"]),
+        "workloads": {"put_block": _summarise(put), "sum_reduce": _summarise(red),
+                      "alltoall": _summarise(a2a)},
+    }
+    print(json.dumps(line))
+    return 0 if line["verified"] else 1
+
+
+if __name__ == "__main__":
+    sys.exit(main())

@@ -37,6 +37,11 @@ enum { NVSHMEM_PERFTEST_SCOPE_THREAD = 0, NVSHMEM_PERFTEST_SCOPE_WARP = 1,
 int nvshmem_perftest_ring_rma(void *dest, const void *src, size_t bytes, int blocks_per_pe,
                               int threads, int scope, int is_get, int iters, void *stream);
 
+/* Counter calibration: PE 0's `src` -> PE 0's `dst`, `bytes` (multiple of 16) with a plain
+ * one-vector-per-thread kernel that uses nothing of the NVSHMEM API.  Reads and writes exactly
+ * `bytes` each. */
+int nvshmem_perftest_plain_copy(void *dst, const void *src, size_t bytes, void *stream);
+
 /* PE p writes value_base + p into word [p] of PE (p+1)%npes's `words` with nvshmem_uint64_p, then
  * (after a barrier) reads word [q] of every PE q's `words`... with nvshmem_uint64_g into
  * out[q] of its own `out`.  words and out hold npes uint64 each. */

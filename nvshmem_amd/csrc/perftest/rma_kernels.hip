@@ -125,6 +125,13 @@ __global__ void ring_reduce_kernel(int32_t *dst, const int32_t *src, size_t nred
     if (threadIdx.x == 0) *(uint64_t *)nvshmem_ptr(signal, me) = 0;  // ready for the next run
 }
 
+// Calibration kernel for hardware counters: a plain copy of a known size that uses nothing of the
+// NVSHMEM API (one 16-byte vector per thread).
+__global__ void plain_copy_kernel(nvshmemi_v4u *dst, const nvshmemi_v4u *src, size_t nvec) {
+    const size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i < nvec) dst[i] = src[i];
+}
+
 template <int SCOPE>
 int launch_ring(bool is_get, char *dest, const char *src, size_t bytes, int blocks, int threads,
                 hipStream_t stream) {
@@ -169,6 +176,17 @@ int nvshmem_perftest_ring_rma(void *dest, const void *src, size_t bytes, int blo
         }
     }
     return rc;
+}
+
+int nvshmem_perftest_plain_copy(void *dst, const void *src, size_t bytes, void *stream) {
+    if (!perftest::ready() || (bytes % 16) || ((uintptr_t)dst % 16) || ((uintptr_t)src % 16) ||
+        !perftest::check_range(dst, bytes) || !perftest::check_range(src, bytes))
+        return NVSHMEMX_ERROR_INVALID_VALUE;
+    const size_t nvec = bytes / 16;
+    if (nvec == 0) return 0;
+    hipLaunchKernelGGL(plain_copy_kernel, dim3((unsigned)((nvec + 255) / 256)), dim3(256), 0,
+                       (hipStream_t)stream, (nvshmemi_v4u *)dst, (const nvshmemi_v4u *)src, nvec);
+    return perftest::launch_status("plain_copy");
 }
 
 int nvshmem_perftest_p_g(uint64_t *words, uint64_t *out, uint64_t value_base, void *stream) {
