@@ -43,12 +43,19 @@ __global__ void moe_dispatch_kernel(char *recv, const char *send, const int32_t 
         const size_t wave = blockIdx.x * waves_per_block + threadIdx.x / NVSHMEMI_WARP_SIZE;
         const size_t nwaves = (size_t)gridDim.x * waves_per_block;
         const bool lane0 = (threadIdx.x % NVSHMEMI_WARP_SIZE) == 0;
-        for (size_t r = wave; r < rows; r += nwaves) {
-            const int pe = my_dest_pe[r];
-            if (!row_ok(pe, my_dest_row[r], np, recv_cap_rows)) continue;
-            nvshmemx_putmem_nbi_warp(recv + (size_t)my_dest_row[r] * row_bytes,
-                                     send + (r / (size_t)topk) * row_bytes, row_bytes, pe);
-            if (lane0) atomicAdd(&tally[pe], 1u);
+        // A wavefront takes a token and pushes its topk copies back to back: the first put streams
+        // the row from HBM, the others find it in this XCD's L2, so every source row crosses the HBM
+        // interface once and is written topk times.
+        for (size_t t = wave; t < (size_t)tokens; t += nwaves) {
+            const char *src_row = send + t * row_bytes;
+            for (int k = 0; k < topk; ++k) {
+                const size_t r = t * (size_t)topk + (size_t)k;
+                const int pe = my_dest_pe[r];
+                const int64_t row = my_dest_row[r];
+                if (!row_ok(pe, row, np, recv_cap_rows)) continue;
+                nvshmemx_putmem_nbi_warp(recv + (size_t)row * row_bytes, src_row, row_bytes, pe);
+                if (lane0) atomicAdd(&tally[pe], 1u);
+            }
         }
     } else {
         for (size_t r = blockIdx.x; r < rows; r += gridDim.x) {
