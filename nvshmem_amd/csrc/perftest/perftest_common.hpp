@@ -20,7 +20,7 @@ inline bool ready() {
 }
 
 inline bool check_launch(int blocks, int threads) {
-    if (blocks >= 1 && blocks <= 65535 && threads >= 1 && threads <= 1024) return true;
+    if (blocks >= 1 && blocks <= (1 << 22) && threads >= 1 && threads <= 1024) return true;
     fprintf(stderr, "nvshmem_perftest: bad launch shape: %d blocks x %d threads\n", blocks, threads);
     return false;
 }
