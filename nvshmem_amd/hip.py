@@ -103,3 +103,35 @@ class Event:
         if self.handle:
             lib().hipEventDestroy(self.handle)
             self.handle = C.c_void_p()
+
+
+class Graph:
+    """Stream capture into a HIP graph: `with Graph(stream) as g: ...enqueue...`, then g.launch()."""
+
+    def __init__(self, stream):
+        self.stream = stream
+        self.graph = C.c_void_p()
+        self.exe = C.c_void_p()
+
+    def __enter__(self):
+        # hipStreamCaptureModeThreadLocal = 1
+        check(lib().hipStreamBeginCapture(self.stream.handle, C.c_int(1)), "hipStreamBeginCapture")
+        return self
+
+    def __exit__(self, exc_type, exc, tb):
+        code = lib().hipStreamEndCapture(self.stream.handle, C.byref(self.graph))
+        if exc_type is None:
+            check(code, "hipStreamEndCapture")
+            check(lib().hipGraphInstantiate(C.byref(self.exe), self.graph, None, None, C.c_size_t(0)),
+                  "hipGraphInstantiate")
+
+    def launch(self):
+        check(lib().hipGraphLaunch(self.exe, self.stream.handle), "hipGraphLaunch")
+
+    def destroy(self):
+        if self.exe:
+            lib().hipGraphExecDestroy(self.exe)
+            self.exe = C.c_void_p()
+        if self.graph:
+            lib().hipGraphDestroy(self.graph)
+            self.graph = C.c_void_p()

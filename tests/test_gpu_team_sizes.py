@@ -1,0 +1,78 @@
+"""GPU parity for team sizes other than the headline 8 / 16: 1, 2, 3, 5 (not a power of two),
+32 and 64 (the reduce kernel then gives a PE fewer than 64 lanes)."""
+import numpy as np
+import pytest
+
+import nvshmem_amd as N
+import oracle_lib as O
+from gpu_util import bits_equal, note, runtime
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.mark.parametrize("npes", [1, 2, 3, 5, 32, 64])
+def test_collectives_and_rma_for_team_size(npes):
+    rng = np.random.default_rng(npes)
+    with runtime(npes, 16 << 20) as rt:
+        perf = rt.perftest()
+        assert rt.lib.nvshmem_n_pes() == npes
+        n = 5003
+        src = rt.malloc(npes * n * 8 + 64); dst = rt.malloc(npes * n * 8 + 64)
+        # host-launched reduce: fp32 sum (order-sensitive), bf16 max, int64 xor, in place too
+        f = (rng.standard_normal((npes, n)) * 10.0 ** rng.integers(-3, 4, (npes, n))).astype(np.float32)
+        rt.upload_all(src, f)
+        note("npes=%d float sum" % npes)
+        rt.reduce("float", "sum", dst, src, n)
+        want = O.reduce("f32", "sum", f)
+        for pe in {0, npes // 2, npes - 1}:
+            assert bits_equal(rt.download(dst, pe, (n,), np.float32), want), pe
+        rt.reduce("float", "sum", src, src, n)
+        assert bits_equal(rt.download(src, npes - 1, (n,), np.float32), want)
+        b = (rng.standard_normal((npes, n)).astype(np.float32).view(np.uint32) >> 16).astype(np.uint16)
+        rt.upload_all(src, b)
+        rt.reduce("bfloat16", "max", dst, src, n)
+        assert bits_equal(rt.download(dst, 0, (n,), np.uint16), O.reduce("bf16", "max", b))
+        x = rng.integers(-2**63, 2**63 - 1, (npes, n), dtype=np.int64)
+        rt.upload_all(src, x)
+        rt.reduce("int64", "xor", dst, src, n)
+        assert np.array_equal(rt.download(dst, npes - 1, (n,), np.int64), O.reduce("i64", "xor", x))
+        # fcollect / alltoall with a ragged block size
+        seg = 1237
+        data = rng.integers(0, 256, (npes, npes * seg), dtype=np.uint8)
+        rt.upload_all(src, data)
+        note("npes=%d alltoall/fcollect" % npes)
+        rt.alltoallmem(dst, src, seg)
+        assert np.array_equal(rt.download_all(dst, (npes * seg,), np.uint8), O.alltoall(data))
+        rt.fcollectmem(dst, src, seg)
+        assert np.array_equal(rt.download_all(dst, (npes * seg,), np.uint8), O.fcollect(data[:, :seg]))
+        # device-initiated ring put and the in-kernel barrier / reduce / alltoall
+        note("npes=%d device ring put" % npes)
+        assert perf.nvshmem_perftest_ring_rma(dst, src, 70001, 2, 256, N.SCOPE_BLOCK, 0, 1, None) == 0
+        rt.sync()
+        got = rt.download_all(dst, (70001,), np.uint8)
+        raw = rt.download_all(src, (70001,), np.uint8)
+        assert np.array_equal(got, O.ring_put(raw))
+        counter = rt.calloc(1, 8); errors = rt.calloc(1, 8)
+        note("npes=%d device barrier" % npes)
+        assert perf.nvshmem_perftest_device_barrier(counter, errors, 50, N.SCOPE_BLOCK, 128, None) == 0
+        rt.sync()
+        assert not rt.download_all(errors, (1,), np.uint64).any()
+        ints = rng.integers(-2**20, 2**20, (npes, n), dtype=np.int32)
+        rt.upload_all(src, ints)
+        note("npes=%d device reduce" % npes)
+        assert perf.nvshmem_perftest_device_reduce(N.DTYPES["i32"], N.OPS["sum"], dst, src, n,
+                                                   N.SCOPE_BLOCK, 256, None) == 0
+        rt.sync()
+        assert np.array_equal(rt.download(dst, npes - 1, (n,), np.int32), O.reduce("i32", "sum", ints))
+        rt.upload_all(src, data)
+        assert perf.nvshmem_perftest_device_alltoall(dst, src, seg, N.SCOPE_WARP, 64, None) == 0
+        rt.sync()
+        assert np.array_equal(rt.download_all(dst, (npes * seg,), np.uint8), O.alltoall(data))
+        assert all(rt.read_timeout(pe)[0] == 0 for pe in range(npes))
+
+
+def test_init_rejects_bad_team_sizes():
+    lib = N.load()
+    assert lib.nvshmemx_amd_init(0, 1 << 20) != 0
+    assert lib.nvshmemx_amd_init(65, 1 << 20) != 0
+    assert lib.nvshmemx_init_status() == 0
