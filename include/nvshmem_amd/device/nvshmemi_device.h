@@ -129,7 +129,7 @@ NVSHMEMI_DEVICE_INLINE void *nvshmemi_ptr(const void *ptr, int pe) {
  *
  * Byte-exact copy by the lanes of one thread group.  Where the reference picks the widest element
  * both pointers are aligned to and cascades, this version always stores 16-byte vectors: a byte
- * head brings dst to a 16-byte boundary, the body issues eight independent dwordx4 loads per lane
+ * head brings dst to a 16-byte boundary, the body issues four independent dwordx4 loads per lane
  * before the first store (gfx950 accepts unaligned vector loads, so a src that is not co-aligned
  * only costs extra cache-line touches, not narrower instructions), and a byte tail finishes.
  * ---------------------------------------------------------------------------------------------- */
@@ -137,12 +137,14 @@ typedef unsigned int nvshmemi_v4u __attribute__((ext_vector_type(4)));
 typedef nvshmemi_v4u __attribute__((aligned(1))) nvshmemi_v4u_unaligned;
 
 #ifndef NVSHMEMI_AMD_COPY_UNROLL
-#define NVSHMEMI_AMD_COPY_UNROLL 8
+#define NVSHMEMI_AMD_COPY_UNROLL 4
 #endif
 /* bit 0: non-temporal loads, bit 1: non-temporal stores in the vector body.  Stores stream (the
- * copy never reads its destination back); loads stay temporal because callers often push the same
- * source to several PEs (top-k token dispatch, all-push collectives) and the repeats then hit in L2:
- * measured 1.4x on the MoE dispatch, no loss on a pure streaming put. */
+ * copy never reads its destination back).  Loads stay cacheable by default because callers often
+ * push the same source to several PEs (top-k token dispatch, all-push collectives) and the repeats
+ * then hit in L2: measured 1.4x on the MoE dispatch.  A translation unit whose kernels only stream
+ * bulk data once may define NVSHMEMI_AMD_COPY_NT 3 before including nvshmem.h: measured +5 % on a
+ * 256 MiB put. */
 #ifndef NVSHMEMI_AMD_COPY_NT
 #define NVSHMEMI_AMD_COPY_NT 2
 #endif
@@ -164,24 +166,32 @@ NVSHMEMI_DEVICE_INLINE void nvshmemi_amd_stream_store16(char *p, nvshmemi_v4u v)
     else *reinterpret_cast<nvshmemi_v4u *>(p) = v;
 }
 
-/* nvec vectors, lane `tid` of `nthr` takes tid, tid+nthr, ...: UNROLL independent loads are issued
- * before the first store; the last round is predicated instead of falling back to one vector at a
- * time, so a short copy (a 14 KiB row moved by one wavefront, say) still has all its loads in flight
- * at once. */
+/* Lane `tid` of `nthr` owns vectors tid, tid+nthr, ...  Rounds of U vectors per lane are straight-line
+ * code - U independent loads issued before the first store - and run while the lane still has U
+ * vectors left; the remainder is handled by the same code at U/2, U/4, ... 1, so a short copy (a
+ * 14 KiB row moved by one wavefront is 14 vectors per lane: 4 + 4 + 4 + 2) keeps most of its loads in
+ * flight.  No per-vector predicates: branches between the loads would make them wait for each
+ * other. */
+template <bool SRC_ALIGNED, int U>
+NVSHMEMI_DEVICE_INLINE size_t nvshmemi_amd_copy_rounds(char *__restrict__ dst,
+                                                      const char *__restrict__ src, size_t nvec,
+                                                      size_t i, size_t nthr) {
+    for (; i + (U - 1) * nthr < nvec; i += U * nthr) {
+        nvshmemi_v4u v[U];
+#pragma unroll
+        for (int u = 0; u < U; ++u) v[u] = nvshmemi_amd_stream_load16<SRC_ALIGNED>(src + 16 * (i + u * nthr));
+#pragma unroll
+        for (int u = 0; u < U; ++u) nvshmemi_amd_stream_store16(dst + 16 * (i + u * nthr), v[u]);
+    }
+    if constexpr (U > 1) return nvshmemi_amd_copy_rounds<SRC_ALIGNED, U / 2>(dst, src, nvec, i, nthr);
+    return i;
+}
+
 template <bool SRC_ALIGNED>
 NVSHMEMI_DEVICE_INLINE void nvshmemi_amd_copy_vectors(char *__restrict__ dst,
                                                      const char *__restrict__ src, size_t nvec,
                                                      size_t tid, size_t nthr) {
-    constexpr int U = NVSHMEMI_AMD_COPY_UNROLL;
-    for (size_t i = tid; i < nvec; i += U * nthr) {
-        nvshmemi_v4u v[U];
-#pragma unroll
-        for (int u = 0; u < U; ++u)
-            if (i + u * nthr < nvec) v[u] = nvshmemi_amd_stream_load16<SRC_ALIGNED>(src + 16 * (i + u * nthr));
-#pragma unroll
-        for (int u = 0; u < U; ++u)
-            if (i + u * nthr < nvec) nvshmemi_amd_stream_store16(dst + 16 * (i + u * nthr), v[u]);
-    }
+    nvshmemi_amd_copy_rounds<SRC_ALIGNED, NVSHMEMI_AMD_COPY_UNROLL>(dst, src, nvec, tid, nthr);
 }
 
 template <int SCOPE>

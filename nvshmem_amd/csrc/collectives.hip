@@ -32,15 +32,24 @@ namespace {
 #ifndef NVSHMEM_AMD_FCOLLECT_UNROLL /* vectors per lane in an fcollect tile */
 #define NVSHMEM_AMD_FCOLLECT_UNROLL 1
 #endif
-#ifndef NVSHMEM_AMD_COLL_NT /* bit 0: non-temporal loads, bit 1: non-temporal stores */
+#ifndef NVSHMEM_AMD_COLL_NT /* bit 0: non-temporal loads allowed, bit 1: non-temporal stores */
 #define NVSHMEM_AMD_COLL_NT 3
+#endif
+/* Sources up to this many bytes (all PEs together) are loaded with the default, cacheable policy:
+ * they fit the 256 MiB Infinity Cache, so a source that is sent again (or was just produced) is
+ * served from it (measured +30 % on the 1M-element reduce, +20..45 % on 256 MiB collectives).
+ * Larger sources are streamed with non-temporal loads (+5 % at 2 GiB).  Stores always stream. */
+#ifndef NVSHMEM_AMD_CACHEABLE_SOURCE_BYTES
+#define NVSHMEM_AMD_CACHEABLE_SOURCE_BYTES ((uint64_t)256 << 20)
 #endif
 
 constexpr int kThreads = NVSHMEM_AMD_COLL_THREADS;
 constexpr int kCopyThreads = NVSHMEM_AMD_COPY_THREADS;
 
+template <bool NTL>
 __device__ __forceinline__ nvshmemi_v4u stream_load(const char *p) {
-    if (NVSHMEM_AMD_COLL_NT & 1) return __builtin_nontemporal_load(reinterpret_cast<const nvshmemi_v4u *>(p));
+    if (NTL && (NVSHMEM_AMD_COLL_NT & 1))
+        return __builtin_nontemporal_load(reinterpret_cast<const nvshmemi_v4u *>(p));
     return *reinterpret_cast<const nvshmemi_v4u *>(p);
 }
 __device__ __forceinline__ void stream_store(char *p, nvshmemi_v4u v) {
@@ -63,14 +72,14 @@ enum { kModeFcollect = 0, kModeAlltoall = 1 };
 
 // Copies the vectors v0 + t + u*kCopyThreads (u < unroll) that fall inside [0, nvec); indices in front of
 // the segment wrap to huge unsigned values and are skipped the same way as those behind it.
-template <bool SRC_ALIGNED, bool REPLICATE, int kCopyUnroll>
+template <bool SRC_ALIGNED, bool REPLICATE, int kCopyUnroll, bool NTL>
 __device__ __forceinline__ void copy_tile(char *__restrict__ dst, const char *__restrict__ src,
                                           uint64_t v0, uint64_t nvec, uint64_t rep_stride, int nrep) {
     nvshmemi_v4u v[kCopyUnroll];
 #pragma unroll
     for (int u = 0; u < kCopyUnroll; ++u) {
         const uint64_t i = v0 + threadIdx.x + (uint64_t)u * kCopyThreads;
-        if (i < nvec) v[u] = SRC_ALIGNED ? stream_load(src + 16 * i) : nvshmemi_amd_load16<false>(src + 16 * i);
+        if (i < nvec) v[u] = SRC_ALIGNED ? stream_load<NTL>(src + 16 * i) : nvshmemi_amd_load16<false>(src + 16 * i);
     }
     if (REPLICATE) {
         for (int r = 0; r < nrep; ++r) {
@@ -90,7 +99,7 @@ __device__ __forceinline__ void copy_tile(char *__restrict__ dst, const char *__
     }
 }
 
-template <int MODE, int kCopyUnroll>
+template <int MODE, int kCopyUnroll, bool NTL>
 __global__ __launch_bounds__(kCopyThreads) void segment_copy_kernel(char *base, uint32_t shift, int npes,
                                                                 uint64_t dst_off, uint64_t src_off,
                                                                 uint64_t seg_bytes) {
@@ -136,11 +145,11 @@ __global__ __launch_bounds__(kCopyThreads) void segment_copy_kernel(char *base, 
     char *d = dst + head;
     const bool aligned = (((uintptr_t)s) & 15) == 0;
     if (MODE == kModeFcollect) {
-        if (aligned) copy_tile<true, true, kCopyUnroll>(d, s, v0, nvec_total, rep_stride, nrep);
-        else copy_tile<false, true, kCopyUnroll>(d, s, v0, nvec_total, rep_stride, nrep);
+        if (aligned) copy_tile<true, true, kCopyUnroll, NTL>(d, s, v0, nvec_total, rep_stride, nrep);
+        else copy_tile<false, true, kCopyUnroll, NTL>(d, s, v0, nvec_total, rep_stride, nrep);
     } else {
-        if (aligned) copy_tile<true, false, kCopyUnroll>(d, s, v0, nvec_total, rep_stride, 1);
-        else copy_tile<false, false, kCopyUnroll>(d, s, v0, nvec_total, rep_stride, 1);
+        if (aligned) copy_tile<true, false, kCopyUnroll, NTL>(d, s, v0, nvec_total, rep_stride, 1);
+        else copy_tile<false, false, kCopyUnroll, NTL>(d, s, v0, nvec_total, rep_stride, 1);
     }
 }
 
@@ -156,7 +165,7 @@ __global__ __launch_bounds__(kCopyThreads) void segment_copy_kernel(char *base, 
 // ---------------------------------------------------------------------------------------------
 // NPES > 0 fixes the team size at compile time (fold fully unrolled, one wavefront per PE);
 // NPES == 0 takes both from the arguments.
-template <typename T, int OP, int NPES>
+template <typename T, int OP, int NPES, bool NTL>
 __global__ __launch_bounds__(NPES ? NPES * 64 : 1024) void reduce_vector_kernel(char *base, uint32_t shift, int npes_arg,
                                                              uint32_t lane_shift_arg, uint64_t dst_off,
                                                              uint64_t src_off, uint64_t nelems) {
@@ -181,7 +190,7 @@ __global__ __launch_bounds__(NPES ? NPES * 64 : 1024) void reduce_vector_kernel(
 
     for (uint64_t tile = blockIdx.x; tile < ntiles; tile += gridDim.x) {
         const uint64_t v = (tile << lane_shift) + i - lead;  // wraps to a huge value in front of the buffer
-        if (v < nvec) stage[threadIdx.x] = stream_load(base + (uint64_t)pe * pe_stride + src_off + 16 * v);
+        if (v < nvec) stage[threadIdx.x] = stream_load<NTL>(base + (uint64_t)pe * pe_stride + src_off + 16 * v);
         __syncthreads();
         for (unsigned e = threadIdx.x; e < tile_elems; e += blockDim.x) {
             T acc = stage_e[e];
@@ -237,10 +246,19 @@ void launch_reduce(Runtime &rt, uint64_t dst_off, uint64_t src_off, uint64_t nel
         if (blocks > 0x7fffffffull) blocks = 0x7fffffffull;  // the tile loop covers the rest
         if (blocks == 0) blocks = 1;                          // only tail elements
         const size_t lds = ((size_t)rt.npes + 1) * 16 << lane_shift;
+        const bool stream_source =
+            (uint64_t)rt.npes * nelems * sizeof(T) > NVSHMEM_AMD_CACHEABLE_SOURCE_BYTES;
 #define NVSHMEM_AMD_LAUNCH_REDUCE(N)                                                              \
-    hipLaunchKernelGGL((reduce_vector_kernel<T, OP, N>), dim3((unsigned)blocks), dim3(threads),   \
-                       lds, stream, rt.base, rt.heap_shift, rt.npes, lane_shift, dst_off,         \
-                       src_off, nelems)
+    do {                                                                                          \
+        if (stream_source)                                                                        \
+            hipLaunchKernelGGL((reduce_vector_kernel<T, OP, N, true>), dim3((unsigned)blocks),    \
+                               dim3(threads), lds, stream, rt.base, rt.heap_shift, rt.npes,       \
+                               lane_shift, dst_off, src_off, nelems);                             \
+        else                                                                                      \
+            hipLaunchKernelGGL((reduce_vector_kernel<T, OP, N, false>), dim3((unsigned)blocks),   \
+                               dim3(threads), lds, stream, rt.base, rt.heap_shift, rt.npes,       \
+                               lane_shift, dst_off, src_off, nelems);                             \
+    } while (0)
         switch (rt.npes) {
             case 8: NVSHMEM_AMD_LAUNCH_REDUCE(8); break;
             case 16: NVSHMEM_AMD_LAUNCH_REDUCE(16); break;
@@ -375,14 +393,19 @@ static int segment_collective(int mode, const char *what, nvshmem_team_t team, v
         set_error("%s: message too large", what);
         return NVSHMEMX_ERROR_INVALID_VALUE;
     }
-    if (mode == kModeFcollect)
-        hipLaunchKernelGGL((segment_copy_kernel<kModeFcollect, NVSHMEM_AMD_FCOLLECT_UNROLL>), dim3((unsigned)tiles, segs),
-                           dim3(kCopyThreads), 0, stream, rt.base, rt.heap_shift, rt.npes, doff, soff,
-                           (uint64_t)seg_bytes);
-    else
-        hipLaunchKernelGGL((segment_copy_kernel<kModeAlltoall, NVSHMEM_AMD_ALLTOALL_UNROLL>), dim3((unsigned)tiles, segs),
-                           dim3(kCopyThreads), 0, stream, rt.base, rt.heap_shift, rt.npes, doff, soff,
-                           (uint64_t)seg_bytes);
+    const bool stream_source = src_bytes * n > NVSHMEM_AMD_CACHEABLE_SOURCE_BYTES;
+    const dim3 grid((unsigned)tiles, segs), block(kCopyThreads);
+#define NVSHMEM_AMD_LAUNCH_SEGCOPY(MODE, U, NTL)                                                   \
+    hipLaunchKernelGGL((segment_copy_kernel<MODE, U, NTL>), grid, block, 0, stream, rt.base,       \
+                       rt.heap_shift, rt.npes, doff, soff, (uint64_t)seg_bytes)
+    if (mode == kModeFcollect) {
+        if (stream_source) NVSHMEM_AMD_LAUNCH_SEGCOPY(kModeFcollect, NVSHMEM_AMD_FCOLLECT_UNROLL, true);
+        else NVSHMEM_AMD_LAUNCH_SEGCOPY(kModeFcollect, NVSHMEM_AMD_FCOLLECT_UNROLL, false);
+    } else {
+        if (stream_source) NVSHMEM_AMD_LAUNCH_SEGCOPY(kModeAlltoall, NVSHMEM_AMD_ALLTOALL_UNROLL, true);
+        else NVSHMEM_AMD_LAUNCH_SEGCOPY(kModeAlltoall, NVSHMEM_AMD_ALLTOALL_UNROLL, false);
+    }
+#undef NVSHMEM_AMD_LAUNCH_SEGCOPY
     hipError_t e = hipGetLastError();
     if (e != hipSuccess) {
         set_error("%s: kernel launch failed: %s", what, hipGetErrorString(e));

@@ -7,6 +7,9 @@
 // examples/ring-reduce.cu:88-144.
 #include <hip/hip_runtime.h>
 
+// The kernels of this file move bulk data that is read once: stream the loads too.
+#define NVSHMEMI_AMD_COPY_NT 3
+
 #include "nvshmem_perftest.h"
 #include "nvshmemx.h"
 #include "perftest_common.hpp"
