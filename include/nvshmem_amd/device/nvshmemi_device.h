@@ -515,29 +515,58 @@ NVSHMEMI_DEVICE_INLINE T nvshmemi_amd_fold_step(int i, T acc, T x) {
  * ---------------------------------------------------------------------------------------------- */
 /* Reduce: PE `me` owns the element range [me*chunk, (me+1)*chunk): it folds that range from every
  * PE's source and stores the result into every PE's dest.  Each element is read by exactly one lane
- * before that lane overwrites it, so source == dest is safe, and every source byte is read once. */
+ * before that lane overwrites it, so source == dest is safe, and every source byte is read once.
+ * When both buffers are 16-byte aligned the range is cut on vector boundaries and moved as
+ * dwordx4; otherwise element by element. */
+template <typename T, int OP>
+NVSHMEMI_DEVICE_INLINE T nvshmemi_amd_fold_element(const T *src0, size_t pe_stride, int npes, size_t i) {
+    T acc = src0[i];
+    for (int pe = 1; pe < npes; ++pe)
+        acc = nvshmemi_amd_fold_step<T, OP>(pe, acc, src0[(size_t)pe * pe_stride + i]);
+    return acc;
+}
+
 template <typename T, int OP, int SCOPE>
 NVSHMEMI_DEVICE_INLINE int nvshmemi_reduce_threadgroup(nvshmem_team_t team, T *dest, const T *source,
                                                        size_t nreduce) {
     (void)team;
+    constexpr size_t VEC = 16 / sizeof(T);
+    struct alignas(16) pack_t { T e[VEC]; };
     const int me = nvshmemi_amd_my_pe();
     const int npes = nvshmemi_device_state_d.npes;
     const size_t tid = (size_t)nvshmemi_thread_id_in_threadgroup<SCOPE>();
     const size_t nthr = (size_t)nvshmemi_threadgroup_size<SCOPE>();
     /* every PE's source is complete and visible before anyone reads it */
     nvshmemi_barrier_threadgroup<SCOPE>();
-    const size_t chunk = (nreduce + (size_t)npes - 1) / (size_t)npes;
+    const T *src0 = reinterpret_cast<const T *>(nvshmemi_amd_remote(source, 0));
+    T *dst0 = reinterpret_cast<T *>(nvshmemi_amd_remote(dest, 0));
+    const size_t pe_stride = (size_t)(nvshmemi_device_state_d.heap_size / sizeof(T));
+    const bool vectors = (((uintptr_t)src0 | (uintptr_t)dst0) & 15) == 0;
+    /* chunk in elements, a whole number of vectors on the vector path */
+    size_t chunk = (nreduce + (size_t)npes - 1) / (size_t)npes;
+    if (vectors) chunk = (chunk + VEC - 1) / VEC * VEC;
     size_t lo = (size_t)me * chunk;
     if (lo > nreduce) lo = nreduce;
     size_t hi = lo + chunk;
     if (hi > nreduce) hi = nreduce;
-    const T *src0 = reinterpret_cast<const T *>(nvshmemi_amd_remote(source, 0));
-    T *dst0 = reinterpret_cast<T *>(nvshmemi_amd_remote(dest, 0));
-    const size_t pe_stride = (size_t)(nvshmemi_device_state_d.heap_size / sizeof(T));
-    for (size_t i = lo + tid; i < hi; i += nthr) {
-        T acc = src0[i];
-        for (int pe = 1; pe < npes; ++pe)
-            acc = nvshmemi_amd_fold_step<T, OP>(pe, acc, src0[(size_t)pe * pe_stride + i]);
+    size_t i = lo + tid;
+    if (vectors) {
+        const size_t nvec = (hi - lo) / VEC;
+        for (size_t v = tid; v < nvec; v += nthr) {
+            const size_t at = lo + v * VEC;
+            pack_t acc = *reinterpret_cast<const pack_t *>(src0 + at);
+            for (int pe = 1; pe < npes; ++pe) {
+                const pack_t x = *reinterpret_cast<const pack_t *>(src0 + (size_t)pe * pe_stride + at);
+#pragma unroll
+                for (size_t k = 0; k < VEC; ++k) acc.e[k] = nvshmemi_amd_fold_step<T, OP>(pe, acc.e[k], x.e[k]);
+            }
+            for (int pe = 0; pe < npes; ++pe)
+                *reinterpret_cast<pack_t *>(dst0 + (size_t)pe * pe_stride + at) = acc;
+        }
+        i = lo + nvec * VEC + tid; /* the last PE's range may end inside a vector */
+    }
+    for (; i < hi; i += nthr) {
+        const T acc = nvshmemi_amd_fold_element<T, OP>(src0, pe_stride, npes, i);
         for (int pe = 0; pe < npes; ++pe) dst0[(size_t)pe * pe_stride + i] = acc;
     }
     nvshmemi_barrier_threadgroup<SCOPE>();

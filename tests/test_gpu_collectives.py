@@ -237,6 +237,12 @@ def test_device_scope_collectives(rt8, scope, threads):
                                                threads, None) == 0
     rt8.sync()
     assert bits_equal(rt8.download(src, 4, (n,), np.float32), O.reduce("f32", "sum", data))
+    # buffers offset by one element: the element-at-a-time path of the in-kernel reduce
+    rt8.upload_all(src, data, 4)
+    assert perf.nvshmem_perftest_device_reduce(N.DTYPES["f32"], N.OPS["sum"], dst + 4, src + 4, n, scope,
+                                               threads, None) == 0
+    rt8.sync()
+    assert bits_equal(rt8.download(dst, 6, (n,), np.float32, 4), O.reduce("f32", "sum", data))
     assert perf.nvshmem_perftest_device_reduce(N.DTYPES["f32"], N.OPS["xor"], dst, src, n, scope,
                                                threads, None) == 3   # NVSHMEMX_ERROR_NOT_SUPPORTED
     for seg in (1, 100, 4097):
