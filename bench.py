@@ -30,7 +30,7 @@ MEASURED_TRAFFIC_BYTES = {
     "put_block": (2048 + 2048) << 20,    # profiles/ring_rma_kernel_put_block_8pe_256MiB.txt
     "sum_reduce": (2048 + 2048) << 20,   # profiles/reduce_vector_kernel_float_sum_8pe_64Mi.txt
     "alltoall": (256 + 256) << 20,       # profiles/segment_copy_kernel_alltoall_16pe_4Mi_fp32.txt
-    "alltoall_1GiB": None,
+    "alltoall_1GiB": None,              # not profiled
 }
 
 # put_block launch shape: each block moves a contiguous 16 KiB slice (short-lived blocks keep the

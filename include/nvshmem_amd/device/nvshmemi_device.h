@@ -249,9 +249,30 @@ NVSHMEMI_DEVICE_INLINE void nvshmemi_get(T *dest, const T *source, size_t nelems
     nvshmemi_threadgroup_sync<SCOPE>();
 }
 
+/* The value is stored with an agent-scope atomic store of its bits, so that it leaves this XCD's L2
+ * on its own: the OpenSHMEM idiom "p a flag, the target waits on it" must make progress without a
+ * quiet in between. */
 template <typename T>
 NVSHMEMI_DEVICE_INLINE void nvshmemi_p(T *dest, const T value, int pe) {
-    *reinterpret_cast<T *>(nvshmemi_amd_remote(dest, pe)) = value;
+    char *p = nvshmemi_amd_remote(dest, pe);
+    if constexpr (sizeof(T) == 1) {
+        uint8_t v;
+        __builtin_memcpy(&v, &value, 1);
+        __hip_atomic_store((uint8_t *)p, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    } else if constexpr (sizeof(T) == 2) {
+        uint16_t v;
+        __builtin_memcpy(&v, &value, 2);
+        __hip_atomic_store((uint16_t *)p, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    } else if constexpr (sizeof(T) == 4) {
+        uint32_t v;
+        __builtin_memcpy(&v, &value, 4);
+        __hip_atomic_store((uint32_t *)p, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    } else {
+        static_assert(sizeof(T) == 8, "scalar put supports 1, 2, 4 and 8 byte elements");
+        uint64_t v;
+        __builtin_memcpy(&v, &value, 8);
+        __hip_atomic_store((uint64_t *)p, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    }
 }
 
 /* A remote word may be written by another PE while this kernel runs, so the read is an agent-scope

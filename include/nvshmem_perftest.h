@@ -72,6 +72,13 @@ int nvshmem_perftest_ring_reduce(int32_t *dst, const int32_t *src, size_t nreduc
                                  uint64_t *signal, size_t chunk_elems, int blocks, int threads,
                                  void *stream);
 
+/* Walks through typed / sized / strided RMA in all scopes, scalar p/g, thread-scope put_signal,
+ * typed wait / test and sync_all on small fixed layouts (a, b: 8 KiB; sig: 4 words, zero before
+ * the call; ints: 8 int32, zero; out: 16 int64).  tests/test_gpu_api_matrix.py states what each
+ * region must hold afterwards. */
+int nvshmem_perftest_api_matrix(void *a, void *b, uint64_t *sig, int *ints, int64_t *out,
+                                int threads, void *stream);
+
 /* In-kernel collectives, one thread group per PE (grid 1 x 1 x npes).  dtype/op use the numbering
  * of nvshmemi_amd_dtype_t / nvshmemi_amd_op_t; supported pairs: (i32,sum) (i64,xor) (f32,sum)
  * (f32,max) (bf16,sum) (bf16,max) (u64,and) (f64,prod) (i16,min).  Returns NOT_SUPPORTED else. */

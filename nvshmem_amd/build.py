@@ -27,7 +27,7 @@ HIP_FLAGS = [
 
 RUNTIME_SOURCES = ["mspace.cpp", "runtime.hip", "collectives.hip"]
 PERFTEST_SOURCES = ["perftest/rma_kernels.hip", "perftest/coll_kernels.hip",
-                    "perftest/moe_shuffle.hip"]
+                    "perftest/moe_shuffle.hip", "perftest/api_matrix.hip"]
 
 
 def _run(cmd):

@@ -45,11 +45,72 @@ def counter_avg(directory, counter):
     return {_short(n): (v, c) for n, v, c in rows}
 
 
+# workloads of nvshmem_amd/profile_workloads.py: kernel -> (file name, description, algorithmic bytes)
+WORKLOADS = {
+    "ring_rma_kernel<2, false>": (
+        "ring_rma_kernel_put_block_8pe_256MiB.txt",
+        "put_block: nvshmemx_putmem_block ring, 8 logical PEs x 256 MiB, 16384 blocks x 512 threads per PE.\n"
+        "Algorithmic bytes per launch: 8 x 256 MiB read + 8 x 256 MiB written = 4 GiB.", 4 << 30),
+    "reduce_vector_kernel<float, 5, 8, true>": (
+        "reduce_vector_kernel_float_sum_8pe_64Mi.txt",
+        "sum_reduce: nvshmemx_float_sum_reduce_on_stream, 8 logical PEs x 2^26 fp32.\n"
+        "Algorithmic bytes per launch: 8 sources read once + 8 destinations written once = 4 GiB.", 4 << 30),
+    "segment_copy_kernel<1, 1, false>": (
+        "segment_copy_kernel_alltoall_16pe_4Mi_fp32.txt",
+        "alltoall: nvshmemx_float_alltoall_on_stream, 16 logical PEs x 2^22 fp32 (block 2^18 elements).\n"
+        "Algorithmic bytes per launch: 256 MiB read + 256 MiB written = 512 MiB.  The 256 MiB source fits the\n"
+        "Infinity Cache and the profiled loop re-sends it; FETCH_SIZE counts between L2 and the fabric and\n"
+        "cannot tell a cache hit from an HBM read, but a rate above the HBM peak shows that part of the\n"
+        "reads are served by the cache.", 512 << 20),
+    "segment_copy_kernel<0, 1, false>": (
+        "segment_copy_kernel_fcollect_16pe_4Mi_fp32.txt",
+        "fcollect: nvshmemx_float_fcollect_on_stream, 16 logical PEs x 2^22 fp32.\n"
+        "Algorithmic bytes per launch: 256 MiB read + 16 x 256 MiB written = 4.25 GiB.", (17 * 256) << 20),
+    "plain_copy_kernel": (
+        "plain_copy_kernel_calibration_1GiB.txt",
+        "Counter calibration: plain one-vector-per-thread copy, 1 GiB read + 1 GiB written.", 2 << 30),
+}
+
+COMMANDS = """Commands (from the repository root on the GPU box; every file they run is committed):
+  cd /tmp && export TMPDIR=/tmp
+  rocprofv3 --kernel-trace --stats -d $REPO/gpurun_out/prof_stats -- python3 $REPO/nvshmem_amd/profile_workloads.py
+  rocprofv3 --pmc FETCH_SIZE -d $REPO/gpurun_out/prof_fetch -- python3 $REPO/nvshmem_amd/profile_workloads.py --iters 5
+  rocprofv3 --pmc WRITE_SIZE -d $REPO/gpurun_out/prof_write -- python3 $REPO/nvshmem_amd/profile_workloads.py --iters 5
+  python3 nvshmem_amd/profile_summary.py --stats gpurun_out/prof_stats --fetch gpurun_out/prof_fetch \\
+          --write gpurun_out/prof_write --profiles-dir profiles
+Hardware: one MI355X (gfx950), ROCm 7.2.  Durations are per dispatch from the kernel trace."""
+
+
+def write_profiles(directory, stats, fetch, write, fscale, wscale):
+    os.makedirs(directory, exist_ok=True)
+    by_name = {s[0]: s for s in stats}
+    for kernel, (fname, desc, alg) in WORKLOADS.items():
+        if kernel not in by_name:
+            continue
+        name, calls, avg, lo, hi = by_name[kernel]
+        lines = [desc, "", COMMANDS, "",
+                 "%-46s %6s %12s %12s %12s" % ("kernel", "calls", "avg us", "min us", "max us"),
+                 "%-46s %6d %12.2f %12.2f %12.2f" % (name[:46], calls, avg, lo, hi), ""]
+        if fscale and wscale and kernel in fetch and kernel in write:
+            f, w = fetch[kernel][0], write[kernel][0]
+            lines += ["counters (KiB per dispatch): FETCH_SIZE %.1f  WRITE_SIZE %.1f" % (f, w),
+                      "scale factors from plain_copy_kernel (1 GiB read + 1 GiB written): "
+                      "FETCH_SIZE x%.4f, WRITE_SIZE x%.4f" % (fscale, wscale),
+                      "HBM traffic per dispatch (scaled): read %.1f MiB + written %.1f MiB = %.1f MiB; "
+                      "algorithmic bytes %.1f MiB" % (f * fscale / 1024, w * wscale / 1024,
+                                                      (f * fscale + w * wscale) / 1024, alg / 2**20), ""]
+        lines.append("achieved = algorithmic bytes / average duration = %.0f GB/s = %.1f %% of the "
+                     "8000 GB/s HBM peak" % (alg / avg / 1e3, alg / avg / 1e3 / 80.0))
+        with open(os.path.join(directory, fname), "w") as fh:
+            fh.write("\n".join(lines) + "\n")
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--stats", required=True)
     ap.add_argument("--fetch")
     ap.add_argument("--write")
+    ap.add_argument("--profiles-dir", help="also write one summary file per workload there")
     args = ap.parse_args()
     stats = kernel_stats(args.stats)
     fetch = counter_avg(args.fetch, "FETCH_SIZE") if args.fetch else {}
@@ -72,6 +133,8 @@ def main():
             fs = f * fscale / 1024 if fscale else float("nan")
             ws = w * wscale / 1024 if wscale else float("nan")
             print("%-46s %14.1f %14.1f %14.1f %14.1f" % (name[:46], f, w, fs, ws))
+    if args.profiles_dir:
+        write_profiles(args.profiles_dir, stats, fetch, write, fscale, wscale)
 
 
 if __name__ == "__main__":
