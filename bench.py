@@ -33,11 +33,11 @@ MEASURED_TRAFFIC_BYTES = {
     "alltoall_1GiB": None,              # not profiled
 }
 
-# put_block launch shape: each block moves a contiguous 16 KiB slice (short-lived blocks keep the
+# put_block launch shape: each block moves a contiguous 4 KiB slice (short-lived blocks keep the
 # set of addresses in flight narrow, which is what HBM serves fastest)
 PUT_BYTES = 1 << 28
-PUT_BLOCKS_PER_PE = 16384
-PUT_THREADS = 512
+PUT_BLOCKS_PER_PE = 65536
+PUT_THREADS = 128
 
 
 def _time_steps(fn, steps, warmup, hip):

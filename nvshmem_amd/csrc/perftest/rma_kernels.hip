@@ -30,11 +30,21 @@ __device__ __forceinline__ bool slice_of(size_t bytes, size_t parts, size_t idx,
     return true;
 }
 
+// `per_block` = bytes / gridDim.x, divided once on the host: a block that moves a few KiB should
+// not spend its time in a 64-bit division.
 template <int SCOPE, bool GET>
-__global__ void ring_rma_kernel(char *dest, const char *src, size_t bytes) {
-    const int peer = (nvshmem_my_pe() + 1) % nvshmem_n_pes();
+__global__ void ring_rma_kernel(char *dest, const char *src, size_t bytes, size_t per_block) {
+    const int me = nvshmem_my_pe();
+    const int peer = (me + 1 == nvshmem_n_pes()) ? 0 : me + 1;
     size_t off, len;
-    if (!slice_of(bytes, gridDim.x, blockIdx.x, &off, &len)) return;
+    if (per_block == 0) {  // fewer bytes than blocks: block 0 moves everything
+        if (blockIdx.x != 0) return;
+        off = 0;
+        len = bytes;
+    } else {
+        off = (size_t)blockIdx.x * per_block;
+        len = (blockIdx.x == gridDim.x - 1) ? bytes - off : per_block;
+    }
     if (SCOPE == NVSHMEM_PERFTEST_SCOPE_BLOCK) {
         if (GET) nvshmemx_getmem_block(dest + off, src + off, len, peer);
         else nvshmemx_putmem_block(dest + off, src + off, len, peer);
@@ -139,10 +149,13 @@ template <int SCOPE>
 int launch_ring(bool is_get, char *dest, const char *src, size_t bytes, int blocks, int threads,
                 hipStream_t stream) {
     const dim3 grid((unsigned)blocks, 1, (unsigned)nvshmem_n_pes());
+    const size_t per_block = bytes / (size_t)blocks;
     if (is_get)
-        hipLaunchKernelGGL((ring_rma_kernel<SCOPE, true>), grid, dim3(threads), 0, stream, dest, src, bytes);
+        hipLaunchKernelGGL((ring_rma_kernel<SCOPE, true>), grid, dim3(threads), 0, stream, dest, src, bytes,
+                           per_block);
     else
-        hipLaunchKernelGGL((ring_rma_kernel<SCOPE, false>), grid, dim3(threads), 0, stream, dest, src, bytes);
+        hipLaunchKernelGGL((ring_rma_kernel<SCOPE, false>), grid, dim3(threads), 0, stream, dest, src, bytes,
+                           per_block);
     return perftest::launch_status("ring_rma");
 }
 

@@ -39,7 +39,7 @@ def main():
     src = rt.calloc(S, 1)
     dst = rt.calloc(S, 1)
     for _ in range(args.iters):
-        assert perf.nvshmem_perftest_ring_rma(dst, src, S, 16384, 512, N.SCOPE_BLOCK, 0, 1, None) == 0
+        assert perf.nvshmem_perftest_ring_rma(dst, src, S, 65536, 128, N.SCOPE_BLOCK, 0, 1, None) == 0
     hip.synchronize()
     rt.finalize()
 
