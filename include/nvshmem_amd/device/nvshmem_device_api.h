@@ -128,6 +128,12 @@ NVSHMEMI_REPT_FOR_STANDARD_RMA_TYPES(NVSHMEMI_STAMP_TYPED_RMA)
 #undef NVSHMEMI_STAMP_TYPED_RMA_SCOPE
 
 /* ---- sized RMA put8..put128: nelems elements of BITS/8 bytes ---- */
+template <int BYTES> struct nvshmemi_amd_sized;
+template <> struct nvshmemi_amd_sized<1> { typedef uint8_t type; };
+template <> struct nvshmemi_amd_sized<2> { typedef uint16_t type; };
+template <> struct nvshmemi_amd_sized<4> { typedef uint32_t type; };
+template <> struct nvshmemi_amd_sized<8> { typedef uint64_t type; };
+template <> struct nvshmemi_amd_sized<16> { typedef nvshmemi_v4u type; };
 #define NVSHMEMI_STAMP_SIZED_RMA_SCOPE(BITS, BYTES, PFX, SFX, SC)                                 \
     NVSHMEMI_DEV void PFX##_put##BITS##SFX(void *dest, const void *source, size_t nelems,         \
                                            int pe) {                                              \
@@ -144,6 +150,18 @@ NVSHMEMI_REPT_FOR_STANDARD_RMA_TYPES(NVSHMEMI_STAMP_TYPED_RMA)
     NVSHMEMI_DEV void PFX##_get##BITS##_nbi##SFX(void *dest, const void *source, size_t nelems,   \
                                                  int pe) {                                        \
         nvshmemi_get<char, SC>((char *)dest, (const char *)source, nelems * BYTES, pe);           \
+    }                                                                                             \
+    NVSHMEMI_DEV void PFX##_iput##BITS##SFX(void *dest, const void *source, ptrdiff_t dst,        \
+                                            ptrdiff_t sst, size_t nelems, int pe) {               \
+        nvshmemi_iput<nvshmemi_amd_sized<BYTES>::type, SC>(                                       \
+            (nvshmemi_amd_sized<BYTES>::type *)dest,                                              \
+            (const nvshmemi_amd_sized<BYTES>::type *)source, dst, sst, nelems, pe);               \
+    }                                                                                             \
+    NVSHMEMI_DEV void PFX##_iget##BITS##SFX(void *dest, const void *source, ptrdiff_t dst,        \
+                                            ptrdiff_t sst, size_t nelems, int pe) {               \
+        nvshmemi_iget<nvshmemi_amd_sized<BYTES>::type, SC>(                                       \
+            (nvshmemi_amd_sized<BYTES>::type *)dest,                                              \
+            (const nvshmemi_amd_sized<BYTES>::type *)source, dst, sst, nelems, pe);               \
     }                                                                                             \
     NVSHMEMI_DEV void PFX##_put##BITS##_signal##SFX(void *dest, const void *source,               \
                                                     size_t nelems, uint64_t *sig_addr,            \

@@ -102,17 +102,108 @@ NVSHMEMI_HOST_ONLY void nvshmemx_signal_wait_until_on_stream(uint64_t *sig_addr,
                                                              uint64_t cmp_value,
                                                              nvshmemx_stream_t stream);
 
+/* typed forms: nvshmem_api.h:199-306 (blocking), nvshmemx_api.h:94-248 (on stream).  p takes the
+ * value in the call, g returns it (and therefore waits for the stream).  iput / iget: element i of
+ * the source at stride sst goes to element i*dst of the destination; strides are at least 1. */
 #define NVSHMEMI_DECL_TYPED_RMA_HOST(NAME, TYPE, TAG)                                             \
     NVSHMEMI_HOST_ONLY void nvshmem_##NAME##_put(TYPE *dest, const TYPE *source, size_t nelems,   \
                                                  int pe);                                         \
     NVSHMEMI_HOST_ONLY void nvshmem_##NAME##_get(TYPE *dest, const TYPE *source, size_t nelems,   \
                                                  int pe);                                         \
+    NVSHMEMI_HOST_ONLY void nvshmem_##NAME##_put_nbi(TYPE *dest, const TYPE *source,              \
+                                                     size_t nelems, int pe);                      \
+    NVSHMEMI_HOST_ONLY void nvshmem_##NAME##_get_nbi(TYPE *dest, const TYPE *source,              \
+                                                     size_t nelems, int pe);                      \
+    NVSHMEMI_HOST_ONLY void nvshmem_##NAME##_p(TYPE *dest, const TYPE value, int pe);             \
+    NVSHMEMI_HOST_ONLY TYPE nvshmem_##NAME##_g(const TYPE *src, int pe);                          \
+    NVSHMEMI_HOST_ONLY void nvshmem_##NAME##_iput(TYPE *dest, const TYPE *source, ptrdiff_t dst,  \
+                                                  ptrdiff_t sst, size_t nelems, int pe);          \
+    NVSHMEMI_HOST_ONLY void nvshmem_##NAME##_iget(TYPE *dest, const TYPE *source, ptrdiff_t dst,  \
+                                                  ptrdiff_t sst, size_t nelems, int pe);          \
     NVSHMEMI_HOST_ONLY void nvshmemx_##NAME##_put_on_stream(                                      \
         TYPE *dest, const TYPE *source, size_t nelems, int pe, nvshmemx_stream_t stream);         \
     NVSHMEMI_HOST_ONLY void nvshmemx_##NAME##_get_on_stream(                                      \
-        TYPE *dest, const TYPE *source, size_t nelems, int pe, nvshmemx_stream_t stream);
+        TYPE *dest, const TYPE *source, size_t nelems, int pe, nvshmemx_stream_t stream);         \
+    NVSHMEMI_HOST_ONLY void nvshmemx_##NAME##_put_nbi_on_stream(                                  \
+        TYPE *dest, const TYPE *source, size_t nelems, int pe, nvshmemx_stream_t stream);         \
+    NVSHMEMI_HOST_ONLY void nvshmemx_##NAME##_get_nbi_on_stream(                                  \
+        TYPE *dest, const TYPE *source, size_t nelems, int pe, nvshmemx_stream_t stream);         \
+    NVSHMEMI_HOST_ONLY void nvshmemx_##NAME##_p_on_stream(TYPE *dest, const TYPE value, int pe,   \
+                                                          nvshmemx_stream_t stream);              \
+    NVSHMEMI_HOST_ONLY TYPE nvshmemx_##NAME##_g_on_stream(const TYPE *src, int pe,                \
+                                                          nvshmemx_stream_t stream);              \
+    NVSHMEMI_HOST_ONLY void nvshmemx_##NAME##_iput_on_stream(                                     \
+        TYPE *dest, const TYPE *source, ptrdiff_t dst, ptrdiff_t sst, size_t nelems, int pe,      \
+        nvshmemx_stream_t stream);                                                                \
+    NVSHMEMI_HOST_ONLY void nvshmemx_##NAME##_iget_on_stream(                                     \
+        TYPE *dest, const TYPE *source, ptrdiff_t dst, ptrdiff_t sst, size_t nelems, int pe,      \
+        nvshmemx_stream_t stream);                                                                \
+    NVSHMEMI_HOST_ONLY void nvshmemx_##NAME##_put_signal_on_stream(                               \
+        TYPE *dest, const TYPE *source, size_t nelems, uint64_t *sig_addr, uint64_t signal,       \
+        int sig_op, int pe, nvshmemx_stream_t stream);                                            \
+    NVSHMEMI_HOST_ONLY void nvshmemx_##NAME##_put_signal_nbi_on_stream(                           \
+        TYPE *dest, const TYPE *source, size_t nelems, uint64_t *sig_addr, uint64_t signal,       \
+        int sig_op, int pe, nvshmemx_stream_t stream);
 NVSHMEMI_REPT_FOR_STANDARD_RMA_TYPES(NVSHMEMI_DECL_TYPED_RMA_HOST)
 #undef NVSHMEMI_DECL_TYPED_RMA_HOST
+
+/* sized forms put8 .. put128: nelems elements of BITS/8 bytes (nvshmem_api.h:214-306,
+ * nvshmemx_api.h:106-248) */
+#define NVSHMEMI_DECL_SIZED_RMA_HOST(BITS, BYTES)                                                 \
+    NVSHMEMI_HOST_ONLY void nvshmem_put##BITS(void *dest, const void *source, size_t nelems,      \
+                                              int pe);                                            \
+    NVSHMEMI_HOST_ONLY void nvshmem_get##BITS(void *dest, const void *source, size_t nelems,      \
+                                              int pe);                                            \
+    NVSHMEMI_HOST_ONLY void nvshmem_put##BITS##_nbi(void *dest, const void *source,               \
+                                                    size_t nelems, int pe);                       \
+    NVSHMEMI_HOST_ONLY void nvshmem_get##BITS##_nbi(void *dest, const void *source,               \
+                                                    size_t nelems, int pe);                       \
+    NVSHMEMI_HOST_ONLY void nvshmem_iput##BITS(void *dest, const void *source, ptrdiff_t dst,     \
+                                               ptrdiff_t sst, size_t nelems, int pe);             \
+    NVSHMEMI_HOST_ONLY void nvshmem_iget##BITS(void *dest, const void *source, ptrdiff_t dst,     \
+                                               ptrdiff_t sst, size_t nelems, int pe);             \
+    NVSHMEMI_HOST_ONLY void nvshmemx_put##BITS##_on_stream(void *dest, const void *source,        \
+                                                           size_t nelems, int pe,                 \
+                                                           nvshmemx_stream_t stream);             \
+    NVSHMEMI_HOST_ONLY void nvshmemx_get##BITS##_on_stream(void *dest, const void *source,        \
+                                                           size_t nelems, int pe,                 \
+                                                           nvshmemx_stream_t stream);             \
+    NVSHMEMI_HOST_ONLY void nvshmemx_put##BITS##_nbi_on_stream(void *dest, const void *source,    \
+                                                               size_t nelems, int pe,             \
+                                                               nvshmemx_stream_t stream);         \
+    NVSHMEMI_HOST_ONLY void nvshmemx_get##BITS##_nbi_on_stream(void *dest, const void *source,    \
+                                                               size_t nelems, int pe,             \
+                                                               nvshmemx_stream_t stream);         \
+    NVSHMEMI_HOST_ONLY void nvshmemx_iput##BITS##_on_stream(void *dest, const void *source,       \
+                                                            ptrdiff_t dst, ptrdiff_t sst,         \
+                                                            size_t nelems, int pe,                \
+                                                            nvshmemx_stream_t stream);            \
+    NVSHMEMI_HOST_ONLY void nvshmemx_iget##BITS##_on_stream(void *dest, const void *source,       \
+                                                            ptrdiff_t dst, ptrdiff_t sst,         \
+                                                            size_t nelems, int pe,                \
+                                                            nvshmemx_stream_t stream);            \
+    NVSHMEMI_HOST_ONLY void nvshmemx_put##BITS##_signal_on_stream(                                \
+        void *dest, const void *source, size_t nelems, uint64_t *sig_addr, uint64_t signal,       \
+        int sig_op, int pe, nvshmemx_stream_t stream);                                            \
+    NVSHMEMI_HOST_ONLY void nvshmemx_put##BITS##_signal_nbi_on_stream(                            \
+        void *dest, const void *source, size_t nelems, uint64_t *sig_addr, uint64_t signal,       \
+        int sig_op, int pe, nvshmemx_stream_t stream);
+NVSHMEMI_REPT_FOR_SIZES(NVSHMEMI_DECL_SIZED_RMA_HOST)
+#undef NVSHMEMI_DECL_SIZED_RMA_HOST
+
+/* typed waits on a stream (nvshmemx_api.h:255-273): a one-block kernel that spins (bounded by the
+ * spin limit) on the local word(s); `status` is device-accessible or NULL.  nvshmem_signal_fetch
+ * (nvshmem_api.h:343) reads the calling PE's signal word. */
+#define NVSHMEMI_DECL_WAIT_ON_STREAM(NAME, TYPE)                                                  \
+    NVSHMEMI_HOST_ONLY void nvshmemx_##NAME##_wait_until_on_stream(TYPE *ivar, int cmp,           \
+                                                                   TYPE cmp_value,                \
+                                                                   nvshmemx_stream_t stream);     \
+    NVSHMEMI_HOST_ONLY void nvshmemx_##NAME##_wait_until_all_on_stream(                           \
+        TYPE *ivars, size_t nelems, const int *status, int cmp, TYPE cmp_value,                   \
+        nvshmemx_stream_t stream);
+NVSHMEMI_REPT_FOR_WAIT_TYPES(NVSHMEMI_DECL_WAIT_ON_STREAM)
+#undef NVSHMEMI_DECL_WAIT_ON_STREAM
+NVSHMEMI_HOST_ONLY uint64_t nvshmem_signal_fetch(uint64_t *sig_addr);
 
 /* ---- collectives: src/include/host/nvshmem_coll_api.h:27-80, nvshmemx_coll_api.h:27-80 ----
  * One call serves every PE of the team.  dest and src are canonical symmetric addresses.

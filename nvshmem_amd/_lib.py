@@ -133,7 +133,7 @@ def load_perftest():
 def declared_symbols(header_paths=None):
     """Names of every function the public headers declare as host entry points (macro-stamped ones
     expanded), for the export check."""
-    from .host import RMA_TYPES, REDUCE_TYPES_BITWISE, REDUCE_TYPES_STANDARD
+    from .host import RMA_TYPES, REDUCE_TYPES_BITWISE, REDUCE_TYPES_STANDARD, WAIT_TYPES
     names = set()
     text = open(os.path.join(INCLUDE, "nvshmem_amd", "nvshmem_host_api.h")).read()
     # drop the macro bodies, then collect plain declarations
@@ -141,10 +141,19 @@ def declared_symbols(header_paths=None):
     for m in re.finditer(r"NVSHMEMI_HOST_ONLY\s+[\w\s\*]+?\b(nvshmem\w+)\s*\(", plain):
         names.add(m.group(1))
     for t in RMA_TYPES:
-        names.update({"nvshmem_%s_put" % t, "nvshmem_%s_get" % t, "nvshmemx_%s_put_on_stream" % t,
-                      "nvshmemx_%s_get_on_stream" % t, "nvshmem_%s_alltoall" % t,
-                      "nvshmem_%s_fcollect" % t, "nvshmemx_%s_alltoall_on_stream" % t,
-                      "nvshmemx_%s_fcollect_on_stream" % t})
+        for form in ("put", "get", "put_nbi", "get_nbi", "p", "g", "iput", "iget"):
+            names.add("nvshmem_%s_%s" % (t, form))
+            names.add("nvshmemx_%s_%s_on_stream" % (t, form))
+        names.update({"nvshmemx_%s_put_signal_on_stream" % t, "nvshmemx_%s_put_signal_nbi_on_stream" % t,
+                      "nvshmem_%s_alltoall" % t, "nvshmem_%s_fcollect" % t,
+                      "nvshmemx_%s_alltoall_on_stream" % t, "nvshmemx_%s_fcollect_on_stream" % t})
+    for bits in (8, 16, 32, 64, 128):
+        for form in ("put%d", "get%d", "put%d_nbi", "get%d_nbi", "iput%d", "iget%d"):
+            names.add("nvshmem_" + form % bits)
+            names.add("nvshmemx_" + form % bits + "_on_stream")
+        names.update({"nvshmemx_put%d_signal_on_stream" % bits, "nvshmemx_put%d_signal_nbi_on_stream" % bits})
+    for t in WAIT_TYPES:
+        names.update({"nvshmemx_%s_wait_until_on_stream" % t, "nvshmemx_%s_wait_until_all_on_stream" % t})
     for op in ("and", "or", "xor"):
         for t in REDUCE_TYPES_BITWISE:
             names.update({"nvshmem_%s_%s_reduce" % (t, op), "nvshmemx_%s_%s_reduce_on_stream" % (t, op)})

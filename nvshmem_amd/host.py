@@ -31,6 +31,8 @@ RMA_TYPES = {
     "uint32": (np.uint32, "u32"), "uint64": (np.uint64, "u64"), "size": (np.uint64, "u64"),
     "ptrdiff": (np.int64, "i64"),
 }
+WAIT_TYPES = ["short", "int", "long", "longlong", "ushort", "uint", "ulong", "ulonglong", "int32",
+              "int64", "uint32", "uint64", "size", "ptrdiff"]
 REDUCE_TYPES_BITWISE = ["uchar", "ushort", "uint", "ulong", "ulonglong", "int8", "int16", "int32",
                         "int64", "uint8", "uint16", "uint32", "uint64", "size"]
 REDUCE_TYPES_STANDARD = REDUCE_TYPES_BITWISE + ["char", "schar", "short", "int", "long", "longlong",

@@ -1,0 +1,106 @@
+"""GPU parity of the host-initiated typed / sized / strided RMA forms and the typed waits on a
+stream.  Expected values follow the operator definitions (strided forms: element i of the source
+at stride sst goes to element i*dst of the destination)."""
+import ctypes as C
+
+import numpy as np
+import pytest
+
+import nvshmem_amd as N
+import oracle_lib as O
+from gpu_util import note, runtime
+from nvshmem_amd import hip
+
+pytestmark = pytest.mark.gpu
+NPES = 4
+vp, sz, pd, i32 = C.c_void_p, C.c_size_t, C.c_ssize_t, C.c_int
+
+
+def _fn(lib, name, restype, argtypes):
+    f = getattr(lib, name)
+    f.restype, f.argtypes = restype, argtypes
+    return f
+
+
+def test_host_typed_sized_strided_rma_and_waits():
+    with runtime(NPES, 16 << 20) as rt:
+        lib = rt.lib
+        n = 4096
+        a = rt.malloc(n); b = rt.malloc(n)
+        A = O.fill_all("bytes", NPES, n, 55)
+        rt.upload_all(a, A)
+        s = hip.Stream()
+
+        def reset():
+            rt.fill(b, 0xEE, n)
+
+        # sized put / get, blocking and on a stream
+        reset()
+        note("put64 / get16_on_stream / put128_nbi")
+        _fn(lib, "nvshmem_put64", None, [vp, vp, sz, i32])(b, a, 5, 2)            # PE0.a -> PE2.b, 40 B
+        assert np.array_equal(rt.download(b, 2, (40,), np.uint8), A[0, :40])
+        _fn(lib, "nvshmemx_get16_on_stream", None, [vp, vp, sz, i32, vp])(b + 64, a + 64, 7, 3, s.ptr)
+        _fn(lib, "nvshmemx_put128_nbi_on_stream", None, [vp, vp, sz, i32, vp])(b + 128, a + 128, 2, 1, s.ptr)
+        s.synchronize()
+        assert np.array_equal(rt.download(b, 0, (14,), np.uint8, 64), A[3, 64:78])
+        assert np.array_equal(rt.download(b, 1, (32,), np.uint8, 128), A[0, 128:160])
+
+        # strided: iput / iget, typed and sized
+        reset()
+        note("int32_iput / iget64_on_stream")
+        _fn(lib, "nvshmem_int32_iput", None, [vp, vp, pd, pd, sz, i32])(b, a, 3, 2, 10, 1)
+        got = rt.download(b, 1, (n,), np.uint8).view(np.int32)
+        src = A[0].view(np.int32)
+        want = np.full(n // 4, 0xEEEEEEEE, np.uint32).view(np.int32)
+        for i in range(10):
+            want[i * 3] = src[i * 2]
+        assert np.array_equal(got, want)
+        _fn(lib, "nvshmemx_iget64_on_stream", None, [vp, vp, pd, pd, sz, i32, vp])(b + 1024, a + 1024, 2, 5, 6, 3, s.ptr)
+        s.synchronize()
+        got = rt.download(b, 0, (n - 1024,), np.uint8, 1024).view(np.int64)
+        src = A[3, 1024:].view(np.int64)
+        for i in range(6):
+            assert got[i * 2] == src[i * 5]
+            assert got[i * 2 + 1] == np.int64(-0x1111111111111112)          # 0xEE.. untouched
+        # a stride below 1 is refused
+        _fn(lib, "nvshmem_iput8", None, [vp, vp, pd, pd, sz, i32])(b, a, 0, 1, 4, 1)
+        assert b"stride" in lib.nvshmemx_amd_last_error()
+
+        # scalar p / g
+        note("float_p / int64_g / bfloat16 p,g")
+        _fn(lib, "nvshmem_float_p", None, [vp, C.c_float, i32])(b + 2048, 3.25, 2)
+        assert rt.download(b, 2, (1,), np.float32, 2048)[0] == np.float32(3.25)
+        g = _fn(lib, "nvshmem_int64_g", C.c_int64, [vp, i32])
+        assert g(a + 512, 3) == A[3, 512:520].view(np.int64)[0]
+        _fn(lib, "nvshmemx_uint16_p_on_stream", None, [vp, C.c_uint16, i32, vp])(b + 2060, 0xBEEF, 1, s.ptr)
+        s.synchronize()
+        assert rt.download(b, 1, (1,), np.uint16, 2060)[0] == 0xBEEF
+        gd = _fn(lib, "nvshmemx_double_g_on_stream", C.c_double, [vp, i32, vp])
+        assert np.float64(gd(a + 256, 1, s.ptr)).view(np.int64) == A[1, 256:264].view(np.int64)[0]
+
+        # typed put with signal on a stream, signal_fetch, typed waits
+        note("double_put_signal_on_stream / signal_fetch / int_wait_until_on_stream")
+        sig = rt.calloc(2, 8)
+        _fn(lib, "nvshmemx_double_put_signal_on_stream", None,
+            [vp, vp, sz, vp, C.c_uint64, i32, i32, vp])(b + 3000 + 8, a + 3000 + 8, 4, sig, 9, N.SIGNAL_ADD, 0, s.ptr)
+        s.synchronize()
+        assert _fn(lib, "nvshmem_signal_fetch", C.c_uint64, [vp])(sig) == 9
+        assert np.array_equal(rt.download(b, 0, (32,), np.uint8, 3008), A[0, 3008:3040])
+        flags = rt.calloc(4, 4)
+        rt.upload(flags, 0, np.array([-5, 7, 7, 7], np.int32))
+        status = rt.malloc(16)
+        rt.upload(status, 0, np.array([1, 0, 0, 0], np.int32))          # element 0 is excluded
+        _fn(lib, "nvshmemx_int_wait_until_on_stream", None, [vp, i32, i32, vp])(flags, N.CMP["LT"], 0, s.ptr)
+        _fn(lib, "nvshmemx_int_wait_until_all_on_stream", None,
+            [vp, sz, vp, i32, i32, vp])(flags, 4, status, N.CMP["EQ"], 7, s.ptr)
+        _fn(lib, "nvshmemx_uint64_wait_until_on_stream", None, [vp, i32, C.c_uint64, vp])(sig, N.CMP["GE"], 9, s.ptr)
+        s.synchronize()
+        assert rt.read_timeout(0)[0] == 0
+        # signed comparison is really signed: -5 < 0 held above; an unsigned type must not see it so
+        rt.lib.nvshmemx_amd_set_spin_limit(100)
+        _fn(lib, "nvshmemx_uint_wait_until_on_stream", None, [vp, i32, C.c_uint, vp])(flags, N.CMP["LT"], 5, s.ptr)
+        s.synchronize()
+        rt.lib.nvshmemx_amd_set_spin_limit(1 << 22)
+        flag, rec = rt.read_timeout(0)
+        assert flag == 1 and rec[2] == 0xFFFFFFFB and rec[3] == 5      # found (uint)-5, expected 5
+        s.destroy()
