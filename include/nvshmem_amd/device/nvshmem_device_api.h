@@ -227,6 +227,10 @@ NVSHMEMI_REPT_FOR_WAIT_TYPES(NVSHMEMI_STAMP_WAIT)
     NVSHMEMI_DEV int PFX##_##NAME##_fcollect##SFX(nvshmem_team_t team, TYPE *dest,                \
                                                   const TYPE *src, size_t nelems) {               \
         return nvshmemi_fcollect_threadgroup<TYPE, SC>(team, dest, src, nelems);                  \
+    }                                                                                             \
+    NVSHMEMI_DEV int PFX##_##NAME##_broadcast##SFX(nvshmem_team_t team, TYPE *dest,               \
+                                                   const TYPE *src, size_t nelems, int PE_root) { \
+        return nvshmemi_broadcast_threadgroup<TYPE, SC>(team, dest, src, nelems, PE_root);        \
     }
 #define NVSHMEMI_STAMP_COLL(NAME, TYPE, TAG)                                                      \
     NVSHMEMI_STAMP_COLL_SCOPE(NAME, TYPE, nvshmem, , NVSHMEMI_THREADGROUP_THREAD)                 \
@@ -246,6 +250,11 @@ NVSHMEMI_REPT_FOR_STANDARD_RMA_TYPES(NVSHMEMI_STAMP_COLL)
                                             size_t nelems) {                                      \
         return nvshmemi_fcollect_threadgroup<char, SC>(team, (char *)dest, (const char *)src,     \
                                                        nelems);                                   \
+    }                                                                                             \
+    NVSHMEMI_DEV int PFX##_broadcastmem##SFX(nvshmem_team_t team, void *dest, const void *src,    \
+                                             size_t nelems, int PE_root) {                        \
+        return nvshmemi_broadcast_threadgroup<char, SC>(team, (char *)dest, (const char *)src,    \
+                                                        nelems, PE_root);                         \
     }
 NVSHMEMI_STAMP_MEM_COLL(nvshmem, , NVSHMEMI_THREADGROUP_THREAD)
 NVSHMEMI_STAMP_MEM_COLL(nvshmemx, _warp, NVSHMEMI_THREADGROUP_WARP)
@@ -267,6 +276,26 @@ NVSHMEMI_STAMP_MEM_COLL(nvshmemx, _block, NVSHMEMI_THREADGROUP_BLOCK)
                                                            const TYPE *src, size_t nreduce) {     \
         return nvshmemi_reduce_threadgroup<TYPE, NVSHMEMI_OP_##OP, NVSHMEMI_THREADGROUP_BLOCK>(   \
             team, dest, src, nreduce);                                                            \
+    }                                                                                             \
+    NVSHMEMI_DEV int nvshmem_##NAME##_##OP##_reducescatter(nvshmem_team_t team, TYPE *dest,       \
+                                                           const TYPE *src, size_t nreduce) {     \
+        return nvshmemi_reducescatter_threadgroup<TYPE, NVSHMEMI_OP_##OP,                         \
+                                                  NVSHMEMI_THREADGROUP_THREAD>(team, dest, src,   \
+                                                                               nreduce);          \
+    }                                                                                             \
+    NVSHMEMI_DEV int nvshmemx_##NAME##_##OP##_reducescatter_warp(nvshmem_team_t team, TYPE *dest, \
+                                                                 const TYPE *src,                 \
+                                                                 size_t nreduce) {                \
+        return nvshmemi_reducescatter_threadgroup<TYPE, NVSHMEMI_OP_##OP,                         \
+                                                  NVSHMEMI_THREADGROUP_WARP>(team, dest, src,     \
+                                                                             nreduce);            \
+    }                                                                                             \
+    NVSHMEMI_DEV int nvshmemx_##NAME##_##OP##_reducescatter_block(nvshmem_team_t team,            \
+                                                                  TYPE *dest, const TYPE *src,    \
+                                                                  size_t nreduce) {               \
+        return nvshmemi_reducescatter_threadgroup<TYPE, NVSHMEMI_OP_##OP,                         \
+                                                  NVSHMEMI_THREADGROUP_BLOCK>(team, dest, src,    \
+                                                                              nreduce);           \
     }
 NVSHMEMI_REPT_FOR_ALL_REDUCE_TYPES_AND_OPS(NVSHMEMI_STAMP_REDUCE)
 #undef NVSHMEMI_STAMP_REDUCE

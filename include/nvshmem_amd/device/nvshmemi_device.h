@@ -627,4 +627,69 @@ NVSHMEMI_DEVICE_INLINE int nvshmemi_alltoall_threadgroup(nvshmem_team_t team, T 
     return 0;
 }
 
+/* Broadcast (reference coll/broadcast.cuh:298-337, the put-to-all algorithm): the root's thread
+ * group copies its source into every PE's dest, its own included unless dest == source; the closing
+ * barrier completes the copies and tells the receivers. */
+template <typename T, int SCOPE>
+NVSHMEMI_DEVICE_INLINE int nvshmemi_broadcast_threadgroup(nvshmem_team_t team, T *dest,
+                                                          const T *source, size_t nelems,
+                                                          int PE_root) {
+    (void)team;
+    const int me = nvshmemi_amd_my_pe();
+    const int npes = nvshmemi_device_state_d.npes;
+    if (me == PE_root) {
+        const void *from = nvshmemi_amd_local(source);
+        for (int ii = 0; ii < npes; ++ii) {
+            const int peer = (me + ii) % npes;
+            void *to = nvshmemi_amd_remote(dest, peer);
+            if (to != from) nvshmemi_memcpy_threadgroup<SCOPE>(to, from, nelems * sizeof(T));
+        }
+    }
+    nvshmemi_barrier_threadgroup<SCOPE>();
+    return 0;
+}
+
+/* Reducescatter (reference coll/reducescatter.cuh:36-90): PE `me` folds block `me` (nreduce
+ * elements) of every PE's source into its own dest, in the order acc = op(x0, x1);
+ * acc = op(acc, x_p).  dest must not overlap source: other PEs read the blocks of this PE's source
+ * while it writes its dest. */
+template <typename T, int OP, int SCOPE>
+NVSHMEMI_DEVICE_INLINE int nvshmemi_reducescatter_threadgroup(nvshmem_team_t team, T *dest,
+                                                              const T *source, size_t nreduce) {
+    (void)team;
+    constexpr size_t VEC = 16 / sizeof(T);
+    struct alignas(16) pack_t { T e[VEC]; };
+    const int me = nvshmemi_amd_my_pe();
+    const int npes = nvshmemi_device_state_d.npes;
+    const size_t tid = (size_t)nvshmemi_thread_id_in_threadgroup<SCOPE>();
+    const size_t nthr = (size_t)nvshmemi_threadgroup_size<SCOPE>();
+    /* every PE's source is complete and visible before anyone reads it */
+    nvshmemi_barrier_threadgroup<SCOPE>();
+    const T *src0 = reinterpret_cast<const T *>(nvshmemi_amd_remote(source, 0)) + (size_t)me * nreduce;
+    T *dst = reinterpret_cast<T *>(nvshmemi_amd_remote(dest, me));
+    const size_t pe_stride = (size_t)(nvshmemi_device_state_d.heap_size / sizeof(T));
+    size_t i = tid;
+    if ((((uintptr_t)src0 | (uintptr_t)dst) & 15) == 0) {
+        const size_t nvec = nreduce / VEC;
+        for (size_t v = tid; v < nvec; v += nthr) {
+            pack_t acc = *reinterpret_cast<const pack_t *>(src0 + v * VEC);
+            for (int pe = 1; pe < npes; ++pe) {
+                const pack_t x = *reinterpret_cast<const pack_t *>(src0 + (size_t)pe * pe_stride + v * VEC);
+#pragma unroll
+                for (size_t k = 0; k < VEC; ++k) acc.e[k] = nvshmemi_amd_reduce_op<T, OP>(acc.e[k], x.e[k]);
+            }
+            *reinterpret_cast<pack_t *>(dst + v * VEC) = acc;
+        }
+        i = nvec * VEC + tid;
+    }
+    for (; i < nreduce; i += nthr) {
+        T acc = src0[i];
+        for (int pe = 1; pe < npes; ++pe)
+            acc = nvshmemi_amd_reduce_op<T, OP>(acc, src0[(size_t)pe * pe_stride + i]);
+        dst[i] = acc;
+    }
+    nvshmemi_barrier_threadgroup<SCOPE>();
+    return 0;
+}
+
 #endif

@@ -208,7 +208,12 @@ NVSHMEMI_HOST_ONLY uint64_t nvshmem_signal_fetch(uint64_t *sig_addr);
 /* ---- collectives: src/include/host/nvshmem_coll_api.h:27-80, nvshmemx_coll_api.h:27-80 ----
  * One call serves every PE of the team.  dest and src are canonical symmetric addresses.
  * alltoall: dest@j[i*nelems + k] = src@i[j*nelems + k];  fcollect: dest@j[i*nelems + k] = src@i[k];
- * reduce:   dest@j[k] = fold over PEs 0..n-1 in that order of src@i[k].  All return 0 on success. */
+ * reduce:   dest@j[k] = fold over PEs 0..n-1 in that order of src@i[k];
+ * broadcast (nvshmem_coll_api.h:46-54, nvshmemx_coll_api.h:43-52): dest@j[k] = src@PE_root[k] for
+ * every PE j of the team, the root included; dest == src is the in-place form;
+ * reducescatter (nvshmem_coll_api.h:82-96, nvshmemx_coll_api.h:80-96):
+ * dest@j[k] = fold over PEs i = 0..n-1 of src@i[j*nreduce + k]; dest must not overlap src.
+ * All return 0 on success. */
 #define NVSHMEMI_DECL_TYPED_COLL_HOST(NAME, TYPE, TAG)                                            \
     NVSHMEMI_HOST_ONLY int nvshmem_##NAME##_alltoall(nvshmem_team_t team, TYPE *dest,             \
                                                      const TYPE *src, size_t nelems);             \
@@ -217,7 +222,13 @@ NVSHMEMI_HOST_ONLY uint64_t nvshmem_signal_fetch(uint64_t *sig_addr);
     NVSHMEMI_HOST_ONLY int nvshmemx_##NAME##_alltoall_on_stream(                                  \
         nvshmem_team_t team, TYPE *dest, const TYPE *src, size_t nelems, nvshmemx_stream_t s);    \
     NVSHMEMI_HOST_ONLY int nvshmemx_##NAME##_fcollect_on_stream(                                  \
-        nvshmem_team_t team, TYPE *dest, const TYPE *src, size_t nelems, nvshmemx_stream_t s);
+        nvshmem_team_t team, TYPE *dest, const TYPE *src, size_t nelems, nvshmemx_stream_t s);    \
+    NVSHMEMI_HOST_ONLY int nvshmem_##NAME##_broadcast(nvshmem_team_t team, TYPE *dest,            \
+                                                      const TYPE *src, size_t nelems,             \
+                                                      int PE_root);                               \
+    NVSHMEMI_HOST_ONLY int nvshmemx_##NAME##_broadcast_on_stream(                                 \
+        nvshmem_team_t team, TYPE *dest, const TYPE *src, size_t nelems, int PE_root,             \
+        nvshmemx_stream_t s);
 NVSHMEMI_REPT_FOR_STANDARD_RMA_TYPES(NVSHMEMI_DECL_TYPED_COLL_HOST)
 #undef NVSHMEMI_DECL_TYPED_COLL_HOST
 
@@ -225,6 +236,11 @@ NVSHMEMI_HOST_ONLY int nvshmem_alltoallmem(nvshmem_team_t team, void *dest, cons
                                            size_t nelems);
 NVSHMEMI_HOST_ONLY int nvshmem_fcollectmem(nvshmem_team_t team, void *dest, const void *src,
                                            size_t nelems);
+NVSHMEMI_HOST_ONLY int nvshmem_broadcastmem(nvshmem_team_t team, void *dest, const void *src,
+                                            size_t nelems, int PE_root);
+NVSHMEMI_HOST_ONLY int nvshmemx_broadcastmem_on_stream(nvshmem_team_t team, void *dest,
+                                                       const void *src, size_t nelems,
+                                                       int PE_root, nvshmemx_stream_t stream);
 NVSHMEMI_HOST_ONLY int nvshmemx_alltoallmem_on_stream(nvshmem_team_t team, void *dest,
                                                       const void *src, size_t nelems,
                                                       nvshmemx_stream_t stream);
@@ -236,6 +252,10 @@ NVSHMEMI_HOST_ONLY int nvshmemx_fcollectmem_on_stream(nvshmem_team_t team, void 
     NVSHMEMI_HOST_ONLY int nvshmem_##NAME##_##OP##_reduce(nvshmem_team_t team, TYPE *dest,        \
                                                           const TYPE *src, size_t nreduce);       \
     NVSHMEMI_HOST_ONLY int nvshmemx_##NAME##_##OP##_reduce_on_stream(                             \
+        nvshmem_team_t team, TYPE *dest, const TYPE *src, size_t nreduce, nvshmemx_stream_t s);   \
+    NVSHMEMI_HOST_ONLY int nvshmem_##NAME##_##OP##_reducescatter(                                 \
+        nvshmem_team_t team, TYPE *dest, const TYPE *src, size_t nreduce);                        \
+    NVSHMEMI_HOST_ONLY int nvshmemx_##NAME##_##OP##_reducescatter_on_stream(                      \
         nvshmem_team_t team, TYPE *dest, const TYPE *src, size_t nreduce, nvshmemx_stream_t s);
 NVSHMEMI_REPT_FOR_ALL_REDUCE_TYPES_AND_OPS(NVSHMEMI_DECL_TYPED_REDUCE_HOST)
 #undef NVSHMEMI_DECL_TYPED_REDUCE_HOST

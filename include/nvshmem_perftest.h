@@ -88,6 +88,13 @@ int nvshmem_perftest_device_fcollect(void *dest, const void *src, size_t bytes, 
                                      int threads, void *stream);
 int nvshmem_perftest_device_alltoall(void *dest, const void *src, size_t bytes, int scope,
                                      int threads, void *stream);
+/* reducescatter: src holds npes blocks of nreduce elements, dest nreduce elements; supported pairs:
+ * (i32,sum) (f32,sum) (f32,max) (bf16,sum) (u64,xor).  broadcast: `bytes` from PE root's src into
+ * every PE's dest. */
+int nvshmem_perftest_device_reducescatter(int dtype, int op, void *dest, const void *src,
+                                          size_t nreduce, int scope, int threads, void *stream);
+int nvshmem_perftest_device_broadcast(void *dest, const void *src, size_t bytes, int root,
+                                      int scope, int threads, void *stream);
 /* `rounds` barriers; before round r each PE stores r into its `counter`, after the barrier it reads
  * every PE's counter and adds to its own errors[0] the number that are < r.  counter and errors
  * hold one uint64 each. */

@@ -68,6 +68,8 @@ def load():
         "nvshmem_fcollectmem": (i32, [i32, vp, vp, sz]),
         "nvshmemx_alltoallmem_on_stream": (i32, [i32, vp, vp, sz, vp]),
         "nvshmemx_fcollectmem_on_stream": (i32, [i32, vp, vp, sz, vp]),
+        "nvshmem_broadcastmem": (i32, [i32, vp, vp, sz, i32]),
+        "nvshmemx_broadcastmem_on_stream": (i32, [i32, vp, vp, sz, i32, vp]),
         "nvshmemx_amd_collective_launch": (i32, [vp] + [C.c_uint] * 6 + [vp, sz, vp]),
         "nvshmemx_amd_collective_launch_query_gridsize": (i32, [vp] + [C.c_uint] * 3 + [sz, C.POINTER(i32)]),
         "nvshmemx_amd_module_init": (i32, []),
@@ -91,11 +93,12 @@ def load():
     return lib
 
 
-def typed_coll(lib, name, on_stream=False):
-    """Typed collective entry point, e.g. nvshmem_float_sum_reduce / nvshmemx_int64_alltoall_on_stream."""
+def typed_coll(lib, name, on_stream=False, rooted=False):
+    """Typed collective entry point, e.g. nvshmem_float_sum_reduce / nvshmemx_int64_alltoall_on_stream;
+    rooted adds the PE_root argument of broadcast."""
     fn = getattr(lib, name)
     fn.restype = i32
-    fn.argtypes = [i32, vp, vp, sz] + ([vp] if on_stream else [])
+    fn.argtypes = [i32, vp, vp, sz] + ([i32] if rooted else []) + ([vp] if on_stream else [])
     return fn
 
 
@@ -115,6 +118,8 @@ def load_perftest():
         "nvshmem_perftest_ring_reduce": [vp, vp, sz, vp, sz, i32, i32, vp],
         "nvshmem_perftest_device_reduce": [i32, i32, vp, vp, sz, i32, i32, vp],
         "nvshmem_perftest_device_fcollect": [vp, vp, sz, i32, i32, vp],
+        "nvshmem_perftest_device_reducescatter": [i32, i32, vp, vp, sz, i32, i32, vp],
+        "nvshmem_perftest_device_broadcast": [vp, vp, sz, i32, i32, i32, vp],
         "nvshmem_perftest_device_alltoall": [vp, vp, sz, i32, i32, vp],
         "nvshmem_perftest_device_barrier": [vp, vp, i32, i32, i32, vp],
         "nvshmem_perftest_moe_dispatch": [vp, sz, vp, vp, vp, vp, vp, i32, i32, sz, i32, i32, vp],
@@ -146,7 +151,8 @@ def declared_symbols(header_paths=None):
             names.add("nvshmemx_%s_%s_on_stream" % (t, form))
         names.update({"nvshmemx_%s_put_signal_on_stream" % t, "nvshmemx_%s_put_signal_nbi_on_stream" % t,
                       "nvshmem_%s_alltoall" % t, "nvshmem_%s_fcollect" % t,
-                      "nvshmemx_%s_alltoall_on_stream" % t, "nvshmemx_%s_fcollect_on_stream" % t})
+                      "nvshmemx_%s_alltoall_on_stream" % t, "nvshmemx_%s_fcollect_on_stream" % t,
+                      "nvshmem_%s_broadcast" % t, "nvshmemx_%s_broadcast_on_stream" % t})
     for bits in (8, 16, 32, 64, 128):
         for form in ("put%d", "get%d", "put%d_nbi", "get%d_nbi", "iput%d", "iget%d"):
             names.add("nvshmem_" + form % bits)
@@ -156,10 +162,14 @@ def declared_symbols(header_paths=None):
         names.update({"nvshmemx_%s_wait_until_on_stream" % t, "nvshmemx_%s_wait_until_all_on_stream" % t})
     for op in ("and", "or", "xor"):
         for t in REDUCE_TYPES_BITWISE:
-            names.update({"nvshmem_%s_%s_reduce" % (t, op), "nvshmemx_%s_%s_reduce_on_stream" % (t, op)})
+            names.update({"nvshmem_%s_%s_reduce" % (t, op), "nvshmemx_%s_%s_reduce_on_stream" % (t, op),
+                          "nvshmem_%s_%s_reducescatter" % (t, op),
+                          "nvshmemx_%s_%s_reducescatter_on_stream" % (t, op)})
     for op in ("max", "min", "sum", "prod"):
         for t in REDUCE_TYPES_STANDARD:
-            names.update({"nvshmem_%s_%s_reduce" % (t, op), "nvshmemx_%s_%s_reduce_on_stream" % (t, op)})
+            names.update({"nvshmem_%s_%s_reduce" % (t, op), "nvshmemx_%s_%s_reduce_on_stream" % (t, op),
+                          "nvshmem_%s_%s_reducescatter" % (t, op),
+                          "nvshmemx_%s_%s_reducescatter_on_stream" % (t, op)})
     perf = open(os.path.join(INCLUDE, "nvshmem_perftest.h")).read()
     perf_names = set(re.findall(r"\bint\s+(nvshmem_perftest_\w+)\s*\(", perf))
     return names, perf_names

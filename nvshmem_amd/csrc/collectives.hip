@@ -11,6 +11,12 @@
 //   reduce    dest@q[k] = fold_{p = 0..n-1, in that order} src@p[k]      for every PE q
 //   fcollect  dest@q[p*nelems + k] = src@p[k]                            for every PE q
 //   alltoall  dest@q[p*nelems + k] = src@p[q*nelems + k]
+//   broadcast dest@q[k] = src@root[k]                                    for every PE q
+//   reducescatter  dest@q[k] = fold_{p = 0..n-1} src@p[q*nreduce + k]
+//
+// Reference counterparts of the last two: src/host/coll/broadcast/broadcast.cpp with
+// coll/broadcast.cuh:276-337, src/host/coll/reducescatter/reducescatter_on_stream.cpp with
+// coll/reducescatter.cuh:36-90.
 #include <cstdio>
 
 #include "nvshmem.h"
@@ -68,7 +74,7 @@ __device__ __forceinline__ void stream_store(char *p, nvshmemi_v4u v) {
 // last one.
 // ---------------------------------------------------------------------------------------------
 
-enum { kModeFcollect = 0, kModeAlltoall = 1 };
+enum { kModeFcollect = 0, kModeAlltoall = 1, kModeBroadcast = 2 };
 
 // Copies the vectors v0 + t + u*kCopyThreads (u < unroll) that fall inside [0, nvec); indices in front of
 // the segment wrap to huge unsigned values and are skipped the same way as those behind it.
@@ -102,7 +108,7 @@ __device__ __forceinline__ void copy_tile(char *__restrict__ dst, const char *__
 template <int MODE, int kCopyUnroll, bool NTL>
 __global__ __launch_bounds__(kCopyThreads) void segment_copy_kernel(char *base, uint32_t shift, int npes,
                                                                 uint64_t dst_off, uint64_t src_off,
-                                                                uint64_t seg_bytes) {
+                                                                uint64_t seg_bytes, int root) {
     const unsigned seg = blockIdx.y;
     const char *src;
     char *dst;
@@ -111,6 +117,11 @@ __global__ __launch_bounds__(kCopyThreads) void segment_copy_kernel(char *base, 
         // segment p: PE p's source -> slot p of every PE's destination
         src = base + ((uint64_t)seg << shift) + src_off;
         dst = base + dst_off + (uint64_t)seg * seg_bytes;
+        nrep = npes;
+    } else if (MODE == kModeBroadcast) {
+        // one segment: the root's source -> every PE's destination
+        src = base + ((uint64_t)root << shift) + src_off;
+        dst = base + dst_off;
         nrep = npes;
     } else {
         // segment (p, q): block q of PE p's source -> slot p of PE q's destination
@@ -144,7 +155,7 @@ __global__ __launch_bounds__(kCopyThreads) void segment_copy_kernel(char *base, 
     const char *s = src + head;
     char *d = dst + head;
     const bool aligned = (((uintptr_t)s) & 15) == 0;
-    if (MODE == kModeFcollect) {
+    if (MODE != kModeAlltoall) {
         if (aligned) copy_tile<true, true, kCopyUnroll, NTL>(d, s, v0, nvec_total, rep_stride, nrep);
         else copy_tile<false, true, kCopyUnroll, NTL>(d, s, v0, nvec_total, rep_stride, nrep);
     } else {
@@ -165,7 +176,16 @@ __global__ __launch_bounds__(kCopyThreads) void segment_copy_kernel(char *base, 
 // ---------------------------------------------------------------------------------------------
 // NPES > 0 fixes the team size at compile time (fold fully unrolled, one wavefront per PE);
 // NPES == 0 takes both from the arguments.
-template <typename T, int OP, int NPES, bool NTL>
+// SCATTER turns the kernel into reducescatter: blockIdx.y is the destination PE q, the fold runs over
+// block q (nelems elements, a whole number of vectors) of every PE's source with the operands in
+// reducescatter's order, and only PE q's destination is written.  Tiles are then cut on the
+// source's boundaries, because the loads are npes times the stores.
+template <typename T, int OP, bool SCATTER>
+__device__ __forceinline__ T fold_next(int p, T acc, T x) {
+    return SCATTER ? nvshmemi_amd_reduce_op<T, OP>(acc, x) : nvshmemi_amd_fold_step<T, OP>(p, acc, x);
+}
+
+template <typename T, int OP, int NPES, bool NTL, bool SCATTER = false>
 __global__ __launch_bounds__(NPES ? NPES * 64 : 1024) void reduce_vector_kernel(char *base, uint32_t shift, int npes_arg,
                                                              uint32_t lane_shift_arg, uint64_t dst_off,
                                                              uint64_t src_off, uint64_t nelems) {
@@ -179,9 +199,13 @@ __global__ __launch_bounds__(NPES ? NPES * 64 : 1024) void reduce_vector_kernel(
     // tiles are cut on absolute (16 * lanes)-byte boundaries of the destination, so a wavefront's
     // access is one aligned 1 KiB piece whatever the buffer's own alignment: `lead` vector slots of
     // the first tile lie in front of the buffer
-    const uint64_t lead = ((uint64_t)(uintptr_t)(base + dst_off) >> 4) & (lanes - 1);
-    const uint64_t ntiles = (nvec + lead + lanes - 1) >> lane_shift;
     const uint64_t pe_stride = 1ull << shift;
+    if (SCATTER) {
+        src_off += (uint64_t)blockIdx.y * nelems * sizeof(T);
+        dst_off += (uint64_t)blockIdx.y * pe_stride;
+    }
+    const uint64_t lead = ((uint64_t)(uintptr_t)(base + (SCATTER ? src_off : dst_off)) >> 4) & (lanes - 1);
+    const uint64_t ntiles = (nvec + lead + lanes - 1) >> lane_shift;
     nvshmemi_v4u *stage = reinterpret_cast<nvshmemi_v4u *>(lds);           // [npes][lanes]
     nvshmemi_v4u *result = stage + ((size_t)npes << lane_shift);           // [lanes]
     const T *stage_e = reinterpret_cast<const T *>(stage);
@@ -196,12 +220,17 @@ __global__ __launch_bounds__(NPES ? NPES * 64 : 1024) void reduce_vector_kernel(
             T acc = stage_e[e];
 #pragma unroll
             for (int p = 1; p < npes; ++p)
-                acc = nvshmemi_amd_fold_step<T, OP>(p, acc, stage_e[(size_t)p * tile_elems + e]);
+                acc = fold_next<T, OP, SCATTER>(p, acc, stage_e[(size_t)p * tile_elems + e]);
             result_e[e] = acc;
         }
         __syncthreads();
-        if (v < nvec) stream_store(base + (uint64_t)pe * pe_stride + dst_off + 16 * v, result[i]);
+        if (SCATTER) {
+            if (v < nvec && pe == 0) stream_store(base + dst_off + 16 * v, result[i]);
+        } else {
+            if (v < nvec) stream_store(base + (uint64_t)pe * pe_stride + dst_off + 16 * v, result[i]);
+        }
     }
+    if (SCATTER) return;  // a block of the source is a whole number of vectors
     // elements behind the last full vector
     const uint64_t done = nvec * VEC;
     const uint64_t gid = (uint64_t)blockIdx.x * blockDim.x + threadIdx.x;
@@ -217,18 +246,19 @@ __global__ __launch_bounds__(NPES ? NPES * 64 : 1024) void reduce_vector_kernel(
 }
 
 // Element-at-a-time variant for buffers that are not 16-byte aligned.
-template <typename T, int OP>
+template <typename T, int OP, bool SCATTER = false>
 __global__ __launch_bounds__(kThreads) void reduce_scalar_kernel(char *base, uint32_t shift, int npes,
                                                                  uint64_t dst_off, uint64_t src_off,
                                                                  uint64_t nelems) {
     const uint64_t gsz = (uint64_t)gridDim.x * kThreads;
     const uint64_t es = (1ull << shift) / sizeof(T);
-    const T *s = reinterpret_cast<const T *>(base + src_off);
-    T *d = reinterpret_cast<T *>(base + dst_off);
+    const T *s = reinterpret_cast<const T *>(base + src_off) + (SCATTER ? (uint64_t)blockIdx.y * nelems : 0);
+    T *d = reinterpret_cast<T *>(base + dst_off) + (SCATTER ? (uint64_t)blockIdx.y * es : 0);
     for (uint64_t i = (uint64_t)blockIdx.x * kThreads + threadIdx.x; i < nelems; i += gsz) {
         T acc = s[i];
-        for (int pe = 1; pe < npes; ++pe) acc = nvshmemi_amd_fold_step<T, OP>(pe, acc, s[(uint64_t)pe * es + i]);
-        for (int pe = 0; pe < npes; ++pe) d[(uint64_t)pe * es + i] = acc;
+        for (int pe = 1; pe < npes; ++pe) acc = fold_next<T, OP, SCATTER>(pe, acc, s[(uint64_t)pe * es + i]);
+        if (SCATTER) d[i] = acc;
+        else for (int pe = 0; pe < npes; ++pe) d[(uint64_t)pe * es + i] = acc;
     }
 }
 
@@ -274,42 +304,83 @@ void launch_reduce(Runtime &rt, uint64_t dst_off, uint64_t src_off, uint64_t nel
     }
 }
 
+// reducescatter: grid.y = destination PE; nelems is the element count of one PE's result
+template <typename T, int OP>
+void launch_reducescatter(Runtime &rt, uint64_t dst_off, uint64_t src_off, uint64_t nelems,
+                          hipStream_t stream) {
+    const bool vector_ok = ((dst_off | src_off | (nelems * sizeof(T))) & 15) == 0;
+    if (vector_ok) {
+        uint32_t lane_shift = 6;
+        while (((uint32_t)rt.npes << lane_shift) > 1024) --lane_shift;
+        const unsigned threads = (unsigned)rt.npes << lane_shift;
+        const uint64_t nvec = nelems / (16 / sizeof(T));
+        uint64_t blocks = (nvec + (2u << lane_shift) - 1) >> lane_shift;
+        if (blocks > 0x7fffffffull) blocks = 0x7fffffffull;
+        const size_t lds = ((size_t)rt.npes + 1) * 16 << lane_shift;
+        const dim3 grid((unsigned)blocks, (unsigned)rt.npes);
+        const bool stream_source =
+            (uint64_t)rt.npes * rt.npes * nelems * sizeof(T) > NVSHMEM_AMD_CACHEABLE_SOURCE_BYTES;
+#define NVSHMEM_AMD_LAUNCH_SCATTER(N, NTL)                                                        \
+    hipLaunchKernelGGL((reduce_vector_kernel<T, OP, N, NTL, true>), grid, dim3(threads), lds,     \
+                       stream, rt.base, rt.heap_shift, rt.npes, lane_shift, dst_off, src_off, nelems)
+        if (rt.npes == 8) {
+            if (stream_source) NVSHMEM_AMD_LAUNCH_SCATTER(8, true);
+            else NVSHMEM_AMD_LAUNCH_SCATTER(8, false);
+        } else {
+            if (stream_source) NVSHMEM_AMD_LAUNCH_SCATTER(0, true);
+            else NVSHMEM_AMD_LAUNCH_SCATTER(0, false);
+        }
+#undef NVSHMEM_AMD_LAUNCH_SCATTER
+    } else {
+        uint64_t blocks = (nelems + kThreads - 1) / kThreads;
+        const uint64_t cap = (uint64_t)rt.num_cus * 64 / (uint64_t)rt.npes + 1;
+        if (blocks > cap) blocks = cap;
+        hipLaunchKernelGGL((reduce_scalar_kernel<T, OP, true>), dim3((unsigned)blocks, (unsigned)rt.npes),
+                           dim3(kThreads), 0, stream, rt.base, rt.heap_shift, rt.npes, dst_off,
+                           src_off, nelems);
+    }
+}
+
 typedef void (*reduce_launcher_t)(Runtime &, uint64_t, uint64_t, uint64_t, hipStream_t);
 
-template <typename T>
+template <typename T, bool SCATTER>
 reduce_launcher_t pick_arith(int op) {
+#define NVSHMEM_AMD_PICK(OP) \
+    case NVSHMEMI_OP_##OP: return SCATTER ? launch_reducescatter<T, NVSHMEMI_OP_##OP> : launch_reduce<T, NVSHMEMI_OP_##OP>
     switch (op) {
-        case NVSHMEMI_OP_min: return launch_reduce<T, NVSHMEMI_OP_min>;
-        case NVSHMEMI_OP_max: return launch_reduce<T, NVSHMEMI_OP_max>;
-        case NVSHMEMI_OP_sum: return launch_reduce<T, NVSHMEMI_OP_sum>;
-        case NVSHMEMI_OP_prod: return launch_reduce<T, NVSHMEMI_OP_prod>;
+        NVSHMEM_AMD_PICK(min);
+        NVSHMEM_AMD_PICK(max);
+        NVSHMEM_AMD_PICK(sum);
+        NVSHMEM_AMD_PICK(prod);
         default: return nullptr;
     }
 }
-template <typename T>
+template <typename T, bool SCATTER>
 reduce_launcher_t pick_integer(int op) {
     switch (op) {
-        case NVSHMEMI_OP_and: return launch_reduce<T, NVSHMEMI_OP_and>;
-        case NVSHMEMI_OP_or: return launch_reduce<T, NVSHMEMI_OP_or>;
-        case NVSHMEMI_OP_xor: return launch_reduce<T, NVSHMEMI_OP_xor>;
-        default: return pick_arith<T>(op);
+        NVSHMEM_AMD_PICK(and);
+        NVSHMEM_AMD_PICK(or);
+        NVSHMEM_AMD_PICK(xor);
+        default: return pick_arith<T, SCATTER>(op);
     }
+#undef NVSHMEM_AMD_PICK
 }
 
+template <bool SCATTER>
 reduce_launcher_t pick_reduce(int dtype, int op) {
     switch (dtype) {
-        case NVSHMEMI_DT_i8: return pick_integer<int8_t>(op);
-        case NVSHMEMI_DT_i16: return pick_integer<int16_t>(op);
-        case NVSHMEMI_DT_i32: return pick_integer<int32_t>(op);
-        case NVSHMEMI_DT_i64: return pick_integer<int64_t>(op);
-        case NVSHMEMI_DT_u8: return pick_integer<uint8_t>(op);
-        case NVSHMEMI_DT_u16: return pick_integer<uint16_t>(op);
-        case NVSHMEMI_DT_u32: return pick_integer<uint32_t>(op);
-        case NVSHMEMI_DT_u64: return pick_integer<uint64_t>(op);
-        case NVSHMEMI_DT_f16: return pick_arith<__half>(op);
-        case NVSHMEMI_DT_bf16: return pick_arith<__hip_bfloat16>(op);
-        case NVSHMEMI_DT_f32: return pick_arith<float>(op);
-        case NVSHMEMI_DT_f64: return pick_arith<double>(op);
+        case NVSHMEMI_DT_i8: return pick_integer<int8_t, SCATTER>(op);
+        case NVSHMEMI_DT_i16: return pick_integer<int16_t, SCATTER>(op);
+        case NVSHMEMI_DT_i32: return pick_integer<int32_t, SCATTER>(op);
+        case NVSHMEMI_DT_i64: return pick_integer<int64_t, SCATTER>(op);
+        case NVSHMEMI_DT_u8: return pick_integer<uint8_t, SCATTER>(op);
+        case NVSHMEMI_DT_u16: return pick_integer<uint16_t, SCATTER>(op);
+        case NVSHMEMI_DT_u32: return pick_integer<uint32_t, SCATTER>(op);
+        case NVSHMEMI_DT_u64: return pick_integer<uint64_t, SCATTER>(op);
+        case NVSHMEMI_DT_f16: return pick_arith<__half, SCATTER>(op);
+        case NVSHMEMI_DT_bf16: return pick_arith<__hip_bfloat16, SCATTER>(op);
+        case NVSHMEMI_DT_f32: return pick_arith<float, SCATTER>(op);
+        case NVSHMEMI_DT_f64: return pick_arith<double, SCATTER>(op);
         default: return nullptr;
     }
 }
@@ -334,7 +405,7 @@ int reduce_on_stream(int dtype, int op, nvshmem_team_t team, void *dest, const v
                      size_t nreduce, hipStream_t stream) {
     Runtime &rt = Runtime::get();
     if (!team_ok(rt, "reduce", team)) return NVSHMEMX_ERROR_INVALID_VALUE;
-    reduce_launcher_t fn = pick_reduce(dtype, op);
+    reduce_launcher_t fn = pick_reduce<false>(dtype, op);
     if (!fn) {
         set_error("reduce: operator %d is not defined for element kind %d", op, dtype);
         return NVSHMEMX_ERROR_INVALID_VALUE;
@@ -361,6 +432,84 @@ int reduce_on_stream(int dtype, int op, nvshmem_team_t team, void *dest, const v
     hipError_t e = hipGetLastError();
     if (e != hipSuccess) {
         set_error("reduce: kernel launch failed: %s", hipGetErrorString(e));
+        return NVSHMEMX_ERROR_INTERNAL;
+    }
+    return 0;
+}
+
+int reducescatter_on_stream(int dtype, int op, nvshmem_team_t team, void *dest, const void *src,
+                            size_t nreduce, hipStream_t stream) {
+    Runtime &rt = Runtime::get();
+    if (!team_ok(rt, "reducescatter", team)) return NVSHMEMX_ERROR_INVALID_VALUE;
+    reduce_launcher_t fn = pick_reduce<true>(dtype, op);
+    if (!fn) {
+        set_error("reducescatter: operator %d is not defined for element kind %d", op, dtype);
+        return NVSHMEMX_ERROR_INVALID_VALUE;
+    }
+    if (nreduce == 0) return 0;
+    const size_t es = kDtypeSize[dtype];
+    const uint64_t n = (uint64_t)rt.npes;
+    if (nreduce > rt.heap_size / es / n) {
+        set_error("reducescatter: %zu elements of %zu bytes x %d PEs leave the PE's heap slice",
+                  nreduce, es, rt.npes);
+        return NVSHMEMX_ERROR_INVALID_VALUE;
+    }
+    uint64_t doff = 0, soff = 0;
+    if (!check_symmetric_range(rt, "reducescatter dest", dest, nreduce * es, &doff) ||
+        !check_symmetric_range(rt, "reducescatter source", src, nreduce * es * n, &soff))
+        return NVSHMEMX_ERROR_INVALID_VALUE;
+    if ((doff % es) || (soff % es)) {
+        set_error("reducescatter: buffers must be aligned to the element size");
+        return NVSHMEMX_ERROR_INVALID_VALUE;
+    }
+    // PE q writes dest while other PEs' blocks of the source at the same offsets are still read
+    if (doff < soff + nreduce * es * n && soff < doff + nreduce * es) {
+        set_error("reducescatter: dest and source overlap");
+        return NVSHMEMX_ERROR_INVALID_VALUE;
+    }
+    fn(rt, doff, soff, nreduce, stream);
+    hipError_t e = hipGetLastError();
+    if (e != hipSuccess) {
+        set_error("reducescatter: kernel launch failed: %s", hipGetErrorString(e));
+        return NVSHMEMX_ERROR_INTERNAL;
+    }
+    return 0;
+}
+
+int broadcast_on_stream(nvshmem_team_t team, void *dest, const void *src, size_t bytes, int root,
+                        hipStream_t stream) {
+    Runtime &rt = Runtime::get();
+    if (!team_ok(rt, "broadcast", team)) return NVSHMEMX_ERROR_INVALID_VALUE;
+    if (root < 0 || root >= rt.npes) {
+        set_error("broadcast: root %d is not a PE of the team (0..%d)", root, rt.npes - 1);
+        return NVSHMEMX_ERROR_INVALID_VALUE;
+    }
+    if (bytes == 0) return 0;
+    uint64_t doff = 0, soff = 0;
+    if (!check_symmetric_range(rt, "broadcast dest", dest, bytes, &doff) ||
+        !check_symmetric_range(rt, "broadcast source", src, bytes, &soff))
+        return NVSHMEMX_ERROR_INVALID_VALUE;
+    // identical buffers are the in-place form (the root keeps its data); a partial overlap would
+    // let the root's destination clobber source bytes that are still to be read
+    if (doff != soff && doff < soff + bytes && soff < doff + bytes) {
+        set_error("broadcast: dest and source overlap without being identical");
+        return NVSHMEMX_ERROR_INVALID_VALUE;
+    }
+    const uint64_t tiles = (bytes / 16 + 64 + kCopyThreads - 1) / kCopyThreads + 1;
+    if (tiles > 0x7fffffffull) {
+        set_error("broadcast: message too large");
+        return NVSHMEMX_ERROR_INVALID_VALUE;
+    }
+    const dim3 grid((unsigned)tiles, 1), block(kCopyThreads);
+    if (bytes > NVSHMEM_AMD_CACHEABLE_SOURCE_BYTES)
+        hipLaunchKernelGGL((segment_copy_kernel<kModeBroadcast, 1, true>), grid, block, 0, stream,
+                           rt.base, rt.heap_shift, rt.npes, doff, soff, (uint64_t)bytes, root);
+    else
+        hipLaunchKernelGGL((segment_copy_kernel<kModeBroadcast, 1, false>), grid, block, 0, stream,
+                           rt.base, rt.heap_shift, rt.npes, doff, soff, (uint64_t)bytes, root);
+    hipError_t e = hipGetLastError();
+    if (e != hipSuccess) {
+        set_error("broadcast: kernel launch failed: %s", hipGetErrorString(e));
         return NVSHMEMX_ERROR_INTERNAL;
     }
     return 0;
@@ -397,7 +546,7 @@ static int segment_collective(int mode, const char *what, nvshmem_team_t team, v
     const dim3 grid((unsigned)tiles, segs), block(kCopyThreads);
 #define NVSHMEM_AMD_LAUNCH_SEGCOPY(MODE, U, NTL)                                                   \
     hipLaunchKernelGGL((segment_copy_kernel<MODE, U, NTL>), grid, block, 0, stream, rt.base,       \
-                       rt.heap_shift, rt.npes, doff, soff, (uint64_t)seg_bytes)
+                       rt.heap_shift, rt.npes, doff, soff, (uint64_t)seg_bytes, 0)
     if (mode == kModeFcollect) {
         if (stream_source) NVSHMEM_AMD_LAUNCH_SEGCOPY(kModeFcollect, NVSHMEM_AMD_FCOLLECT_UNROLL, true);
         else NVSHMEM_AMD_LAUNCH_SEGCOPY(kModeFcollect, NVSHMEM_AMD_FCOLLECT_UNROLL, false);
@@ -443,6 +592,16 @@ extern "C" {
                                              size_t nelems, nvshmemx_stream_t s) {                \
         return fcollect_on_stream(team, dest, src, nelems * sizeof(TYPE), (hipStream_t)s);        \
     }                                                                                             \
+    int nvshmemx_##NAME##_broadcast_on_stream(nvshmem_team_t team, TYPE *dest, const TYPE *src,   \
+                                              size_t nelems, int PE_root, nvshmemx_stream_t s) {  \
+        return broadcast_on_stream(team, dest, src, nelems * sizeof(TYPE), PE_root,               \
+                                   (hipStream_t)s);                                               \
+    }                                                                                             \
+    int nvshmem_##NAME##_broadcast(nvshmem_team_t team, TYPE *dest, const TYPE *src,              \
+                                   size_t nelems, int PE_root) {                                  \
+        return finish_blocking(                                                                   \
+            broadcast_on_stream(team, dest, src, nelems * sizeof(TYPE), PE_root, nullptr));       \
+    }                                                                                             \
     int nvshmem_##NAME##_alltoall(nvshmem_team_t team, TYPE *dest, const TYPE *src,               \
                                   size_t nelems) {                                                \
         return finish_blocking(                                                                   \
@@ -464,6 +623,14 @@ int nvshmemx_fcollectmem_on_stream(nvshmem_team_t team, void *dest, const void *
                                    nvshmemx_stream_t stream) {
     return fcollect_on_stream(team, dest, src, nelems, (hipStream_t)stream);
 }
+int nvshmemx_broadcastmem_on_stream(nvshmem_team_t team, void *dest, const void *src, size_t nelems,
+                                    int PE_root, nvshmemx_stream_t stream) {
+    return broadcast_on_stream(team, dest, src, nelems, PE_root, (hipStream_t)stream);
+}
+int nvshmem_broadcastmem(nvshmem_team_t team, void *dest, const void *src, size_t nelems,
+                         int PE_root) {
+    return finish_blocking(broadcast_on_stream(team, dest, src, nelems, PE_root, nullptr));
+}
 int nvshmem_alltoallmem(nvshmem_team_t team, void *dest, const void *src, size_t nelems) {
     return finish_blocking(alltoall_on_stream(team, dest, src, nelems, nullptr));
 }
@@ -482,6 +649,17 @@ int nvshmem_fcollectmem(nvshmem_team_t team, void *dest, const void *src, size_t
                                        size_t nreduce) {                                          \
         return finish_blocking(reduce_on_stream(NVSHMEMI_DT_##TAG, NVSHMEMI_OP_##OP, team, dest,  \
                                                 src, nreduce, nullptr));                          \
+    }                                                                                             \
+    int nvshmemx_##NAME##_##OP##_reducescatter_on_stream(nvshmem_team_t team, TYPE *dest,         \
+                                                         const TYPE *src, size_t nreduce,         \
+                                                         nvshmemx_stream_t s) {                   \
+        return reducescatter_on_stream(NVSHMEMI_DT_##TAG, NVSHMEMI_OP_##OP, team, dest, src,      \
+                                       nreduce, (hipStream_t)s);                                  \
+    }                                                                                             \
+    int nvshmem_##NAME##_##OP##_reducescatter(nvshmem_team_t team, TYPE *dest, const TYPE *src,   \
+                                              size_t nreduce) {                                   \
+        return finish_blocking(reducescatter_on_stream(NVSHMEMI_DT_##TAG, NVSHMEMI_OP_##OP, team, \
+                                                       dest, src, nreduce, nullptr));             \
     }
 NVSHMEMI_REPT_FOR_ALL_REDUCE_TYPES_AND_OPS(NVSHMEMI_DEFINE_TYPED_REDUCE_HOST)
 #undef NVSHMEMI_DEFINE_TYPED_REDUCE_HOST

@@ -37,6 +37,21 @@ DEFINE_REDUCE_KERNEL(uint64, uint64_t, and)
 DEFINE_REDUCE_KERNEL(double, double, prod)
 DEFINE_REDUCE_KERNEL(int16, int16_t, min)
 
+#define DEFINE_SCATTER_KERNEL(TNAME, TYPE, OP)                                                   \
+    template <int SCOPE>                                                                         \
+    __global__ void reducescatter_##TNAME##_##OP##_kernel(TYPE *dest, const TYPE *src, size_t n) { \
+        SCOPED_CALL(SCOPE, TNAME##_##OP##_reducescatter, NVSHMEM_TEAM_WORLD, dest, src, n);      \
+    }
+DEFINE_SCATTER_KERNEL(int32, int32_t, sum)
+DEFINE_SCATTER_KERNEL(float, float, sum)
+DEFINE_SCATTER_KERNEL(float, float, max)
+DEFINE_SCATTER_KERNEL(bfloat16, nvshmem_bfloat16_t, sum)
+DEFINE_SCATTER_KERNEL(uint64, uint64_t, xor)
+
+template <int SCOPE>
+__global__ void broadcast_kernel(char *dest, const char *src, size_t bytes, int root) {
+    SCOPED_CALL(SCOPE, broadcastmem, NVSHMEM_TEAM_WORLD, dest, src, bytes, root);
+}
 template <int SCOPE>
 __global__ void fcollect_kernel(char *dest, const char *src, size_t bytes) {
     SCOPED_CALL(SCOPE, fcollectmem, NVSHMEM_TEAM_WORLD, dest, src, bytes);
@@ -79,9 +94,46 @@ int launch_scoped(int scope, void (*kb)(Args...), void (*kw)(Args...), void (*kt
         reduce_##TNAME##_##OP##_kernel<NVSHMEM_PERFTEST_SCOPE_THREAD>, threads, stream,          \
         (TYPE *)dest, (const TYPE *)src, nreduce)
 
+#define LAUNCH_SCATTER(TNAME, TYPE, OP)                                                          \
+    return launch_scoped<TYPE *, const TYPE *, size_t>(                                          \
+        scope, reducescatter_##TNAME##_##OP##_kernel<NVSHMEM_PERFTEST_SCOPE_BLOCK>,              \
+        reducescatter_##TNAME##_##OP##_kernel<NVSHMEM_PERFTEST_SCOPE_WARP>,                      \
+        reducescatter_##TNAME##_##OP##_kernel<NVSHMEM_PERFTEST_SCOPE_THREAD>, threads, stream,   \
+        (TYPE *)dest, (const TYPE *)src, nreduce)
+
 }  // namespace
 
 extern "C" {
+
+int nvshmem_perftest_device_reducescatter(int dtype, int op, void *dest, const void *src,
+                                          size_t nreduce, int scope, int threads, void *stream) {
+    static const size_t esize[NVSHMEMI_DT_COUNT] = {1, 2, 4, 8, 1, 2, 4, 8, 2, 2, 4, 8};
+    if (!perftest::ready() || dtype < 0 || dtype >= NVSHMEMI_DT_COUNT || scope < 0 || scope > 2 ||
+        !perftest::check_launch(1, threads) || !perftest::check_range(dest, nreduce * esize[dtype]) ||
+        !perftest::check_range(src, nreduce * esize[dtype] * (size_t)nvshmem_n_pes()))
+        return NVSHMEMX_ERROR_INVALID_VALUE;
+    const int key = dtype * 16 + op;
+    switch (key) {
+        case NVSHMEMI_DT_i32 * 16 + NVSHMEMI_OP_sum: LAUNCH_SCATTER(int32, int32_t, sum);
+        case NVSHMEMI_DT_f32 * 16 + NVSHMEMI_OP_sum: LAUNCH_SCATTER(float, float, sum);
+        case NVSHMEMI_DT_f32 * 16 + NVSHMEMI_OP_max: LAUNCH_SCATTER(float, float, max);
+        case NVSHMEMI_DT_bf16 * 16 + NVSHMEMI_OP_sum: LAUNCH_SCATTER(bfloat16, nvshmem_bfloat16_t, sum);
+        case NVSHMEMI_DT_u64 * 16 + NVSHMEMI_OP_xor: LAUNCH_SCATTER(uint64, uint64_t, xor);
+        default: return NVSHMEMX_ERROR_NOT_SUPPORTED;
+    }
+}
+
+int nvshmem_perftest_device_broadcast(void *dest, const void *src, size_t bytes, int root,
+                                      int scope, int threads, void *stream) {
+    if (!perftest::ready() || scope < 0 || scope > 2 || root < 0 || root >= nvshmem_n_pes() ||
+        !perftest::check_launch(1, threads) || !perftest::check_range(dest, bytes) ||
+        !perftest::check_range(src, bytes))
+        return NVSHMEMX_ERROR_INVALID_VALUE;
+    return launch_scoped<char *, const char *, size_t, int>(
+        scope, broadcast_kernel<NVSHMEM_PERFTEST_SCOPE_BLOCK>, broadcast_kernel<NVSHMEM_PERFTEST_SCOPE_WARP>,
+        broadcast_kernel<NVSHMEM_PERFTEST_SCOPE_THREAD>, threads, stream, (char *)dest,
+        (const char *)src, bytes, root);
+}
 
 int nvshmem_perftest_device_reduce(int dtype, int op, void *dest, const void *src, size_t nreduce,
                                    int scope, int threads, void *stream) {

@@ -134,6 +134,31 @@ class Runtime:
             rc = _lib.typed_coll(self.lib, name, True)(team, dest, src, nreduce, stream.ptr)
         self._check(rc, name)
 
+    def reducescatter(self, type_name, op, dest, src, nreduce, stream=None, team=TEAM_WORLD):
+        if stream is None:
+            name = "nvshmem_%s_%s_reducescatter" % (type_name, op)
+            rc = _lib.typed_coll(self.lib, name)(team, dest, src, nreduce)
+        else:
+            name = "nvshmemx_%s_%s_reducescatter_on_stream" % (type_name, op)
+            rc = _lib.typed_coll(self.lib, name, True)(team, dest, src, nreduce, stream.ptr)
+        self._check(rc, name)
+
+    def broadcast(self, type_name, dest, src, nelems, root, stream=None, team=TEAM_WORLD):
+        if stream is None:
+            name = "nvshmem_%s_broadcast" % type_name
+            rc = _lib.typed_coll(self.lib, name, rooted=True)(team, dest, src, nelems, root)
+        else:
+            name = "nvshmemx_%s_broadcast_on_stream" % type_name
+            rc = _lib.typed_coll(self.lib, name, True, True)(team, dest, src, nelems, root, stream.ptr)
+        self._check(rc, name)
+
+    def broadcastmem(self, dest, src, nbytes, root, stream=None):
+        if stream is None:
+            self._check(self.lib.nvshmem_broadcastmem(TEAM_WORLD, dest, src, nbytes, root), "broadcastmem")
+        else:
+            self._check(self.lib.nvshmemx_broadcastmem_on_stream(TEAM_WORLD, dest, src, nbytes, root,
+                                                                 stream.ptr), "broadcastmem_on_stream")
+
     def fcollect(self, type_name, dest, src, nelems, stream=None, team=TEAM_WORLD):
         if stream is None:
             name = "nvshmem_%s_fcollect" % type_name

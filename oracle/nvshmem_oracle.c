@@ -300,6 +300,51 @@ int oracle_reduce(int dtype, int op, int npes, size_t nelems, const void *src, v
     return 0;
 }
 
+/* reducescatter: reference nvshmemi_reducescatter_allpush_threadgroup,
+ * src/include/non_abi/device/coll/reducescatter.cuh:36-90: PE q gathers block q of every PE's source
+ * and folds it as  acc = op(x0, x1);  acc = op(acc, x_p)  for p = 2 .. npes-1  (:63-86, where
+ * gpu_linear_reduce(op1 = dest, op2 = x_p) computes op(dest, x_p)). */
+#define SCATTER_LOOP(NAME, T)                                                        \
+    {                                                                                \
+        const T *s = (const T *)src;                                                 \
+        T *d = (T *)dst;                                                             \
+        const size_t row = (size_t)npes * nelems;                                    \
+        _Pragma("omp parallel for schedule(static)")                                 \
+        for (size_t g = 0; g < row; ++g) { /* g = q*nelems + k */                    \
+            T acc = s[g];                                                            \
+            for (int p = 1; p < npes; ++p) acc = NAME##_apply(op, acc, s[(size_t)p * row + g]); \
+            d[g] = acc;                                                              \
+        }                                                                            \
+    }                                                                                \
+    break;
+
+int oracle_reducescatter(int dtype, int op, int npes, size_t nelems, const void *src, void *dst) {
+    if (op < ORC_and || op > ORC_prod) return -1;
+    if (dtype >= ORC_f16 && op < ORC_min) return -1;
+    switch (dtype) {
+        case ORC_i8: SCATTER_LOOP(i8, int8_t)
+        case ORC_i16: SCATTER_LOOP(i16, int16_t)
+        case ORC_i32: SCATTER_LOOP(i32, int32_t)
+        case ORC_i64: SCATTER_LOOP(i64, int64_t)
+        case ORC_u8: SCATTER_LOOP(u8, uint8_t)
+        case ORC_u16: SCATTER_LOOP(u16, uint16_t)
+        case ORC_u32: SCATTER_LOOP(u32, uint32_t)
+        case ORC_u64: SCATTER_LOOP(u64, uint64_t)
+        case ORC_f16: SCATTER_LOOP(f16, uint16_t)
+        case ORC_bf16: SCATTER_LOOP(bf16, uint16_t)
+        case ORC_f32: SCATTER_LOOP(f32, float)
+        case ORC_f64: SCATTER_LOOP(f64, double)
+        default: return -1;
+    }
+    return 0;
+}
+
+/* broadcast: reference src/include/non_abi/device/coll/broadcast.cuh:276-337 (every PE's dest gets
+ * the root's source; the root copies too when dest != source, :97) */
+void oracle_broadcast(int npes, size_t bytes, int root, const uint8_t *src, uint8_t *dst) {
+    for (int q = 0; q < npes; ++q) memcpy(dst + (size_t)q * bytes, src + (size_t)root * bytes, bytes);
+}
+
 /* ------------------------------------------------------------------------------------------- */
 /* fcollect: reference nvshmemi_fcollect_p2p_allpush_threadgroup,
  *   src/include/non_abi/device/coll/fcollect.cuh:331-344: PE p copies its source into slot p of

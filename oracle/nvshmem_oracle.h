@@ -11,6 +11,9 @@
  *   copies / ring put / fcollect / alltoall / moe maps  brute-force index maps on tiny inputs,
  *       involution and replication invariants, the reference's own known answers
  *       (examples/put-block.cu:93-104);
+ *   broadcast / reducescatter   brute force, the reference's known answer for broadcast
+ *       (examples/ring-bcast.cu:68-72), slices of the pinned reduce for order-free operators, numpy
+ *       folds and hand-evaluated NaN cases for the operand order;
  *   integer reduce        order-free closed forms, numpy, reference known answer dst[i]==i*npes
  *       (examples/ring-reduce.cu:242-248, examples/user-buffer.cu:141-152);
  *   fp32 / fp16 / bf16 reduce   numpy / torch CPU left folds in the element type, order-sensitive
@@ -80,6 +83,13 @@ int oracle_reduce(int dtype, int op, int npes, size_t nelems, const void *src, v
 void oracle_fcollect(int npes, size_t seg_bytes, const uint8_t *src, uint8_t *dst);
 /* dst[q][p*seg + k] = src[p][q*seg + k]; src and dst are [npes][npes*seg_bytes] */
 void oracle_alltoall(int npes, size_t seg_bytes, const uint8_t *src, uint8_t *dst);
+
+/* dst[q][k] = fold over p of src[p][q*nelems + k], order acc = op(x0, x1); acc = op(acc, x_p) for
+ * p >= 2 (operands the other way round than in oracle_reduce); src is [npes][npes*nelems], dst is
+ * [npes][nelems].  Returns 0, or -1 when op is not defined for dtype. */
+int oracle_reducescatter(int dtype, int op, int npes, size_t nelems, const void *src, void *dst);
+/* dst[q][k] = src[root][k] for every q including the root; src, dst are [npes][bytes] */
+void oracle_broadcast(int npes, size_t bytes, int root, const uint8_t *src, uint8_t *dst);
 
 /* ---- allocator model (independent structure: one ordered block list) ---- */
 typedef struct oracle_space oracle_space_t;

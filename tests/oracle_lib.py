@@ -50,6 +50,8 @@ def lib():
         "oracle_compare_i64": (i32, [C.c_int64, i32, C.c_int64]),
         "oracle_ptr": (u64, [u64, u64, i32, u64, i32]),
         "oracle_reduce": (i32, [i32, i32, i32, sz, vp, vp]),
+        "oracle_reducescatter": (i32, [i32, i32, i32, sz, vp, vp]),
+        "oracle_broadcast": (None, [i32, sz, i32, vp, vp]),
         "oracle_fcollect": (None, [i32, sz, vp, vp]),
         "oracle_alltoall": (None, [i32, sz, vp, vp]),
         "oracle_space_create": (vp, [u64, u64]),
@@ -109,6 +111,25 @@ def reduce(dtype, op, src):
     rc = lib().oracle_reduce(DT[dtype], OP[op], npes, n, _p(src), _p(out))
     if rc != 0:
         raise ValueError("oracle_reduce: %s/%s undefined" % (dtype, op))
+    return out
+
+
+def reducescatter(dtype, op, src):
+    """src: [npes, npes*n] -> [npes, n]."""
+    src = np.ascontiguousarray(src)
+    npes, total = src.shape
+    n = total // npes
+    out = np.empty((npes, n), dtype=src.dtype)
+    rc = lib().oracle_reducescatter(DT[dtype], OP[op], npes, n, _p(src), _p(out))
+    if rc != 0:
+        raise ValueError("oracle_reducescatter: %s/%s undefined" % (dtype, op))
+    return out
+
+
+def broadcast(src_bytes, root):
+    src = np.ascontiguousarray(src_bytes, dtype=np.uint8)
+    out = np.empty_like(src)
+    lib().oracle_broadcast(src.shape[0], src.shape[1], root, _p(src), _p(out))
     return out
 
 

@@ -76,3 +76,27 @@ def test_init_rejects_bad_team_sizes():
     assert lib.nvshmemx_amd_init(0, 1 << 20) != 0
     assert lib.nvshmemx_amd_init(65, 1 << 20) != 0
     assert lib.nvshmemx_init_status() == 0
+
+
+@pytest.mark.parametrize("npes", [1, 2, 3, 16, 24])
+def test_broadcast_and_reducescatter_on_other_team_sizes(npes):
+    rng = np.random.default_rng(npes)
+    n = 2052
+    with runtime(npes, 1 << 22) as rt:
+        src = rt.malloc(npes * n * 4); dst = rt.malloc(n * 4)
+        data = rng.standard_normal((npes, npes * n)).astype(np.float32)
+        rt.upload_all(src, data)
+        note("npes=%d reducescatter float sum" % npes)
+        rt.reducescatter("float", "sum", dst, src, n)
+        assert bits_equal(rt.download_all(dst, (n,), np.float32), O.reducescatter("f32", "sum", data))
+        idata = rng.integers(-2**31, 2**31 - 1, (npes, npes * n), dtype=np.int32)
+        rt.upload_all(src, idata)
+        rt.reducescatter("int32", "xor", dst, src, n)
+        assert bits_equal(rt.download_all(dst, (n,), np.int32), O.reducescatter("i32", "xor", idata))
+        root = npes - 1
+        note("npes=%d broadcast root=%d" % (npes, root))
+        rt.broadcastmem(dst + 1, src + 3, n * 4 - 7, root)
+        got = rt.download_all(dst, (n * 4 - 7,), np.uint8, 1)
+        want = idata.view(np.uint8)[root, 3:3 + n * 4 - 7]
+        assert all(np.array_equal(got[pe], want) for pe in range(npes))
+        rt.free(src); rt.free(dst)

@@ -329,3 +329,51 @@ def test_moe_plan_brute_force():
             assert np.array_equal(recv[dest_pe[src, r]][dest_row[src, r]], send[src, r // K])
     back = O.moe_combine(recv, dest_pe, dest_row, T, K, 24)
     assert np.array_equal(back, np.repeat(send, K, axis=1))
+
+
+# ---------------------------------------------------------------------------------------------
+# broadcast / reducescatter
+# ---------------------------------------------------------------------------------------------
+def test_broadcast_brute_force_and_reference_known_answer():
+    rng = np.random.default_rng(4)
+    for npes, nbytes, root in ((1, 5, 0), (3, 7, 2), (8, 64, 5)):
+        src = rng.integers(0, 256, (npes, nbytes), dtype=np.uint8)
+        got = O.broadcast(src, root)
+        for q in range(npes):
+            assert np.array_equal(got[q], src[root])
+    # examples/ring-bcast.cu:44-72: the root (PE 0) holds mype + i = i, every PE ends with i
+    npes, n = 4, 100
+    data = np.stack([(pe + np.arange(n)).astype(np.int32) for pe in range(npes)])
+    got = O.broadcast(data.view(np.uint8), 0).view(np.int32)
+    assert all((got[pe] == np.arange(n)).all() for pe in range(npes))
+
+
+def test_reducescatter_is_the_sliced_reduce_and_keeps_its_operand_order():
+    rng = np.random.default_rng(6)
+    npes, n = 5, 37
+    # order-free operators: PE q's result is slice q of the (already pinned) allreduce
+    for kind in ("i32", "u64", "i8"):
+        dt = O.NP_STORAGE[kind]
+        info = np.iinfo(dt)
+        src = rng.integers(info.min, info.max, (npes, npes * n), dtype=dt, endpoint=True)
+        for op in ("sum", "xor", "min", "prod"):
+            got = O.reducescatter(kind, op, src)
+            want = O.reduce(kind, op, src).reshape(npes, n)
+            assert np.array_equal(got, want), (kind, op)
+    # fp32 sum: numpy left fold acc = acc + x_p
+    f = (rng.standard_normal((npes, npes * n)) * 10.0 ** rng.integers(-5, 6, (npes, npes * n))).astype(np.float32)
+    acc = f[0].copy()
+    for p in range(1, npes):
+        acc = acc + f[p]
+    assert np.array_equal(O.reducescatter("f32", "sum", f).reshape(-1), acc)
+
+    # operand order acc = op(acc, x) with max(a, b) = (a > b) ? a : b, evaluated by hand; the last
+    # case tells it apart from the allreduce order acc = op(x, acc), which gives NaN there
+    def rs_max(xs):
+        col = np.array(xs, np.float32)[:, None]
+        return O.reducescatter("f32", "max", np.tile(col, (1, len(xs))))[0, 0]
+    nan = float("nan")
+    assert np.isnan(rs_max([1, 2, nan]))      # max(1,2)=2 ; (2>nan)?2:nan = nan
+    assert rs_max([nan, 1, 2]) == 2.0         # (nan>1)?nan:1 = 1 ; (1>2)?1:2 = 2
+    assert rs_max([1, nan, 0]) == 0.0         # (1>nan)?1:nan = nan ; (nan>0)?nan:0 = 0
+    assert np.isnan(O.reduce("f32", "max", np.array([[1], [nan], [0]], np.float32))[0])
