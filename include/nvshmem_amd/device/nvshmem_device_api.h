@@ -17,8 +17,12 @@
 /* ---- identity and translation ---- */
 NVSHMEMI_DEV int nvshmem_my_pe(void) { return nvshmemi_amd_my_pe(); }
 NVSHMEMI_DEV int nvshmem_n_pes(void) { return nvshmemi_amd_n_pes(); }
-NVSHMEMI_DEV int nvshmem_team_my_pe(nvshmem_team_t) { return nvshmemi_amd_my_pe(); }
-NVSHMEMI_DEV int nvshmem_team_n_pes(nvshmem_team_t) { return nvshmemi_amd_n_pes(); }
+NVSHMEMI_DEV int nvshmem_team_my_pe(nvshmem_team_t team) { return nvshmemi_team_my_pe(team); }
+NVSHMEMI_DEV int nvshmem_team_n_pes(nvshmem_team_t team) { return nvshmemi_team_n_pes(team); }
+NVSHMEMI_DEV int nvshmem_team_translate_pe(nvshmem_team_t src_team, int src_pe,
+                                           nvshmem_team_t dest_team) {
+    return nvshmemi_team_translate_pe(src_team, src_pe, dest_team);
+}
 NVSHMEMI_DEV void *nvshmem_ptr(const void *ptr, int pe) { return nvshmemi_ptr(ptr, pe); }
 
 /* ---- ordering ---- */
@@ -27,16 +31,16 @@ NVSHMEMI_DEV void nvshmem_fence(void) { nvshmemi_quiet<NVSHMEMI_THREADGROUP_THRE
 NVSHMEMI_DEV void nvshmemx_quiet_warp(void) { nvshmemi_quiet<NVSHMEMI_THREADGROUP_WARP>(); }
 NVSHMEMI_DEV void nvshmemx_quiet_block(void) { nvshmemi_quiet<NVSHMEMI_THREADGROUP_BLOCK>(); }
 
-/* ---- barrier / sync over all PEs: one thread group per PE calls ---- */
+/* ---- barrier / sync over all PEs or a team: one thread group per member PE calls ---- */
 #define NVSHMEMI_STAMP_BARRIER(PFX, SFX, SC)                                                     \
     NVSHMEMI_DEV void PFX##_barrier_all##SFX(void) { nvshmemi_barrier_threadgroup<SC>(); }       \
-    NVSHMEMI_DEV int PFX##_barrier##SFX(nvshmem_team_t) {                                        \
-        nvshmemi_barrier_threadgroup<SC>();                                                      \
+    NVSHMEMI_DEV int PFX##_barrier##SFX(nvshmem_team_t team) {                                   \
+        nvshmemi_barrier_threadgroup<SC>(team);                                                  \
         return 0;                                                                                \
     }                                                                                            \
     NVSHMEMI_DEV void PFX##_sync_all##SFX(void) { nvshmemi_sync_threadgroup<SC>(); }             \
-    NVSHMEMI_DEV int PFX##_team_sync##SFX(nvshmem_team_t) {                                      \
-        nvshmemi_sync_threadgroup<SC>();                                                         \
+    NVSHMEMI_DEV int PFX##_team_sync##SFX(nvshmem_team_t team) {                                 \
+        nvshmemi_sync_threadgroup<SC>(team);                                                     \
         return 0;                                                                                \
     }
 NVSHMEMI_STAMP_BARRIER(nvshmem, , NVSHMEMI_THREADGROUP_THREAD)

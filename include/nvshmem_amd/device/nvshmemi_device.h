@@ -435,6 +435,60 @@ NVSHMEMI_DEVICE_INLINE int nvshmemi_test(T *ivar, int cmp, T value) {
 }
 
 /* ------------------------------------------------------------------------------------------------
+ * Teams (reference non_abi/device/team/nvshmemi_team_defines.cuh:95-141).  A team is the strided
+ * PE set {start + i*stride, i < size}; the table holds every team as each PE sees it.
+ * ---------------------------------------------------------------------------------------------- */
+NVSHMEMI_DEVICE_INLINE nvshmemi_amd_team_view_t nvshmemi_amd_team_view_of(nvshmem_team_t team, int pe) {
+    nvshmemi_amd_team_view_t v;
+    if (team == NVSHMEM_TEAM_WORLD) {
+        v.start = 0; v.stride = 1; v.size = nvshmemi_device_state_d.npes; v.my_pe = pe;
+    } else if (team < 0 || team >= NVSHMEMI_AMD_MAX_TEAMS) {
+        v.start = 0; v.stride = 1; v.size = 0; v.my_pe = -1;
+    } else {
+        v = nvshmemi_device_state_d.team_views[team * NVSHMEMI_AMD_MAX_PES + pe];
+    }
+    return v;
+}
+NVSHMEMI_DEVICE_INLINE nvshmemi_amd_team_view_t nvshmemi_amd_team_view(nvshmem_team_t team) {
+    return nvshmemi_amd_team_view_of(team, nvshmemi_amd_my_pe());
+}
+/* world PE of member `idx` */
+NVSHMEMI_DEVICE_INLINE int nvshmemi_amd_team_pe(const nvshmemi_amd_team_view_t &v, int idx) {
+    return v.start + idx * v.stride;
+}
+NVSHMEMI_DEVICE_INLINE int nvshmemi_team_my_pe(nvshmem_team_t team) {
+    const nvshmemi_amd_team_view_t v = nvshmemi_amd_team_view(team);
+    return v.size > 0 ? v.my_pe : -1;
+}
+NVSHMEMI_DEVICE_INLINE int nvshmemi_team_n_pes(nvshmem_team_t team) {
+    const nvshmemi_amd_team_view_t v = nvshmemi_amd_team_view(team);
+    return v.size > 0 ? v.size : -1;
+}
+/* Member src_pe of src_team as an index of dest_team, or -1; an index equal to the size wraps to
+ * member 0 and larger ones give -1, as in the reference (nvshmemi_team_defines.cuh:120-141). */
+NVSHMEMI_DEVICE_INLINE int nvshmemi_team_translate_pe(nvshmem_team_t src_team, int src_pe,
+                                                      nvshmem_team_t dest_team) {
+    const nvshmemi_amd_team_view_t s = nvshmemi_amd_team_view(src_team);
+    const nvshmemi_amd_team_view_t d = nvshmemi_amd_team_view(dest_team);
+    if (s.size <= 0 || d.size <= 0 || src_pe < 0 || src_pe > s.size) return -1;
+    const int off = nvshmemi_amd_team_pe(s, src_pe % s.size) - d.start;
+    if (off < 0 || off % d.stride != 0 || off / d.stride >= d.size) return -1;
+    return off / d.stride;
+}
+/* arrival words of PE `pe` for `team`, and that PE's epoch word */
+NVSHMEMI_DEVICE_INLINE uint64_t *nvshmemi_amd_sync_row(nvshmem_team_t team, int pe) {
+    if (team == NVSHMEM_TEAM_WORLD)
+        return reinterpret_cast<uint64_t *>(nvshmemi_amd_remote(nvshmemi_device_state_d.sync_flags, pe));
+    return nvshmemi_device_state_d.team_sync +
+           ((size_t)team * NVSHMEMI_AMD_MAX_PES + (size_t)pe) * NVSHMEMI_AMD_TEAM_SYNC_WORDS;
+}
+NVSHMEMI_DEVICE_INLINE uint64_t *nvshmemi_amd_sync_epoch(nvshmem_team_t team, int pe) {
+    if (team == NVSHMEM_TEAM_WORLD)
+        return reinterpret_cast<uint64_t *>(nvshmemi_amd_remote(nvshmemi_device_state_d.sync_epoch, pe));
+    return nvshmemi_amd_sync_row(team, pe) + NVSHMEMI_AMD_MAX_PES;
+}
+
+/* ------------------------------------------------------------------------------------------------
  * barrier / sync  (reference coll/barrier.cuh:24-251, coll/utils.cuh:38-51)
  *
  * One thread group per PE takes part.  Flat exchange (the reference's dissemination with radix =
@@ -443,31 +497,31 @@ NVSHMEMI_DEVICE_INLINE int nvshmemi_test(T *ivar, int cmp, T value) {
  * row have reached that epoch.  Epochs only grow, so rows are never reset.
  * ---------------------------------------------------------------------------------------------- */
 template <int SCOPE>
-NVSHMEMI_DEVICE_INLINE void nvshmemi_sync_threadgroup() {
+NVSHMEMI_DEVICE_INLINE void nvshmemi_sync_threadgroup(nvshmem_team_t team = NVSHMEM_TEAM_WORLD) {
     const int me = nvshmemi_amd_my_pe();
-    const int npes = nvshmemi_device_state_d.npes;
+    const nvshmemi_amd_team_view_t v = nvshmemi_amd_team_view(team);
+    if (v.size <= 0) return; /* not a member */
     const int tid = nvshmemi_thread_id_in_threadgroup<SCOPE>();
     const int nthr = nvshmemi_threadgroup_size<SCOPE>();
-    uint64_t *epoch_p =
-        reinterpret_cast<uint64_t *>(nvshmemi_amd_remote(nvshmemi_device_state_d.sync_epoch, me));
+    uint64_t *epoch_p = nvshmemi_amd_sync_epoch(team, me);
     nvshmemi_threadgroup_sync<SCOPE>();
     const uint64_t epoch = *reinterpret_cast<volatile uint64_t *>(epoch_p) + 1;
     nvshmemi_threadgroup_sync<SCOPE>();
     if (tid == 0) *reinterpret_cast<volatile uint64_t *>(epoch_p) = epoch;
-    for (int pe = tid; pe < npes; pe += nthr) {
-        uint64_t *flag =
-            reinterpret_cast<uint64_t *>(nvshmemi_amd_remote(nvshmemi_device_state_d.sync_flags, pe)) + me;
+    for (int i = tid; i < v.size; i += nthr) {
+        uint64_t *flag = nvshmemi_amd_sync_row(team, nvshmemi_amd_team_pe(v, i)) + v.my_pe;
         __hip_atomic_store(flag, epoch, __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_AGENT);
     }
-    uint64_t *row = reinterpret_cast<uint64_t *>(nvshmemi_amd_remote(nvshmemi_device_state_d.sync_flags, me));
-    for (int pe = tid; pe < npes; pe += nthr) nvshmemi_wait_until<uint64_t>(row + pe, NVSHMEM_CMP_GE, epoch);
+    uint64_t *row = nvshmemi_amd_sync_row(team, me);
+    for (int i = tid; i < v.size; i += nthr)
+        nvshmemi_wait_until<uint64_t>(row + i, NVSHMEM_CMP_GE, epoch);
     nvshmemi_threadgroup_sync<SCOPE>();
 }
 
 template <int SCOPE>
-NVSHMEMI_DEVICE_INLINE void nvshmemi_barrier_threadgroup() {
+NVSHMEMI_DEVICE_INLINE void nvshmemi_barrier_threadgroup(nvshmem_team_t team = NVSHMEM_TEAM_WORLD) {
     nvshmemi_quiet<SCOPE>();
-    nvshmemi_sync_threadgroup<SCOPE>();
+    nvshmemi_sync_threadgroup<SCOPE>(team);
 }
 
 /* ------------------------------------------------------------------------------------------------
@@ -550,18 +604,20 @@ NVSHMEMI_DEVICE_INLINE T nvshmemi_amd_fold_element(const T *src0, size_t pe_stri
 template <typename T, int OP, int SCOPE>
 NVSHMEMI_DEVICE_INLINE int nvshmemi_reduce_threadgroup(nvshmem_team_t team, T *dest, const T *source,
                                                        size_t nreduce) {
-    (void)team;
     constexpr size_t VEC = 16 / sizeof(T);
     struct alignas(16) pack_t { T e[VEC]; };
-    const int me = nvshmemi_amd_my_pe();
-    const int npes = nvshmemi_device_state_d.npes;
+    const nvshmemi_amd_team_view_t tv = nvshmemi_amd_team_view(team);
+    if (tv.size <= 0) return 1; /* the calling PE is not a member */
+    const int me = tv.my_pe;
+    const int npes = tv.size;
     const size_t tid = (size_t)nvshmemi_thread_id_in_threadgroup<SCOPE>();
     const size_t nthr = (size_t)nvshmemi_threadgroup_size<SCOPE>();
     /* every PE's source is complete and visible before anyone reads it */
-    nvshmemi_barrier_threadgroup<SCOPE>();
-    const T *src0 = reinterpret_cast<const T *>(nvshmemi_amd_remote(source, 0));
-    T *dst0 = reinterpret_cast<T *>(nvshmemi_amd_remote(dest, 0));
-    const size_t pe_stride = (size_t)(nvshmemi_device_state_d.heap_size / sizeof(T));
+    nvshmemi_barrier_threadgroup<SCOPE>(team);
+    /* member 0's copies; member i's are i * pe_stride elements further */
+    const T *src0 = reinterpret_cast<const T *>(nvshmemi_amd_remote(source, tv.start));
+    T *dst0 = reinterpret_cast<T *>(nvshmemi_amd_remote(dest, tv.start));
+    const size_t pe_stride = (size_t)(nvshmemi_device_state_d.heap_size / sizeof(T)) * (size_t)tv.stride;
     const bool vectors = (((uintptr_t)src0 | (uintptr_t)dst0) & 15) == 0;
     /* chunk in elements, a whole number of vectors on the vector path */
     size_t chunk = (nreduce + (size_t)npes - 1) / (size_t)npes;
@@ -590,84 +646,87 @@ NVSHMEMI_DEVICE_INLINE int nvshmemi_reduce_threadgroup(nvshmem_team_t team, T *d
         const T acc = nvshmemi_amd_fold_element<T, OP>(src0, pe_stride, npes, i);
         for (int pe = 0; pe < npes; ++pe) dst0[(size_t)pe * pe_stride + i] = acc;
     }
-    nvshmemi_barrier_threadgroup<SCOPE>();
+    nvshmemi_barrier_threadgroup<SCOPE>(team);
     return 0;
 }
 
 template <typename T, int SCOPE>
 NVSHMEMI_DEVICE_INLINE int nvshmemi_fcollect_threadgroup(nvshmem_team_t team, T *dest,
                                                          const T *source, size_t nelems) {
-    (void)team;
-    const int me = nvshmemi_amd_my_pe();
-    const int npes = nvshmemi_device_state_d.npes;
+    const nvshmemi_amd_team_view_t tv = nvshmemi_amd_team_view(team);
+    if (tv.size <= 0) return 1;
+    const int me = tv.my_pe;
+    const int npes = tv.size;
     nvshmemi_threadgroup_sync<SCOPE>();
     for (int ii = 0; ii < npes; ++ii) {
-        const int peer = (me + ii) % npes;
+        const int peer = nvshmemi_amd_team_pe(tv, (me + ii) % npes);
         nvshmemi_memcpy_threadgroup<SCOPE>(nvshmemi_amd_remote(dest + (size_t)me * nelems, peer),
                                            nvshmemi_amd_local(source), nelems * sizeof(T));
     }
-    nvshmemi_barrier_threadgroup<SCOPE>();
+    nvshmemi_barrier_threadgroup<SCOPE>(team);
     return 0;
 }
 
 template <typename T, int SCOPE>
 NVSHMEMI_DEVICE_INLINE int nvshmemi_alltoall_threadgroup(nvshmem_team_t team, T *dest,
                                                          const T *source, size_t nelems) {
-    (void)team;
-    const int me = nvshmemi_amd_my_pe();
-    const int npes = nvshmemi_device_state_d.npes;
+    const nvshmemi_amd_team_view_t tv = nvshmemi_amd_team_view(team);
+    if (tv.size <= 0) return 1;
+    const int me = tv.my_pe;
+    const int npes = tv.size;
     nvshmemi_threadgroup_sync<SCOPE>();
     for (int ii = 0; ii < npes; ++ii) {
-        const int peer = (me + ii) % npes;
-        nvshmemi_memcpy_threadgroup<SCOPE>(nvshmemi_amd_remote(dest + (size_t)me * nelems, peer),
-                                           nvshmemi_amd_local(source + (size_t)peer * nelems),
-                                           nelems * sizeof(T));
+        const int idx = (me + ii) % npes;
+        nvshmemi_memcpy_threadgroup<SCOPE>(
+            nvshmemi_amd_remote(dest + (size_t)me * nelems, nvshmemi_amd_team_pe(tv, idx)),
+            nvshmemi_amd_local(source + (size_t)idx * nelems), nelems * sizeof(T));
     }
-    nvshmemi_barrier_threadgroup<SCOPE>();
+    nvshmemi_barrier_threadgroup<SCOPE>(team);
     return 0;
 }
 
 /* Broadcast (reference coll/broadcast.cuh:298-337, the put-to-all algorithm): the root's thread
- * group copies its source into every PE's dest, its own included unless dest == source; the closing
- * barrier completes the copies and tells the receivers. */
+ * group copies its source into every member's dest, its own included unless dest == source; the
+ * closing barrier completes the copies and tells the receivers.  PE_root is an index of the team. */
 template <typename T, int SCOPE>
 NVSHMEMI_DEVICE_INLINE int nvshmemi_broadcast_threadgroup(nvshmem_team_t team, T *dest,
                                                           const T *source, size_t nelems,
                                                           int PE_root) {
-    (void)team;
-    const int me = nvshmemi_amd_my_pe();
-    const int npes = nvshmemi_device_state_d.npes;
+    const nvshmemi_amd_team_view_t tv = nvshmemi_amd_team_view(team);
+    if (tv.size <= 0) return 1;
+    const int me = tv.my_pe;
+    const int npes = tv.size;
     if (me == PE_root) {
         const void *from = nvshmemi_amd_local(source);
         for (int ii = 0; ii < npes; ++ii) {
-            const int peer = (me + ii) % npes;
-            void *to = nvshmemi_amd_remote(dest, peer);
+            void *to = nvshmemi_amd_remote(dest, nvshmemi_amd_team_pe(tv, (me + ii) % npes));
             if (to != from) nvshmemi_memcpy_threadgroup<SCOPE>(to, from, nelems * sizeof(T));
         }
     }
-    nvshmemi_barrier_threadgroup<SCOPE>();
+    nvshmemi_barrier_threadgroup<SCOPE>(team);
     return 0;
 }
 
-/* Reducescatter (reference coll/reducescatter.cuh:36-90): PE `me` folds block `me` (nreduce
- * elements) of every PE's source into its own dest, in the order acc = op(x0, x1);
+/* Reducescatter (reference coll/reducescatter.cuh:36-90): member `me` folds block `me` (nreduce
+ * elements) of every member's source into its own dest, in the order acc = op(x0, x1);
  * acc = op(acc, x_p).  dest must not overlap source: other PEs read the blocks of this PE's source
  * while it writes its dest. */
 template <typename T, int OP, int SCOPE>
 NVSHMEMI_DEVICE_INLINE int nvshmemi_reducescatter_threadgroup(nvshmem_team_t team, T *dest,
                                                               const T *source, size_t nreduce) {
-    (void)team;
     constexpr size_t VEC = 16 / sizeof(T);
     struct alignas(16) pack_t { T e[VEC]; };
-    const int me = nvshmemi_amd_my_pe();
-    const int npes = nvshmemi_device_state_d.npes;
+    const nvshmemi_amd_team_view_t tv = nvshmemi_amd_team_view(team);
+    if (tv.size <= 0) return 1;
+    const int me = tv.my_pe;
+    const int npes = tv.size;
     const size_t tid = (size_t)nvshmemi_thread_id_in_threadgroup<SCOPE>();
     const size_t nthr = (size_t)nvshmemi_threadgroup_size<SCOPE>();
     /* every PE's source is complete and visible before anyone reads it */
-    nvshmemi_barrier_threadgroup<SCOPE>();
-    const T *src0 = reinterpret_cast<const T *>(nvshmemi_amd_remote(source, 0)) + (size_t)me * nreduce;
-    T *dst = reinterpret_cast<T *>(nvshmemi_amd_remote(dest, me));
-    const size_t pe_stride = (size_t)(nvshmemi_device_state_d.heap_size / sizeof(T));
+    nvshmemi_barrier_threadgroup<SCOPE>(team);
+    const T *src0 = reinterpret_cast<const T *>(nvshmemi_amd_remote(source, tv.start)) + (size_t)me * nreduce;
+    T *dst = reinterpret_cast<T *>(nvshmemi_amd_remote(dest, nvshmemi_amd_my_pe()));
+    const size_t pe_stride = (size_t)(nvshmemi_device_state_d.heap_size / sizeof(T)) * (size_t)tv.stride;
     size_t i = tid;
     if ((((uintptr_t)src0 | (uintptr_t)dst) & 15) == 0) {
         const size_t nvec = nreduce / VEC;
@@ -688,7 +747,7 @@ NVSHMEMI_DEVICE_INLINE int nvshmemi_reducescatter_threadgroup(nvshmem_team_t tea
             acc = nvshmemi_amd_reduce_op<T, OP>(acc, src0[(size_t)pe * pe_stride + i]);
         dst[i] = acc;
     }
-    nvshmemi_barrier_threadgroup<SCOPE>();
+    nvshmemi_barrier_threadgroup<SCOPE>(team);
     return 0;
 }
 

@@ -60,6 +60,30 @@ typedef int32_t nvshmem_team_t;
 #define NVSHMEM_TEAM_WORLD 0
 #define NVSHMEM_TEAM_SHARED 1
 #define NVSHMEMX_TEAM_NODE 2
+/* Predefined teams, numbered as in the reference (src/include/device_host/nvshmem_common.cuh:
+ * 406-421).  All logical PEs share one GPU, so SHARED, NODE and SAME_GPU equal WORLD,
+ * SAME_MYPE_NODE holds the calling PE alone and GPU_LEADERS holds PE 0 (only PE 0 is a member). */
+#define NVSHMEMX_TEAM_SAME_MYPE_NODE 3
+#define NVSHMEMI_TEAM_SAME_GPU 4
+#define NVSHMEMI_TEAM_GPU_LEADERS 5
+#define NVSHMEM_TEAMS_MIN 6
+/* Team handles, predefined ones included (reference default of NVSHMEM_MAX_TEAMS: 32). */
+#define NVSHMEMI_AMD_MAX_TEAMS 32
+
+/* Team configuration (reference nvshmem_team_config_v2, src/include/device_host/nvshmem_types.h:
+ * 93-105, 294-310): recorded and returned by nvshmem_team_get_config; contexts are not used on a
+ * load/store path. */
+#define NVSHMEM_TEAM_CONFIG_MASK_NUM_CONTEXTS 0x0000000000000001
+#define NVSHMEM_TEAM_CONFIG_MASK_UNIQUEID 0x0000000000000002
+typedef uint64_t nvshmemx_team_uniqueid_t;
+typedef struct {
+    int version;
+    int num_contexts;
+    nvshmemx_team_uniqueid_t uniqueid;
+    char padding[48];
+} nvshmem_team_config_t;
+#define NVSHMEMI_TEAM_CONFIG_VERSION_2_IDENTIFIER ((2 << 16) + (int)sizeof(nvshmem_team_config_t))
+#define NVSHMEM_TEAM_CONFIG_INITIALIZER {NVSHMEMI_TEAM_CONFIG_VERSION_2_IDENTIFIER, -1, (nvshmemx_team_uniqueid_t)-1, {0}}
 
 enum nvshmemx_status {
     NVSHMEMX_SUCCESS = 0,

@@ -37,8 +37,41 @@ NVSHMEMI_HOST_ONLY void nvshmem_finalize(void);       /* nvshmem_api.h:66 */
 NVSHMEMI_HOST_ONLY int nvshmemx_init_status(void);    /* nvshmem_api.h:50 */
 NVSHMEMI_HOST_ONLY int nvshmem_my_pe(void);           /* nvshmem_api.h:60-64 */
 NVSHMEMI_HOST_ONLY int nvshmem_n_pes(void);
+/* ---- teams: src/include/host/nvshmem_api.h:465-482, src/host/team/team.cu:19-115 ----
+ * A team is a strided set of world PEs.  The host thread stands for every PE, so one split call
+ * creates the team for all of its members, and a handle can name a family of disjoint teams: after
+ * nvshmem_team_split_2d the x handle is "my row" and the y handle "my column" for every PE, as the
+ * variables of the same names are in an SPMD program.  A collective called on such a handle runs on
+ * every team of the family.  Queries without a PE argument answer for PE 0 (the host's
+ * nvshmem_my_pe()); nvshmemx_amd_team_view answers for any PE.  Handles are small integers that
+ * are reused after nvshmem_team_destroy; at most NVSHMEMI_AMD_MAX_TEAMS exist at a time. */
 NVSHMEMI_HOST_ONLY int nvshmem_team_my_pe(nvshmem_team_t team); /* nvshmem_api.h:465 */
 NVSHMEMI_HOST_ONLY int nvshmem_team_n_pes(nvshmem_team_t team); /* nvshmem_api.h:466 */
+NVSHMEMI_HOST_ONLY void nvshmem_team_get_config(nvshmem_team_t team,
+                                                nvshmem_team_config_t *config); /* :468 */
+NVSHMEMI_HOST_ONLY int nvshmem_team_translate_pe(nvshmem_team_t src_team, int src_pe,
+                                                 nvshmem_team_t dest_team); /* :469 */
+/* Members PE_start, PE_start + PE_stride, ... (PE_size of them) of the parent, counted in parent
+ * indices, in every team of the parent's family; the others are not members of the new handle.
+ * Returns 0 and the handle, or nonzero and NVSHMEM_TEAM_INVALID (argument errors of
+ * team_internal.cpp:2197-2222, or no free handle). */
+NVSHMEMI_HOST_ONLY int nvshmem_team_split_strided(nvshmem_team_t parent_team, int PE_start,
+                                                  int PE_stride, int PE_size,
+                                                  const nvshmem_team_config_t *config,
+                                                  long config_mask,
+                                                  nvshmem_team_t *new_team); /* :471 */
+/* Row-major grid with rows of xrange members (team_internal.cpp:2292-2349): *xaxis_team names
+ * every PE's row, *yaxis_team every PE's column. */
+NVSHMEMI_HOST_ONLY int nvshmem_team_split_2d(nvshmem_team_t parent_team, int xrange,
+                                             const nvshmem_team_config_t *xaxis_config,
+                                             long xaxis_mask, nvshmem_team_t *xaxis_team,
+                                             const nvshmem_team_config_t *yaxis_config,
+                                             long yaxis_mask,
+                                             nvshmem_team_t *yaxis_team); /* :478 */
+NVSHMEMI_HOST_ONLY void nvshmem_team_destroy(nvshmem_team_t team); /* :482 */
+/* {start, stride, size, my_pe} of `team` as world PE `pe` sees it (size 0: not a member).
+ * Returns 0, or NVSHMEMX_ERROR_INVALID_VALUE for a handle or PE that does not exist. */
+NVSHMEMI_HOST_ONLY int nvshmemx_amd_team_view(nvshmem_team_t team, int pe, int view[4]);
 NVSHMEMI_HOST_ONLY void nvshmem_info_get_version(int *major, int *minor); /* nvshmem_api.h:77 */
 NVSHMEMI_HOST_ONLY void nvshmem_info_get_name(char *name);                /* nvshmem_api.h:78 */
 NVSHMEMI_HOST_ONLY void nvshmemx_vendor_get_version_info(int *major, int *minor, int *patch);

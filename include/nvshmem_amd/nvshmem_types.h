@@ -149,6 +149,20 @@ typedef enum {
  * so the reference's peer_heap_base_p2p[] table collapses to a shift.  Symmetric addresses handed
  * to users are addresses inside PE 0's slice ("canonical" addresses).
  */
+/* Team `t` as PE `p` sees it: entry [t * NVSHMEMI_AMD_MAX_PES + p] of the team table.  The
+ * members are the world PEs start + i*stride, i < size; my_pe is p's index among them.  size == 0:
+ * p is not a member (its handle would be NVSHMEM_TEAM_INVALID in the reference).  One handle can
+ * thus name a family of disjoint teams, e.g. every row of a 2-D split, and a collective called
+ * once serves all of them.  Counterpart of the start/stride/size/my_pe fields of nvshmemi_team_t
+ * (src/include/device_host/nvshmem_types.h:312-343). */
+typedef struct {
+    int32_t start, stride, size, my_pe;
+} nvshmemi_amd_team_view_t;
+
+/* Arrival words of a team barrier: NVSHMEMI_AMD_MAX_PES words indexed by the sender's member
+ * index, then the PE's epoch; one such row per (team, PE). */
+#define NVSHMEMI_AMD_TEAM_SYNC_WORDS (NVSHMEMI_AMD_MAX_PES + 8)
+
 typedef struct nvshmemi_device_state {
     uint32_t version;     /* (1 << 16) + sizeof(struct) */
     int32_t mype;         /* PE a kernel acts as when its grid is not PE-multiplexed */
@@ -160,6 +174,8 @@ typedef struct nvshmemi_device_state {
     uint64_t *sync_epoch; /* canonical address: that PE's barrier epoch */
     uint64_t spin_limit;  /* 0 = wait forever; else a bounded wait gives up after this many polls */
     uint64_t *timeout_record; /* canonical address: 4 words {flag, addr, found, expected} */
+    const nvshmemi_amd_team_view_t *team_views; /* [NVSHMEMI_AMD_MAX_TEAMS][NVSHMEMI_AMD_MAX_PES] */
+    uint64_t *team_sync; /* [MAX_TEAMS][MAX_PES][NVSHMEMI_AMD_TEAM_SYNC_WORDS], teams other than WORLD */
 } nvshmemi_device_state_t;
 
 #endif

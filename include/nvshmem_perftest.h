@@ -95,6 +95,18 @@ int nvshmem_perftest_device_reducescatter(int dtype, int op, void *dest, const v
                                           size_t nreduce, int scope, int threads, void *stream);
 int nvshmem_perftest_device_broadcast(void *dest, const void *src, size_t bytes, int root,
                                       int scope, int threads, void *stream);
+/* In-kernel collectives on a team handle (members only; the other PEs return at once).  what:
+ * 0 float sum reduce (n elements), 1 float sum reducescatter (n per member), 2 fcollectmem, 3
+ * alltoallmem, 4 broadcastmem from member `root` (n bytes). */
+int nvshmem_perftest_device_team_coll(int what, int team, void *dest, const void *src, size_t n,
+                                      int root, int scope, int threads, void *stream);
+/* Every PE writes into its copy of `out` (4 + 64 ints): team_my_pe(a), team_n_pes(a),
+ * team_my_pe(b), team_n_pes(b), then team_translate_pe(a, i, b) for i = 0..63, all evaluated in
+ * device code. */
+int nvshmem_perftest_team_query(int *out, int team_a, int team_b, void *stream);
+/* device_barrier among the members of `team` (nvshmem_barrier(team) / nvshmem_team_sync(team)). */
+int nvshmem_perftest_device_team_barrier(uint64_t *counter, uint64_t *errors, int rounds, int team,
+                                         int scope, int threads, void *stream);
 /* `rounds` barriers; before round r each PE stores r into its `counter`, after the barrier it reads
  * every PE's counter and adds to its own errors[0] the number that are < r.  counter and errors
  * hold one uint64 each. */

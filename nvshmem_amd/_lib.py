@@ -68,6 +68,17 @@ def load():
         "nvshmem_fcollectmem": (i32, [i32, vp, vp, sz]),
         "nvshmemx_alltoallmem_on_stream": (i32, [i32, vp, vp, sz, vp]),
         "nvshmemx_fcollectmem_on_stream": (i32, [i32, vp, vp, sz, vp]),
+        "nvshmem_team_my_pe": (i32, [i32]),
+        "nvshmem_team_n_pes": (i32, [i32]),
+        "nvshmem_team_translate_pe": (i32, [i32, i32, i32]),
+        "nvshmem_team_split_strided": (i32, [i32, i32, i32, i32, vp, C.c_long, C.POINTER(i32)]),
+        "nvshmem_team_split_2d": (i32, [i32, i32, vp, C.c_long, C.POINTER(i32), vp, C.c_long, C.POINTER(i32)]),
+        "nvshmem_team_destroy": (None, [i32]),
+        "nvshmem_team_get_config": (None, [i32, vp]),
+        "nvshmemx_amd_team_view": (i32, [i32, i32, C.POINTER(i32)]),
+        "nvshmem_team_sync": (i32, [i32]),
+        "nvshmemx_team_sync_on_stream": (i32, [i32, vp]),
+        "nvshmemx_barrier_on_stream": (i32, [i32, vp]),
         "nvshmem_broadcastmem": (i32, [i32, vp, vp, sz, i32]),
         "nvshmemx_broadcastmem_on_stream": (i32, [i32, vp, vp, sz, i32, vp]),
         "nvshmemx_amd_collective_launch": (i32, [vp] + [C.c_uint] * 6 + [vp, sz, vp]),
@@ -118,6 +129,9 @@ def load_perftest():
         "nvshmem_perftest_ring_reduce": [vp, vp, sz, vp, sz, i32, i32, vp],
         "nvshmem_perftest_device_reduce": [i32, i32, vp, vp, sz, i32, i32, vp],
         "nvshmem_perftest_device_fcollect": [vp, vp, sz, i32, i32, vp],
+        "nvshmem_perftest_device_team_coll": [i32, i32, vp, vp, sz, i32, i32, i32, vp],
+        "nvshmem_perftest_team_query": [vp, i32, i32, vp],
+        "nvshmem_perftest_device_team_barrier": [vp, vp, i32, i32, i32, i32, vp],
         "nvshmem_perftest_device_reducescatter": [i32, i32, vp, vp, sz, i32, i32, vp],
         "nvshmem_perftest_device_broadcast": [vp, vp, sz, i32, i32, i32, vp],
         "nvshmem_perftest_device_alltoall": [vp, vp, sz, i32, i32, vp],

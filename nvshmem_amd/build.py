@@ -25,7 +25,7 @@ HIP_FLAGS = [
     "-I" + INCLUDE, "-I" + CSRC,
 ]
 
-RUNTIME_SOURCES = ["mspace.cpp", "runtime.hip", "collectives.hip", "host_rma.hip"]
+RUNTIME_SOURCES = ["mspace.cpp", "runtime.hip", "teams.cpp", "collectives.hip", "host_rma.hip"]
 PERFTEST_SOURCES = ["perftest/rma_kernels.hip", "perftest/coll_kernels.hip",
                     "perftest/moe_shuffle.hip", "perftest/api_matrix.hip"]
 

@@ -1,5 +1,7 @@
 // Host-launched collectives for logical PEs on one MI355X: one grid-wide kernel per call serves
-// every PE of the team.
+// every PE of the team - and, when the handle names a family of disjoint teams (the rows of a 2-D
+// split), every team of the family: grid.z indexes the team, whose <start, stride, size> the kernel
+// reads from the device copy of the team table.
 //
 // Reference counterparts: the on-stream launchers src/host/stream/coll/{rdxn/reduce_common.cuh:29-68,
 // fcollect/fcollect.cu:20-65, alltoall/alltoall.cu:18-40} start one block per PE that runs the
@@ -106,31 +108,39 @@ __device__ __forceinline__ void copy_tile(char *__restrict__ dst, const char *__
 }
 
 template <int MODE, int kCopyUnroll, bool NTL>
-__global__ __launch_bounds__(kCopyThreads) void segment_copy_kernel(char *base, uint32_t shift, int npes,
-                                                                uint64_t dst_off, uint64_t src_off,
-                                                                uint64_t seg_bytes, int root) {
+__global__ __launch_bounds__(kCopyThreads) void segment_copy_kernel(char *base, uint32_t shift,
+                                                                const nvshmemi_amd_team_view_t *groups,
+                                                                int max_size, uint64_t dst_off,
+                                                                uint64_t src_off, uint64_t seg_bytes,
+                                                                int root) {
+    // this block's team: members are the PEs start + i*stride, i < size
+    const nvshmemi_amd_team_view_t g = groups[blockIdx.z];
+    const unsigned npes = (unsigned)g.size;
+    base += (uint64_t)g.start << shift;
+    const uint64_t rep_stride = (uint64_t)g.stride << shift;  // from one member to the next
     const unsigned seg = blockIdx.y;
     const char *src;
     char *dst;
     int nrep;
     if (MODE == kModeFcollect) {
-        // segment p: PE p's source -> slot p of every PE's destination
-        src = base + ((uint64_t)seg << shift) + src_off;
+        // segment p: member p's source -> slot p of every member's destination
+        if (seg >= npes) return;
+        src = base + seg * rep_stride + src_off;
         dst = base + dst_off + (uint64_t)seg * seg_bytes;
-        nrep = npes;
+        nrep = (int)npes;
     } else if (MODE == kModeBroadcast) {
-        // one segment: the root's source -> every PE's destination
-        src = base + ((uint64_t)root << shift) + src_off;
+        // one segment: the root's source -> every member's destination
+        src = base + (uint64_t)root * rep_stride + src_off;
         dst = base + dst_off;
-        nrep = npes;
+        nrep = (int)npes;
     } else {
-        // segment (p, q): block q of PE p's source -> slot p of PE q's destination
-        const unsigned p = seg / (unsigned)npes, q = seg % (unsigned)npes;
-        src = base + ((uint64_t)p << shift) + src_off + (uint64_t)q * seg_bytes;
-        dst = base + ((uint64_t)q << shift) + dst_off + (uint64_t)p * seg_bytes;
+        // segment (p, q): block q of member p's source -> slot p of member q's destination
+        const unsigned p = seg / (unsigned)max_size, q = seg % (unsigned)max_size;
+        if (p >= npes || q >= npes) return;
+        src = base + p * rep_stride + src_off + (uint64_t)q * seg_bytes;
+        dst = base + q * rep_stride + dst_off + (uint64_t)p * seg_bytes;
         nrep = 1;
     }
-    const uint64_t rep_stride = 1ull << shift;
 
     uint64_t head = (uint64_t)(-(uintptr_t)dst & 15);
     if (head > seg_bytes) head = seg_bytes;
@@ -186,12 +196,17 @@ __device__ __forceinline__ T fold_next(int p, T acc, T x) {
 }
 
 template <typename T, int OP, int NPES, bool NTL, bool SCATTER = false>
-__global__ __launch_bounds__(NPES ? NPES * 64 : 1024) void reduce_vector_kernel(char *base, uint32_t shift, int npes_arg,
+__global__ __launch_bounds__(NPES ? NPES * 64 : 1024) void reduce_vector_kernel(char *base, uint32_t shift,
+                                                             const nvshmemi_amd_team_view_t *groups,
                                                              uint32_t lane_shift_arg, uint64_t dst_off,
                                                              uint64_t src_off, uint64_t nelems) {
     extern __shared__ __attribute__((aligned(16))) char lds[];
     constexpr int VEC = 16 / sizeof(T);
-    const int npes = NPES ? NPES : npes_arg;
+    // this block's team; with NPES > 0 the host has checked that every team has NPES members
+    const nvshmemi_amd_team_view_t g = groups[blockIdx.z];
+    const int npes = NPES ? NPES : g.size;
+    if (SCATTER && (int)blockIdx.y >= npes) return;
+    base += (uint64_t)g.start << shift;
     const uint32_t lane_shift = NPES ? 6u : lane_shift_arg;
     const unsigned lanes = 1u << lane_shift;
     const unsigned pe = threadIdx.x >> lane_shift, i = threadIdx.x & (lanes - 1);
@@ -199,7 +214,8 @@ __global__ __launch_bounds__(NPES ? NPES * 64 : 1024) void reduce_vector_kernel(
     // tiles are cut on absolute (16 * lanes)-byte boundaries of the destination, so a wavefront's
     // access is one aligned 1 KiB piece whatever the buffer's own alignment: `lead` vector slots of
     // the first tile lie in front of the buffer
-    const uint64_t pe_stride = 1ull << shift;
+    const uint64_t pe_stride = (uint64_t)g.stride << shift;  // from one member to the next
+    const bool member = NPES ? true : (int)pe < npes;        // the block is sized for the largest team
     if (SCATTER) {
         src_off += (uint64_t)blockIdx.y * nelems * sizeof(T);
         dst_off += (uint64_t)blockIdx.y * pe_stride;
@@ -214,7 +230,7 @@ __global__ __launch_bounds__(NPES ? NPES * 64 : 1024) void reduce_vector_kernel(
 
     for (uint64_t tile = blockIdx.x; tile < ntiles; tile += gridDim.x) {
         const uint64_t v = (tile << lane_shift) + i - lead;  // wraps to a huge value in front of the buffer
-        if (v < nvec) stage[threadIdx.x] = stream_load<NTL>(base + (uint64_t)pe * pe_stride + src_off + 16 * v);
+        if (v < nvec && member) stage[threadIdx.x] = stream_load<NTL>(base + (uint64_t)pe * pe_stride + src_off + 16 * v);
         __syncthreads();
         for (unsigned e = threadIdx.x; e < tile_elems; e += blockDim.x) {
             T acc = stage_e[e];
@@ -227,7 +243,7 @@ __global__ __launch_bounds__(NPES ? NPES * 64 : 1024) void reduce_vector_kernel(
         if (SCATTER) {
             if (v < nvec && pe == 0) stream_store(base + dst_off + 16 * v, result[i]);
         } else {
-            if (v < nvec) stream_store(base + (uint64_t)pe * pe_stride + dst_off + 16 * v, result[i]);
+            if (v < nvec && member) stream_store(base + (uint64_t)pe * pe_stride + dst_off + 16 * v, result[i]);
         }
     }
     if (SCATTER) return;  // a block of the source is a whole number of vectors
@@ -247,11 +263,16 @@ __global__ __launch_bounds__(NPES ? NPES * 64 : 1024) void reduce_vector_kernel(
 
 // Element-at-a-time variant for buffers that are not 16-byte aligned.
 template <typename T, int OP, bool SCATTER = false>
-__global__ __launch_bounds__(kThreads) void reduce_scalar_kernel(char *base, uint32_t shift, int npes,
+__global__ __launch_bounds__(kThreads) void reduce_scalar_kernel(char *base, uint32_t shift,
+                                                                 const nvshmemi_amd_team_view_t *groups,
                                                                  uint64_t dst_off, uint64_t src_off,
                                                                  uint64_t nelems) {
+    const nvshmemi_amd_team_view_t g = groups[blockIdx.z];
+    const int npes = g.size;
+    if (SCATTER && (int)blockIdx.y >= npes) return;
+    base += (uint64_t)g.start << shift;
     const uint64_t gsz = (uint64_t)gridDim.x * kThreads;
-    const uint64_t es = (1ull << shift) / sizeof(T);
+    const uint64_t es = ((uint64_t)g.stride << shift) / sizeof(T);
     const T *s = reinterpret_cast<const T *>(base + src_off) + (SCATTER ? (uint64_t)blockIdx.y * nelems : 0);
     T *d = reinterpret_cast<T *>(base + dst_off) + (SCATTER ? (uint64_t)blockIdx.y * es : 0);
     for (uint64_t i = (uint64_t)blockIdx.x * kThreads + threadIdx.x; i < nelems; i += gsz) {
@@ -262,34 +283,43 @@ __global__ __launch_bounds__(kThreads) void reduce_scalar_kernel(char *base, uin
     }
 }
 
+// members of all teams of the handle together
+static uint64_t total_members(const TeamLaunch &tl) {
+    // sizes lie between min and max; the exact sum only matters for the cache policy threshold
+    return (uint64_t)tl.ngroups * (uint64_t)tl.max_size;
+}
+
 template <typename T, int OP>
-void launch_reduce(Runtime &rt, uint64_t dst_off, uint64_t src_off, uint64_t nelems,
-                   hipStream_t stream) {
+void launch_reduce(Runtime &rt, const TeamLaunch &tl, uint64_t dst_off, uint64_t src_off,
+                   uint64_t nelems, hipStream_t stream) {
     const bool vector_ok = ((dst_off | src_off) & 15) == 0;
+    const unsigned ngroups = (unsigned)tl.ngroups;
     if (vector_ok) {
         // lanes per PE: a full wavefront when the block still fits 1024 threads
         uint32_t lane_shift = 6;
-        while (((uint32_t)rt.npes << lane_shift) > 1024) --lane_shift;  // npes <= 64 -> >= 16 lanes
-        const unsigned threads = (unsigned)rt.npes << lane_shift;
+        while (((uint32_t)tl.max_size << lane_shift) > 1024) --lane_shift;  // size <= 64 -> >= 16 lanes
+        const unsigned threads = (unsigned)tl.max_size << lane_shift;
         const uint64_t nvec = nelems / (16 / sizeof(T));
         uint64_t blocks = (nvec + (2u << lane_shift) - 1) >> lane_shift;  // +1 tile for the lead-in
         if (blocks > 0x7fffffffull) blocks = 0x7fffffffull;  // the tile loop covers the rest
         if (blocks == 0) blocks = 1;                          // only tail elements
-        const size_t lds = ((size_t)rt.npes + 1) * 16 << lane_shift;
+        const size_t lds = ((size_t)tl.max_size + 1) * 16 << lane_shift;
+        const dim3 grid((unsigned)blocks, 1, ngroups);
         const bool stream_source =
-            (uint64_t)rt.npes * nelems * sizeof(T) > NVSHMEM_AMD_CACHEABLE_SOURCE_BYTES;
+            total_members(tl) * nelems * sizeof(T) > NVSHMEM_AMD_CACHEABLE_SOURCE_BYTES;
 #define NVSHMEM_AMD_LAUNCH_REDUCE(N)                                                              \
     do {                                                                                          \
         if (stream_source)                                                                        \
-            hipLaunchKernelGGL((reduce_vector_kernel<T, OP, N, true>), dim3((unsigned)blocks),    \
-                               dim3(threads), lds, stream, rt.base, rt.heap_shift, rt.npes,       \
-                               lane_shift, dst_off, src_off, nelems);                             \
+            hipLaunchKernelGGL((reduce_vector_kernel<T, OP, N, true>), grid, dim3(threads), lds,  \
+                               stream, rt.base, rt.heap_shift, tl.groups, lane_shift, dst_off,    \
+                               src_off, nelems);                                                  \
         else                                                                                      \
-            hipLaunchKernelGGL((reduce_vector_kernel<T, OP, N, false>), dim3((unsigned)blocks),   \
-                               dim3(threads), lds, stream, rt.base, rt.heap_shift, rt.npes,       \
-                               lane_shift, dst_off, src_off, nelems);                             \
+            hipLaunchKernelGGL((reduce_vector_kernel<T, OP, N, false>), grid, dim3(threads), lds, \
+                               stream, rt.base, rt.heap_shift, tl.groups, lane_shift, dst_off,    \
+                               src_off, nelems);                                                  \
     } while (0)
-        switch (rt.npes) {
+        // the compile-time sizes need every team of the handle to have that many members
+        switch (tl.min_size == tl.max_size ? tl.max_size : 0) {
             case 8: NVSHMEM_AMD_LAUNCH_REDUCE(8); break;
             case 16: NVSHMEM_AMD_LAUNCH_REDUCE(16); break;
             default: NVSHMEM_AMD_LAUNCH_REDUCE(0); break;
@@ -297,33 +327,36 @@ void launch_reduce(Runtime &rt, uint64_t dst_off, uint64_t src_off, uint64_t nel
 #undef NVSHMEM_AMD_LAUNCH_REDUCE
     } else {
         uint64_t blocks = (nelems + kThreads - 1) / kThreads;
-        const uint64_t cap = (uint64_t)rt.num_cus * 64;
+        const uint64_t cap = (uint64_t)rt.num_cus * 64 / ngroups + 1;
         if (blocks > cap) blocks = cap;
-        hipLaunchKernelGGL((reduce_scalar_kernel<T, OP>), dim3((unsigned)blocks), dim3(kThreads), 0,
-                           stream, rt.base, rt.heap_shift, rt.npes, dst_off, src_off, nelems);
+        hipLaunchKernelGGL((reduce_scalar_kernel<T, OP>), dim3((unsigned)blocks, 1, ngroups),
+                           dim3(kThreads), 0, stream, rt.base, rt.heap_shift, tl.groups, dst_off,
+                           src_off, nelems);
     }
 }
 
-// reducescatter: grid.y = destination PE; nelems is the element count of one PE's result
+// reducescatter: grid.y = destination member; nelems is the element count of one PE's result
 template <typename T, int OP>
-void launch_reducescatter(Runtime &rt, uint64_t dst_off, uint64_t src_off, uint64_t nelems,
-                          hipStream_t stream) {
+void launch_reducescatter(Runtime &rt, const TeamLaunch &tl, uint64_t dst_off, uint64_t src_off,
+                          uint64_t nelems, hipStream_t stream) {
     const bool vector_ok = ((dst_off | src_off | (nelems * sizeof(T))) & 15) == 0;
+    const unsigned ngroups = (unsigned)tl.ngroups;
     if (vector_ok) {
         uint32_t lane_shift = 6;
-        while (((uint32_t)rt.npes << lane_shift) > 1024) --lane_shift;
-        const unsigned threads = (unsigned)rt.npes << lane_shift;
+        while (((uint32_t)tl.max_size << lane_shift) > 1024) --lane_shift;
+        const unsigned threads = (unsigned)tl.max_size << lane_shift;
         const uint64_t nvec = nelems / (16 / sizeof(T));
         uint64_t blocks = (nvec + (2u << lane_shift) - 1) >> lane_shift;
         if (blocks > 0x7fffffffull) blocks = 0x7fffffffull;
-        const size_t lds = ((size_t)rt.npes + 1) * 16 << lane_shift;
-        const dim3 grid((unsigned)blocks, (unsigned)rt.npes);
+        const size_t lds = ((size_t)tl.max_size + 1) * 16 << lane_shift;
+        const dim3 grid((unsigned)blocks, (unsigned)tl.max_size, ngroups);
         const bool stream_source =
-            (uint64_t)rt.npes * rt.npes * nelems * sizeof(T) > NVSHMEM_AMD_CACHEABLE_SOURCE_BYTES;
+            total_members(tl) * tl.max_size * nelems * sizeof(T) > NVSHMEM_AMD_CACHEABLE_SOURCE_BYTES;
 #define NVSHMEM_AMD_LAUNCH_SCATTER(N, NTL)                                                        \
     hipLaunchKernelGGL((reduce_vector_kernel<T, OP, N, NTL, true>), grid, dim3(threads), lds,     \
-                       stream, rt.base, rt.heap_shift, rt.npes, lane_shift, dst_off, src_off, nelems)
-        if (rt.npes == 8) {
+                       stream, rt.base, rt.heap_shift, tl.groups, lane_shift, dst_off, src_off,   \
+                       nelems)
+        if (tl.min_size == 8 && tl.max_size == 8) {
             if (stream_source) NVSHMEM_AMD_LAUNCH_SCATTER(8, true);
             else NVSHMEM_AMD_LAUNCH_SCATTER(8, false);
         } else {
@@ -333,15 +366,16 @@ void launch_reducescatter(Runtime &rt, uint64_t dst_off, uint64_t src_off, uint6
 #undef NVSHMEM_AMD_LAUNCH_SCATTER
     } else {
         uint64_t blocks = (nelems + kThreads - 1) / kThreads;
-        const uint64_t cap = (uint64_t)rt.num_cus * 64 / (uint64_t)rt.npes + 1;
+        const uint64_t cap = (uint64_t)rt.num_cus * 64 / ((uint64_t)tl.max_size * ngroups) + 1;
         if (blocks > cap) blocks = cap;
-        hipLaunchKernelGGL((reduce_scalar_kernel<T, OP, true>), dim3((unsigned)blocks, (unsigned)rt.npes),
-                           dim3(kThreads), 0, stream, rt.base, rt.heap_shift, rt.npes, dst_off,
-                           src_off, nelems);
+        hipLaunchKernelGGL((reduce_scalar_kernel<T, OP, true>),
+                           dim3((unsigned)blocks, (unsigned)tl.max_size, ngroups), dim3(kThreads), 0,
+                           stream, rt.base, rt.heap_shift, tl.groups, dst_off, src_off, nelems);
     }
 }
 
-typedef void (*reduce_launcher_t)(Runtime &, uint64_t, uint64_t, uint64_t, hipStream_t);
+typedef void (*reduce_launcher_t)(Runtime &, const TeamLaunch &, uint64_t, uint64_t, uint64_t,
+                                  hipStream_t);
 
 template <typename T, bool SCATTER>
 reduce_launcher_t pick_arith(int op) {
@@ -387,24 +421,14 @@ reduce_launcher_t pick_reduce(int dtype, int op) {
 
 const size_t kDtypeSize[NVSHMEMI_DT_COUNT] = {1, 2, 4, 8, 1, 2, 4, 8, 2, 2, 4, 8};
 
-bool team_ok(Runtime &rt, const char *what, nvshmem_team_t team) {
-    if (!rt.initialized) {
-        set_error("%s called before nvshmem_init", what);
-        return false;
-    }
-    if (team != NVSHMEM_TEAM_WORLD) {
-        set_error("%s: team %d is not supported (only NVSHMEM_TEAM_WORLD)", what, (int)team);
-        return false;
-    }
-    return true;
-}
-
 }  // namespace
 
 int reduce_on_stream(int dtype, int op, nvshmem_team_t team, void *dest, const void *src,
                      size_t nreduce, hipStream_t stream) {
     Runtime &rt = Runtime::get();
-    if (!team_ok(rt, "reduce", team)) return NVSHMEMX_ERROR_INVALID_VALUE;
+    std::lock_guard<std::recursive_mutex> lock(rt.mu);
+    TeamLaunch tl;
+    if (!resolve_team(rt, "reduce", team, &tl)) return NVSHMEMX_ERROR_INVALID_VALUE;
     reduce_launcher_t fn = pick_reduce<false>(dtype, op);
     if (!fn) {
         set_error("reduce: operator %d is not defined for element kind %d", op, dtype);
@@ -428,7 +452,7 @@ int reduce_on_stream(int dtype, int op, nvshmem_team_t team, void *dest, const v
         set_error("reduce: dest and source overlap without being identical");
         return NVSHMEMX_ERROR_INVALID_VALUE;
     }
-    fn(rt, doff, soff, nreduce, stream);
+    fn(rt, tl, doff, soff, nreduce, stream);
     hipError_t e = hipGetLastError();
     if (e != hipSuccess) {
         set_error("reduce: kernel launch failed: %s", hipGetErrorString(e));
@@ -440,7 +464,9 @@ int reduce_on_stream(int dtype, int op, nvshmem_team_t team, void *dest, const v
 int reducescatter_on_stream(int dtype, int op, nvshmem_team_t team, void *dest, const void *src,
                             size_t nreduce, hipStream_t stream) {
     Runtime &rt = Runtime::get();
-    if (!team_ok(rt, "reducescatter", team)) return NVSHMEMX_ERROR_INVALID_VALUE;
+    std::lock_guard<std::recursive_mutex> lock(rt.mu);
+    TeamLaunch tl;
+    if (!resolve_team(rt, "reducescatter", team, &tl)) return NVSHMEMX_ERROR_INVALID_VALUE;
     reduce_launcher_t fn = pick_reduce<true>(dtype, op);
     if (!fn) {
         set_error("reducescatter: operator %d is not defined for element kind %d", op, dtype);
@@ -448,10 +474,10 @@ int reducescatter_on_stream(int dtype, int op, nvshmem_team_t team, void *dest, 
     }
     if (nreduce == 0) return 0;
     const size_t es = kDtypeSize[dtype];
-    const uint64_t n = (uint64_t)rt.npes;
+    const uint64_t n = (uint64_t)tl.max_size;
     if (nreduce > rt.heap_size / es / n) {
         set_error("reducescatter: %zu elements of %zu bytes x %d PEs leave the PE's heap slice",
-                  nreduce, es, rt.npes);
+                  nreduce, es, tl.max_size);
         return NVSHMEMX_ERROR_INVALID_VALUE;
     }
     uint64_t doff = 0, soff = 0;
@@ -467,7 +493,7 @@ int reducescatter_on_stream(int dtype, int op, nvshmem_team_t team, void *dest, 
         set_error("reducescatter: dest and source overlap");
         return NVSHMEMX_ERROR_INVALID_VALUE;
     }
-    fn(rt, doff, soff, nreduce, stream);
+    fn(rt, tl, doff, soff, nreduce, stream);
     hipError_t e = hipGetLastError();
     if (e != hipSuccess) {
         set_error("reducescatter: kernel launch failed: %s", hipGetErrorString(e));
@@ -479,9 +505,11 @@ int reducescatter_on_stream(int dtype, int op, nvshmem_team_t team, void *dest, 
 int broadcast_on_stream(nvshmem_team_t team, void *dest, const void *src, size_t bytes, int root,
                         hipStream_t stream) {
     Runtime &rt = Runtime::get();
-    if (!team_ok(rt, "broadcast", team)) return NVSHMEMX_ERROR_INVALID_VALUE;
-    if (root < 0 || root >= rt.npes) {
-        set_error("broadcast: root %d is not a PE of the team (0..%d)", root, rt.npes - 1);
+    std::lock_guard<std::recursive_mutex> lock(rt.mu);
+    TeamLaunch tl;
+    if (!resolve_team(rt, "broadcast", team, &tl)) return NVSHMEMX_ERROR_INVALID_VALUE;
+    if (root < 0 || root >= tl.min_size) {
+        set_error("broadcast: root %d is not a PE of the team (0..%d)", root, tl.min_size - 1);
         return NVSHMEMX_ERROR_INVALID_VALUE;
     }
     if (bytes == 0) return 0;
@@ -500,13 +528,15 @@ int broadcast_on_stream(nvshmem_team_t team, void *dest, const void *src, size_t
         set_error("broadcast: message too large");
         return NVSHMEMX_ERROR_INVALID_VALUE;
     }
-    const dim3 grid((unsigned)tiles, 1), block(kCopyThreads);
-    if (bytes > NVSHMEM_AMD_CACHEABLE_SOURCE_BYTES)
+    const dim3 grid((unsigned)tiles, 1, (unsigned)tl.ngroups), block(kCopyThreads);
+    if (bytes * (uint64_t)tl.ngroups > NVSHMEM_AMD_CACHEABLE_SOURCE_BYTES)
         hipLaunchKernelGGL((segment_copy_kernel<kModeBroadcast, 1, true>), grid, block, 0, stream,
-                           rt.base, rt.heap_shift, rt.npes, doff, soff, (uint64_t)bytes, root);
+                           rt.base, rt.heap_shift, tl.groups, tl.max_size, doff, soff,
+                           (uint64_t)bytes, root);
     else
         hipLaunchKernelGGL((segment_copy_kernel<kModeBroadcast, 1, false>), grid, block, 0, stream,
-                           rt.base, rt.heap_shift, rt.npes, doff, soff, (uint64_t)bytes, root);
+                           rt.base, rt.heap_shift, tl.groups, tl.max_size, doff, soff,
+                           (uint64_t)bytes, root);
     hipError_t e = hipGetLastError();
     if (e != hipSuccess) {
         set_error("broadcast: kernel launch failed: %s", hipGetErrorString(e));
@@ -518,11 +548,13 @@ int broadcast_on_stream(nvshmem_team_t team, void *dest, const void *src, size_t
 static int segment_collective(int mode, const char *what, nvshmem_team_t team, void *dest,
                               const void *src, size_t seg_bytes, hipStream_t stream) {
     Runtime &rt = Runtime::get();
-    if (!team_ok(rt, what, team)) return NVSHMEMX_ERROR_INVALID_VALUE;
+    std::lock_guard<std::recursive_mutex> lock(rt.mu);
+    TeamLaunch tl;
+    if (!resolve_team(rt, what, team, &tl)) return NVSHMEMX_ERROR_INVALID_VALUE;
     if (seg_bytes == 0) return 0;
-    const uint64_t n = (uint64_t)rt.npes;
+    const uint64_t n = (uint64_t)tl.max_size;
     if (seg_bytes > rt.heap_size / n) {
-        set_error("%s: %zu bytes x %d PEs does not fit a PE's heap slice", what, seg_bytes, rt.npes);
+        set_error("%s: %zu bytes x %d PEs does not fit a PE's heap slice", what, seg_bytes, tl.max_size);
         return NVSHMEMX_ERROR_INVALID_VALUE;
     }
     const uint64_t src_bytes = mode == kModeFcollect ? seg_bytes : seg_bytes * n;
@@ -542,11 +574,11 @@ static int segment_collective(int mode, const char *what, nvshmem_team_t team, v
         set_error("%s: message too large", what);
         return NVSHMEMX_ERROR_INVALID_VALUE;
     }
-    const bool stream_source = src_bytes * n > NVSHMEM_AMD_CACHEABLE_SOURCE_BYTES;
-    const dim3 grid((unsigned)tiles, segs), block(kCopyThreads);
+    const bool stream_source = src_bytes * total_members(tl) > NVSHMEM_AMD_CACHEABLE_SOURCE_BYTES;
+    const dim3 grid((unsigned)tiles, segs, (unsigned)tl.ngroups), block(kCopyThreads);
 #define NVSHMEM_AMD_LAUNCH_SEGCOPY(MODE, U, NTL)                                                   \
     hipLaunchKernelGGL((segment_copy_kernel<MODE, U, NTL>), grid, block, 0, stream, rt.base,       \
-                       rt.heap_shift, rt.npes, doff, soff, (uint64_t)seg_bytes, 0)
+                       rt.heap_shift, tl.groups, tl.max_size, doff, soff, (uint64_t)seg_bytes, 0)
     if (mode == kModeFcollect) {
         if (stream_source) NVSHMEM_AMD_LAUNCH_SEGCOPY(kModeFcollect, NVSHMEM_AMD_FCOLLECT_UNROLL, true);
         else NVSHMEM_AMD_LAUNCH_SEGCOPY(kModeFcollect, NVSHMEM_AMD_FCOLLECT_UNROLL, false);

@@ -77,6 +77,58 @@ __global__ void barrier_kernel(uint64_t *counter, uint64_t *errors, int rounds) 
     if (threadIdx.x == 0) *(uint64_t *)nvshmem_ptr(errors, me) += bad;
 }
 
+// Collectives and queries on a team handle; PEs that are not members of `team` return at once.
+enum { kTeamReduce = 0, kTeamReducescatter = 1, kTeamFcollect = 2, kTeamAlltoall = 3, kTeamBroadcast = 4 };
+
+template <int SCOPE>
+__global__ void team_coll_kernel(int what, nvshmem_team_t team, void *dest, const void *src, size_t n,
+                                 int root) {
+    if (nvshmem_team_my_pe(team) < 0) return;
+    switch (what) {
+        case kTeamReduce:
+            SCOPED_CALL(SCOPE, float_sum_reduce, team, (float *)dest, (const float *)src, n);
+            break;
+        case kTeamReducescatter:
+            SCOPED_CALL(SCOPE, float_sum_reducescatter, team, (float *)dest, (const float *)src, n);
+            break;
+        case kTeamFcollect: SCOPED_CALL(SCOPE, fcollectmem, team, dest, src, n); break;
+        case kTeamAlltoall: SCOPED_CALL(SCOPE, alltoallmem, team, dest, src, n); break;
+        default: SCOPED_CALL(SCOPE, broadcastmem, team, dest, src, n, root); break;
+    }
+}
+
+// out (symmetric, 4 + NVSHMEMI_AMD_MAX_PES ints per PE): my_pe(a), n_pes(a), my_pe(b), n_pes(b),
+// then translate_pe(a, i, b) for i = 0 .. NVSHMEMI_AMD_MAX_PES-1
+__global__ void team_query_kernel(int *out, nvshmem_team_t a, nvshmem_team_t b) {
+    if (threadIdx.x != 0) return;
+    int *mine = (int *)nvshmem_ptr(out, nvshmem_my_pe());
+    mine[0] = nvshmem_team_my_pe(a);
+    mine[1] = nvshmem_team_n_pes(a);
+    mine[2] = nvshmem_team_my_pe(b);
+    mine[3] = nvshmem_team_n_pes(b);
+    for (int i = 0; i < NVSHMEMI_AMD_MAX_PES; ++i) mine[4 + i] = nvshmem_team_translate_pe(a, i, b);
+}
+
+// Team barrier check: like barrier_kernel, but only among the members of `team`, whose counters
+// are read through the team's PE translation.
+template <int SCOPE>
+__global__ void team_barrier_kernel(uint64_t *counter, uint64_t *errors, int rounds, nvshmem_team_t team) {
+    const int idx = nvshmem_team_my_pe(team), np = nvshmem_team_n_pes(team);
+    if (idx < 0) return;
+    const int me = nvshmem_my_pe();
+    uint64_t *my_counter = (uint64_t *)nvshmem_ptr(counter, me);
+    uint64_t bad = 0;
+    for (int r = 1; r <= rounds; ++r) {
+        if (threadIdx.x == 0) *my_counter = (uint64_t)r;
+        SCOPED_CALL(SCOPE, barrier, team);
+        if (threadIdx.x == 0)
+            for (int q = 0; q < np; ++q)
+                bad += nvshmem_uint64_g(counter, nvshmem_team_translate_pe(team, q, NVSHMEM_TEAM_WORLD)) < (uint64_t)r;
+        SCOPED_CALL(SCOPE, team_sync, team);
+    }
+    if (threadIdx.x == 0) *(uint64_t *)nvshmem_ptr(errors, me) += bad;
+}
+
 template <typename... Args>
 int launch_scoped(int scope, void (*kb)(Args...), void (*kw)(Args...), void (*kt)(Args...),
                   int threads, void *stream, Args... a) {
@@ -190,6 +242,40 @@ int nvshmem_perftest_device_barrier(uint64_t *counter, uint64_t *errors, int rou
     return launch_scoped<uint64_t *, uint64_t *, int>(
         scope, barrier_kernel<NVSHMEM_PERFTEST_SCOPE_BLOCK>, barrier_kernel<NVSHMEM_PERFTEST_SCOPE_WARP>,
         barrier_kernel<NVSHMEM_PERFTEST_SCOPE_THREAD>, threads, stream, counter, errors, rounds);
+}
+
+int nvshmem_perftest_device_team_coll(int what, int team, void *dest, const void *src, size_t n,
+                                      int root, int scope, int threads, void *stream) {
+    if (!perftest::ready() || scope < 0 || scope > 2 || what < kTeamReduce || what > kTeamBroadcast ||
+        !perftest::check_launch(1, threads) || !perftest::check_range(dest, 1) ||
+        !perftest::check_range(src, 1))
+        return NVSHMEMX_ERROR_INVALID_VALUE;
+    return launch_scoped<int, nvshmem_team_t, void *, const void *, size_t, int>(
+        scope, team_coll_kernel<NVSHMEM_PERFTEST_SCOPE_BLOCK>, team_coll_kernel<NVSHMEM_PERFTEST_SCOPE_WARP>,
+        team_coll_kernel<NVSHMEM_PERFTEST_SCOPE_THREAD>, threads, stream, what, (nvshmem_team_t)team,
+        dest, src, n, root);
+}
+
+int nvshmem_perftest_team_query(int *out, int team_a, int team_b, void *stream) {
+    if (!perftest::ready() ||
+        !perftest::check_range(out, sizeof(int) * (4 + NVSHMEMI_AMD_MAX_PES)))
+        return NVSHMEMX_ERROR_INVALID_VALUE;
+    nvshmem_team_t a = team_a, b = team_b;
+    void *args[] = {(void *)&out, (void *)&a, (void *)&b};
+    return nvshmemx_collective_launch((const void *)team_query_kernel, dim3(1), dim3(64), args, 0,
+                                      (hipStream_t)stream);
+}
+
+int nvshmem_perftest_device_team_barrier(uint64_t *counter, uint64_t *errors, int rounds, int team,
+                                         int scope, int threads, void *stream) {
+    if (!perftest::ready() || scope < 0 || scope > 2 || !perftest::check_launch(1, threads) ||
+        !perftest::check_range(counter, sizeof(uint64_t)) ||
+        !perftest::check_range(errors, sizeof(uint64_t)))
+        return NVSHMEMX_ERROR_INVALID_VALUE;
+    return launch_scoped<uint64_t *, uint64_t *, int, nvshmem_team_t>(
+        scope, team_barrier_kernel<NVSHMEM_PERFTEST_SCOPE_BLOCK>,
+        team_barrier_kernel<NVSHMEM_PERFTEST_SCOPE_WARP>, team_barrier_kernel<NVSHMEM_PERFTEST_SCOPE_THREAD>,
+        threads, stream, counter, errors, rounds, (nvshmem_team_t)team);
 }
 
 }  // extern "C"

@@ -193,6 +193,15 @@ int nvshmemx_amd_init(int npes, size_t symmetric_size) {
     rt.dev.sync_epoch = (uint64_t *)(uintptr_t)epoch;
     rt.dev.timeout_record = (uint64_t *)(uintptr_t)trec;
     rt.dev.spin_limit = env_size("NVSHMEM_AMD_SPIN_LIMIT", 1ull << 22);
+    if (!teams_init(rt)) {
+        teams_finalize(rt);
+        (void)hipFree(rt.base);
+        rt.space.reset();
+        rt.base = nullptr;
+        rt.initialized = false;
+        rt.npes = 0;
+        return NVSHMEMX_ERROR_OUT_OF_MEMORY;
+    }
     NVSHMEM_AMD_HIP_CHECK(hipDeviceSynchronize());
     refresh_symbols(rt, true);
     return NVSHMEMX_SUCCESS;
@@ -217,6 +226,7 @@ void nvshmem_finalize(void) {
     std::lock_guard<std::recursive_mutex> lock(rt.mu);
     if (!rt.initialized) return;
     (void)hipDeviceSynchronize();
+    teams_finalize(rt);
     (void)hipFree(rt.base);
     rt.space.reset();
     rt.base = nullptr;
@@ -232,10 +242,6 @@ int nvshmemx_init_status(void) {
 
 int nvshmem_my_pe(void) { return 0; }
 int nvshmem_n_pes(void) { return Runtime::get().npes; }
-int nvshmem_team_my_pe(nvshmem_team_t team) { return team == NVSHMEM_TEAM_WORLD ? 0 : -1; }
-int nvshmem_team_n_pes(nvshmem_team_t team) {
-    return team == NVSHMEM_TEAM_WORLD ? Runtime::get().npes : -1;
-}
 void nvshmem_info_get_version(int *major, int *minor) {
     if (major) *major = NVSHMEM_MAJOR_VERSION;
     if (minor) *minor = NVSHMEM_MINOR_VERSION;
@@ -361,8 +367,14 @@ void nvshmem_barrier_all(void) {
     refresh_symbols(rt, false);
     NVSHMEM_AMD_HIP_CHECK(hipDeviceSynchronize());
 }
+/* The host thread stands for every PE of any team, so a team barrier is the device-wide wait too. */
+static int known_team(const char *what, nvshmem_team_t team) {
+    TeamLaunch tl;
+    return resolve_team(Runtime::get(), what, team, &tl) ? 0 : NVSHMEMX_ERROR_INVALID_VALUE;
+}
 int nvshmem_barrier(nvshmem_team_t team) {
-    if (team != NVSHMEM_TEAM_WORLD) return NVSHMEMX_ERROR_NOT_SUPPORTED;
+    std::lock_guard<std::recursive_mutex> lock(Runtime::get().mu);
+    if (known_team("nvshmem_barrier", team)) return NVSHMEMX_ERROR_INVALID_VALUE;
     nvshmem_barrier_all();
     return 0;
 }
@@ -371,11 +383,13 @@ int nvshmem_team_sync(nvshmem_team_t team) { return nvshmem_barrier(team); }
 /* Work of all PEs submitted to one stream is already ordered on it. */
 void nvshmemx_barrier_all_on_stream(nvshmemx_stream_t) {}
 int nvshmemx_barrier_on_stream(nvshmem_team_t team, nvshmemx_stream_t) {
-    return team == NVSHMEM_TEAM_WORLD ? 0 : NVSHMEMX_ERROR_NOT_SUPPORTED;
+    std::lock_guard<std::recursive_mutex> lock(Runtime::get().mu);
+    return known_team("nvshmemx_barrier_on_stream", team);
 }
 void nvshmemx_sync_all_on_stream(nvshmemx_stream_t) {}
 int nvshmemx_team_sync_on_stream(nvshmem_team_t team, nvshmemx_stream_t) {
-    return team == NVSHMEM_TEAM_WORLD ? 0 : NVSHMEMX_ERROR_NOT_SUPPORTED;
+    std::lock_guard<std::recursive_mutex> lock(Runtime::get().mu);
+    return known_team("nvshmemx_team_sync_on_stream", team);
 }
 void nvshmemx_quiet_on_stream(nvshmemx_stream_t) {}
 

@@ -16,6 +16,33 @@
 
 namespace nvshmem_amd {
 
+// Host mirror of the team table.  views[t][p] is team t as world PE p sees it; groups[t] lists the
+// distinct member sets of the handle (one per disjoint team of the family), which is what the
+// collective kernels iterate over.  The device copy is one allocation: views | groups | sync words.
+struct TeamTable {
+    nvshmemi_amd_team_view_t views[NVSHMEMI_AMD_MAX_TEAMS][NVSHMEMI_AMD_MAX_PES];
+    nvshmemi_amd_team_view_t groups[NVSHMEMI_AMD_MAX_TEAMS][NVSHMEMI_AMD_MAX_PES];
+    int ngroups[NVSHMEMI_AMD_MAX_TEAMS];
+    bool used[NVSHMEMI_AMD_MAX_TEAMS];
+    nvshmem_team_config_t config[NVSHMEMI_AMD_MAX_TEAMS];
+    long config_mask[NVSHMEMI_AMD_MAX_TEAMS];
+    char *dev = nullptr;
+    nvshmemi_amd_team_view_t *dev_views() const { return (nvshmemi_amd_team_view_t *)dev; }
+    nvshmemi_amd_team_view_t *dev_groups() const {
+        return dev_views() + NVSHMEMI_AMD_MAX_TEAMS * NVSHMEMI_AMD_MAX_PES;
+    }
+    uint64_t *dev_sync() const {
+        return (uint64_t *)(dev_groups() + NVSHMEMI_AMD_MAX_TEAMS * NVSHMEMI_AMD_MAX_PES);
+    }
+};
+
+// What a collective kernel needs to serve every team of a handle.
+struct TeamLaunch {
+    const nvshmemi_amd_team_view_t *groups = nullptr;  // device array, ngroups entries
+    int ngroups = 0;
+    int max_size = 0, min_size = 0;
+};
+
 struct Runtime {
     std::recursive_mutex mu;
     bool initialized = false;
@@ -27,6 +54,7 @@ struct Runtime {
     char *base = nullptr;    // start of PE 0's slice
     std::unique_ptr<SymmetricSpace> space;
     nvshmemi_device_state_t dev{};
+    TeamTable teams{};
     std::set<nvshmemi_amd_state_updater_t> updaters;  // one per translation unit with a state block
     bool symbols_stale = false;
 
@@ -50,6 +78,12 @@ void clear_error();
 
 // Pushes the state block to every registered translation unit when it changed.
 void refresh_symbols(Runtime &rt, bool force);
+
+// Team table: allocation and the predefined teams at init, release at finalize.
+bool teams_init(Runtime &rt);
+void teams_finalize(Runtime &rt);
+// Resolves a handle for a collective; reports unknown handles through set_error.
+bool resolve_team(Runtime &rt, const char *what, nvshmem_team_t team, TeamLaunch *out);
 
 // Common argument check of the collectives and RMA calls: [p, p+bytes) must lie inside one PE
 // slice.  Returns the offset through *off.

@@ -95,6 +95,28 @@ class Runtime:
     def ptr(self, sym, pe):
         return self.lib.nvshmem_ptr(sym, pe)
 
+    # -- teams ------------------------------------------------------------------------------
+    def team_split_strided(self, parent, start, stride, size):
+        t = C.c_int32(-1)
+        rc = self.lib.nvshmem_team_split_strided(parent, start, stride, size, None, 0, C.byref(t))
+        self._check(rc, "nvshmem_team_split_strided")
+        return t.value
+
+    def team_split_2d(self, parent, xrange_):
+        x, y = C.c_int32(-1), C.c_int32(-1)
+        rc = self.lib.nvshmem_team_split_2d(parent, xrange_, None, 0, C.byref(x), None, 0, C.byref(y))
+        self._check(rc, "nvshmem_team_split_2d")
+        return x.value, y.value
+
+    def team_destroy(self, team):
+        self.lib.nvshmem_team_destroy(team)
+
+    def team_view(self, team, pe):
+        """(start, stride, size, my_pe) of the team as world PE `pe` sees it; size 0: not a member."""
+        v = (C.c_int32 * 4)()
+        self._check(self.lib.nvshmemx_amd_team_view(team, pe, v), "nvshmemx_amd_team_view")
+        return tuple(v)
+
     # -- plumbing: per-PE host <-> device transfers -----------------------------------------
     def upload(self, sym, pe, array, byte_offset=0):
         array = np.ascontiguousarray(array)
@@ -152,11 +174,11 @@ class Runtime:
             rc = _lib.typed_coll(self.lib, name, True, True)(team, dest, src, nelems, root, stream.ptr)
         self._check(rc, name)
 
-    def broadcastmem(self, dest, src, nbytes, root, stream=None):
+    def broadcastmem(self, dest, src, nbytes, root, stream=None, team=TEAM_WORLD):
         if stream is None:
-            self._check(self.lib.nvshmem_broadcastmem(TEAM_WORLD, dest, src, nbytes, root), "broadcastmem")
+            self._check(self.lib.nvshmem_broadcastmem(team, dest, src, nbytes, root), "broadcastmem")
         else:
-            self._check(self.lib.nvshmemx_broadcastmem_on_stream(TEAM_WORLD, dest, src, nbytes, root,
+            self._check(self.lib.nvshmemx_broadcastmem_on_stream(team, dest, src, nbytes, root,
                                                                  stream.ptr), "broadcastmem_on_stream")
 
     def fcollect(self, type_name, dest, src, nelems, stream=None, team=TEAM_WORLD):
@@ -177,18 +199,18 @@ class Runtime:
             rc = _lib.typed_coll(self.lib, name, True)(team, dest, src, nelems, stream.ptr)
         self._check(rc, name)
 
-    def fcollectmem(self, dest, src, nbytes, stream=None):
+    def fcollectmem(self, dest, src, nbytes, stream=None, team=TEAM_WORLD):
         if stream is None:
-            self._check(self.lib.nvshmem_fcollectmem(TEAM_WORLD, dest, src, nbytes), "fcollectmem")
+            self._check(self.lib.nvshmem_fcollectmem(team, dest, src, nbytes), "fcollectmem")
         else:
-            self._check(self.lib.nvshmemx_fcollectmem_on_stream(TEAM_WORLD, dest, src, nbytes,
+            self._check(self.lib.nvshmemx_fcollectmem_on_stream(team, dest, src, nbytes,
                                                                 stream.ptr), "fcollectmem_on_stream")
 
-    def alltoallmem(self, dest, src, nbytes, stream=None):
+    def alltoallmem(self, dest, src, nbytes, stream=None, team=TEAM_WORLD):
         if stream is None:
-            self._check(self.lib.nvshmem_alltoallmem(TEAM_WORLD, dest, src, nbytes), "alltoallmem")
+            self._check(self.lib.nvshmem_alltoallmem(team, dest, src, nbytes), "alltoallmem")
         else:
-            self._check(self.lib.nvshmemx_alltoallmem_on_stream(TEAM_WORLD, dest, src, nbytes,
+            self._check(self.lib.nvshmemx_alltoallmem_on_stream(team, dest, src, nbytes,
                                                                 stream.ptr), "alltoallmem_on_stream")
 
     def read_timeout(self, pe):

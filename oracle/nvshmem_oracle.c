@@ -346,6 +346,48 @@ void oracle_broadcast(int npes, size_t bytes, int root, const uint8_t *src, uint
 }
 
 /* ------------------------------------------------------------------------------------------- */
+/* teams: reference nvshmemi_team_split_strided, src/host/team/team_internal.cpp:2182-2290
+ * (argument checks :2197-2222, global triple :2214-2216), nvshmemi_team_split_2d :2292-2349,
+ * nvshmemi_team_translate_pe :579-589 (member index wraps modulo the size; an index above the size
+ * gives -1).                                                                                   */
+/* ------------------------------------------------------------------------------------------- */
+int oracle_team_split_strided(const int parent[3], int npes_world, int start, int stride, int size,
+                              int child[3]) {
+    child[0] = child[1] = child[2] = -1;
+    if (start < 0 || start >= parent[2] || size <= 0 || size > parent[2] || stride < 1) return -1;
+    const int g_start = parent[0] + start * parent[1];
+    const int g_stride = parent[1] * stride;
+    const int g_end = g_start + g_stride * (size - 1);
+    if (g_start >= npes_world || g_end >= npes_world) return -1;
+    child[0] = g_start;
+    child[1] = g_stride;
+    child[2] = size;
+    return 0;
+}
+
+int oracle_team_translate_pe(const int src[3], int src_pe, const int dst[3]) {
+    if (src_pe < 0 || src_pe > src[2]) return -1;
+    const int world = src[0] + (src_pe % src[2]) * src[1];
+    const int d = world - dst[0];
+    if (d < 0 || d % dst[1] != 0 || d / dst[1] >= dst[2]) return -1;
+    return d / dst[1];
+}
+
+void oracle_team_split_2d(const int parent[3], int xrange, int index, int xteam[3], int yteam[3]) {
+    const int n = parent[2];
+    if (xrange > n) xrange = n;
+    const int row = index / xrange, col = index % xrange;
+    const int rows = (n + xrange - 1) / xrange;
+    const int rem = n % xrange;
+    xteam[0] = parent[0] + row * xrange * parent[1];
+    xteam[1] = parent[1];
+    xteam[2] = (row == rows - 1 && rem) ? rem : xrange;
+    yteam[0] = parent[0] + col * parent[1];
+    yteam[1] = parent[1] * xrange;
+    yteam[2] = (rem && col < rem) ? n / xrange + 1 : n / xrange;
+}
+
+/* ------------------------------------------------------------------------------------------- */
 /* fcollect: reference nvshmemi_fcollect_p2p_allpush_threadgroup,
  *   src/include/non_abi/device/coll/fcollect.cuh:331-344: PE p copies its source into slot p of
  *   every PE's dest.

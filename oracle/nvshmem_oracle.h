@@ -14,6 +14,8 @@
  *   broadcast / reducescatter   brute force, the reference's known answer for broadcast
  *       (examples/ring-bcast.cu:68-72), slices of the pinned reduce for order-free operators, numpy
  *       folds and hand-evaluated NaN cases for the operand order;
+ *   team arithmetic       PE sets enumerated by brute force from the definitions (members of the
+ *       parent by index, rows and columns of the row-major grid), translate against set lookups;
  *   integer reduce        order-free closed forms, numpy, reference known answer dst[i]==i*npes
  *       (examples/ring-reduce.cu:242-248, examples/user-buffer.cu:141-152);
  *   fp32 / fp16 / bf16 reduce   numpy / torch CPU left folds in the element type, order-sensitive
@@ -90,6 +92,17 @@ void oracle_alltoall(int npes, size_t seg_bytes, const uint8_t *src, uint8_t *ds
 int oracle_reducescatter(int dtype, int op, int npes, size_t nelems, const void *src, void *dst);
 /* dst[q][k] = src[root][k] for every q including the root; src, dst are [npes][bytes] */
 void oracle_broadcast(int npes, size_t bytes, int root, const uint8_t *src, uint8_t *dst);
+
+/* ---- teams: a team is the PE set {start + i*stride, i < size} of world PEs ---- */
+/* child of `parent` = members start, start+stride, ... (size of them) counted in parent indices.
+ * Returns 0, or -1 for the argument errors the reference rejects. */
+int oracle_team_split_strided(const int parent[3], int npes_world, int start, int stride, int size,
+                              int child[3]);
+/* index of team `src`'s member src_pe inside team `dst`, or -1 */
+int oracle_team_translate_pe(const int src[3], int src_pe, const int dst[3]);
+/* the x (row) and y (column) teams of parent member `index` when the parent is laid out row-major
+ * with rows of xrange members; the last row / the right-hand columns may be shorter */
+void oracle_team_split_2d(const int parent[3], int xrange, int index, int xteam[3], int yteam[3]);
 
 /* ---- allocator model (independent structure: one ordered block list) ---- */
 typedef struct oracle_space oracle_space_t;

@@ -52,6 +52,9 @@ def lib():
         "oracle_reduce": (i32, [i32, i32, i32, sz, vp, vp]),
         "oracle_reducescatter": (i32, [i32, i32, i32, sz, vp, vp]),
         "oracle_broadcast": (None, [i32, sz, i32, vp, vp]),
+        "oracle_team_split_strided": (i32, [vp, i32, i32, i32, i32, vp]),
+        "oracle_team_translate_pe": (i32, [vp, i32, vp]),
+        "oracle_team_split_2d": (None, [vp, i32, i32, vp, vp]),
         "oracle_fcollect": (None, [i32, sz, vp, vp]),
         "oracle_alltoall": (None, [i32, sz, vp, vp]),
         "oracle_space_create": (vp, [u64, u64]),
@@ -131,6 +134,35 @@ def broadcast(src_bytes, root):
     out = np.empty_like(src)
     lib().oracle_broadcast(src.shape[0], src.shape[1], root, _p(src), _p(out))
     return out
+
+
+def _triple(t):
+    return np.ascontiguousarray(t, dtype=np.int32)
+
+
+def team_split_strided(parent, npes_world, start, stride, size):
+    """(start, stride, size) of the child in world PEs, or None when the arguments are rejected."""
+    child = np.empty(3, np.int32)
+    par = _triple(parent)
+    rc = lib().oracle_team_split_strided(_p(par), npes_world, start, stride, size, _p(child))
+    return None if rc else tuple(int(v) for v in child)
+
+
+def team_translate_pe(src, src_pe, dst):
+    a, b = _triple(src), _triple(dst)
+    return lib().oracle_team_translate_pe(_p(a), src_pe, _p(b))
+
+
+def team_split_2d(parent, xrange_, index):
+    x = np.empty(3, np.int32); y = np.empty(3, np.int32)
+    par = _triple(parent)
+    lib().oracle_team_split_2d(_p(par), xrange_, index, _p(x), _p(y))
+    return tuple(int(v) for v in x), tuple(int(v) for v in y)
+
+
+def team_members(team):
+    start, stride, size = team
+    return [start + i * stride for i in range(size)]
 
 
 def fcollect(src_bytes):

@@ -32,9 +32,13 @@ def test_constants_have_the_reference_abi_values():
     #include <stdio.h>
     #include "nvshmem.h"
     int main(void) {
-        printf("%d %d %d %d %d %d %d %d %d %d %zu\n", NVSHMEM_CMP_EQ, NVSHMEM_CMP_NE, NVSHMEM_CMP_GT,
+        printf("%d %d %d %d %d %d %d %d %d %d %zu %d %d %d %d %d %d %d %zu\n", NVSHMEM_CMP_EQ,
+               NVSHMEM_CMP_NE, NVSHMEM_CMP_GT,
                NVSHMEM_CMP_LE, NVSHMEM_CMP_LT, NVSHMEM_CMP_GE, NVSHMEM_SIGNAL_SET, NVSHMEM_SIGNAL_ADD,
-               NVSHMEM_TEAM_WORLD, NVSHMEMX_ERROR_INTERNAL, sizeof(nvshmemi_device_state_t));
+               NVSHMEM_TEAM_WORLD, NVSHMEMX_ERROR_INTERNAL, sizeof(nvshmemi_device_state_t),
+               NVSHMEM_TEAM_INVALID, NVSHMEM_TEAM_SHARED, NVSHMEMX_TEAM_NODE,
+               NVSHMEMX_TEAM_SAME_MYPE_NODE, NVSHMEMI_TEAM_SAME_GPU, NVSHMEMI_TEAM_GPU_LEADERS,
+               NVSHMEM_TEAMS_MIN, sizeof(nvshmem_team_config_t));
         return 0;
     }'''
     exe = "/tmp/nvshmem_amd_abi_probe"
@@ -42,7 +46,10 @@ def test_constants_have_the_reference_abi_values():
                     os.path.join(ROOT, "include"), "-o", exe], input=src.encode(), check=True)
     out = subprocess.run([exe], stdout=subprocess.PIPE, check=True).stdout.decode().split()
     assert out[:10] == ["0", "1", "2", "3", "4", "5", "9", "10", "0", "7"]
-    assert int(out[10]) == 64
+    assert int(out[10]) == 80
+    # team ids: src/include/device_host/nvshmem_common.cuh:406-419; the config struct is 64 bytes
+    # (src/include/device_host/nvshmem_types.h:301)
+    assert out[11:] == ["-1", "1", "2", "3", "4", "5", "6", "64"]
 
 
 def test_api_before_init_reports_instead_of_crashing():

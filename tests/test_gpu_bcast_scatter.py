@@ -89,7 +89,7 @@ def test_broadcast_argument_errors(rt8):
     with pytest.raises(N.host.NvshmemError, match="overlap"):
         rt8.broadcastmem(a + 8, a, 64, 0)
     with pytest.raises(N.host.NvshmemError, match="team"):
-        rt8.broadcast("float", a, b, 16, 0, team=2)
+        rt8.broadcast("float", a, b, 16, 0, team=20)
     with pytest.raises(N.host.NvshmemError):
         rt8.broadcastmem(a, b, 1 << 40, 0)
     rt8.broadcastmem(a, b, 0, 0)      # nothing to do

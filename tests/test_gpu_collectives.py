@@ -146,7 +146,7 @@ def test_reduce_in_place_unaligned_stream_and_sizes(rt8):
 def test_collective_argument_errors_are_reported(rt8):
     a = rt8.malloc(4096); b = rt8.malloc(4096)
     with pytest.raises(N.host.NvshmemError, match="team"):
-        rt8.reduce("float", "sum", a, b, 16, team=3)
+        rt8.reduce("float", "sum", a, b, 16, team=20)
     with pytest.raises(N.host.NvshmemError, match="not a symmetric address"):
         rt8.reduce("float", "sum", 0x4000, b, 16)
     with pytest.raises(N.host.NvshmemError, match="overlap"):

@@ -377,3 +377,64 @@ def test_reducescatter_is_the_sliced_reduce_and_keeps_its_operand_order():
     assert rs_max([nan, 1, 2]) == 2.0         # (nan>1)?nan:1 = 1 ; (1>2)?1:2 = 2
     assert rs_max([1, nan, 0]) == 0.0         # (1>nan)?1:nan = nan ; (nan>0)?nan:0 = 0
     assert np.isnan(O.reduce("f32", "max", np.array([[1], [nan], [0]], np.float32))[0])
+
+
+# ---------------------------------------------------------------------------------------------
+# team arithmetic: PE sets enumerated from the definitions
+# ---------------------------------------------------------------------------------------------
+def test_team_split_strided_enumerates_the_parent_members_by_index():
+    npes = 24
+    parents = [(0, 1, 24), (0, 1, 8), (3, 2, 10), (1, 5, 4), (23, 1, 1)]
+    for parent in parents:
+        members = O.team_members(parent)             # parent index -> world PE
+        for start in range(-1, parent[2] + 1):
+            for stride in range(0, 5):
+                for size in range(0, parent[2] + 2):
+                    got = O.team_split_strided(parent, npes, start, stride, size)
+                    ok = 0 <= start < parent[2] and 1 <= size <= parent[2] and stride >= 1
+                    want = None
+                    if ok:
+                        idx = [start + i * stride for i in range(size)]
+                        # the reference checks the world PEs, not the parent's bounds
+                        world = [parent[0] + j * parent[1] for j in idx]
+                        if world[0] < npes and world[-1] < npes:
+                            want = world
+                    if want is None:
+                        assert got is None, (parent, start, stride, size)
+                    else:
+                        assert got is not None and O.team_members(got) == want, (parent, start, stride, size)
+                        if idx[-1] < parent[2]:
+                            assert want == [members[j] for j in idx]
+    # the gemm_allreduce example duplicates the world team: examples/gemm_allreduce/...:434
+    assert O.team_split_strided((0, 1, 8), 8, 0, 1, 8) == (0, 1, 8)
+
+
+def test_team_translate_pe_against_set_lookup():
+    teams = [(0, 1, 16), (0, 2, 8), (1, 2, 8), (4, 3, 4), (5, 1, 1), (0, 4, 4)]
+    for src in teams:
+        sm = O.team_members(src)
+        for dst in teams:
+            dm = O.team_members(dst)
+            for i in range(src[2]):
+                want = dm.index(sm[i]) if sm[i] in dm else -1
+                assert O.team_translate_pe(src, i, dst) == want, (src, i, dst)
+            # the reference wraps an index equal to the size to member 0 and rejects larger ones
+            assert O.team_translate_pe(src, src[2], dst) == (dm.index(sm[0]) if sm[0] in dm else -1)
+            assert O.team_translate_pe(src, src[2] + 1, dst) == -1
+            assert O.team_translate_pe(src, -1, dst) == -1
+
+
+def test_team_split_2d_rows_and_columns_partition_the_parent():
+    for parent in [(0, 1, 16), (0, 1, 10), (2, 3, 7), (0, 1, 1), (1, 2, 12)]:
+        members = O.team_members(parent)
+        n = parent[2]
+        for xrange_ in (1, 2, 3, 4, 5, n, n + 3):
+            xr = min(xrange_, n)
+            rows, cols = {}, {}
+            for i in range(n):                       # row-major grid of parent indices
+                rows.setdefault(i // xr, []).append(members[i])
+                cols.setdefault(i % xr, []).append(members[i])
+            for i in range(n):
+                x, y = O.team_split_2d(parent, xrange_, i)
+                assert O.team_members(x) == rows[i // xr], (parent, xrange_, i)
+                assert O.team_members(y) == cols[i % xr], (parent, xrange_, i)
