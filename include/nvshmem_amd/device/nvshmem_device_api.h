@@ -222,6 +222,63 @@ NVSHMEMI_DEV uint64_t nvshmem_signal_wait_until(uint64_t *sig_addr, int cmp, uin
 NVSHMEMI_REPT_FOR_WAIT_TYPES(NVSHMEMI_STAMP_WAIT)
 #undef NVSHMEMI_STAMP_WAIT
 
+/* ---- atomic memory operations (reference nvshmem_defines.h:742-1236) ---- */
+#define NVSHMEMI_STAMP_AMO_FETCH_SET_SWAP(NAME, TYPE)                                             \
+    NVSHMEMI_DEV TYPE nvshmem_##NAME##_atomic_fetch(const TYPE *target, int pe) {                 \
+        return nvshmemi_atomic_fetch<TYPE>(target, pe);                                           \
+    }                                                                                             \
+    NVSHMEMI_DEV void nvshmem_##NAME##_atomic_set(TYPE *target, TYPE value, int pe) {             \
+        nvshmemi_atomic_set<TYPE>(target, value, pe);                                             \
+    }                                                                                             \
+    NVSHMEMI_DEV TYPE nvshmem_##NAME##_atomic_swap(TYPE *target, TYPE value, int pe) {            \
+        return nvshmemi_atomic_swap<TYPE>(target, value, pe);                                     \
+    }
+NVSHMEMI_REPT_FOR_STANDARD_AMO_TYPES(NVSHMEMI_STAMP_AMO_FETCH_SET_SWAP)
+NVSHMEMI_REPT_FOR_EXTENDED_AMO_TYPES(NVSHMEMI_STAMP_AMO_FETCH_SET_SWAP)
+#undef NVSHMEMI_STAMP_AMO_FETCH_SET_SWAP
+
+#define NVSHMEMI_STAMP_AMO_ARITH(NAME, TYPE)                                                      \
+    NVSHMEMI_DEV TYPE nvshmem_##NAME##_atomic_compare_swap(TYPE *target, TYPE cond, TYPE value,   \
+                                                           int pe) {                              \
+        return nvshmemi_atomic_compare_swap<TYPE>(target, cond, value, pe);                       \
+    }                                                                                             \
+    NVSHMEMI_DEV TYPE nvshmem_##NAME##_atomic_fetch_add(TYPE *target, TYPE value, int pe) {       \
+        return nvshmemi_atomic_fetch_add<TYPE>(target, value, pe);                                \
+    }                                                                                             \
+    NVSHMEMI_DEV void nvshmem_##NAME##_atomic_add(TYPE *target, TYPE value, int pe) {             \
+        (void)nvshmemi_atomic_fetch_add<TYPE>(target, value, pe);                                 \
+    }                                                                                             \
+    NVSHMEMI_DEV TYPE nvshmem_##NAME##_atomic_fetch_inc(TYPE *target, int pe) {                   \
+        return nvshmemi_atomic_fetch_add<TYPE>(target, (TYPE)1, pe);                              \
+    }                                                                                             \
+    NVSHMEMI_DEV void nvshmem_##NAME##_atomic_inc(TYPE *target, int pe) {                         \
+        (void)nvshmemi_atomic_fetch_add<TYPE>(target, (TYPE)1, pe);                               \
+    }
+NVSHMEMI_REPT_FOR_STANDARD_AMO_TYPES(NVSHMEMI_STAMP_AMO_ARITH)
+#undef NVSHMEMI_STAMP_AMO_ARITH
+
+#define NVSHMEMI_STAMP_AMO_BITWISE(NAME, TYPE)                                                    \
+    NVSHMEMI_DEV TYPE nvshmem_##NAME##_atomic_fetch_and(TYPE *target, TYPE value, int pe) {       \
+        return nvshmemi_atomic_fetch_and<TYPE>(target, value, pe);                                \
+    }                                                                                             \
+    NVSHMEMI_DEV TYPE nvshmem_##NAME##_atomic_fetch_or(TYPE *target, TYPE value, int pe) {        \
+        return nvshmemi_atomic_fetch_or<TYPE>(target, value, pe);                                 \
+    }                                                                                             \
+    NVSHMEMI_DEV TYPE nvshmem_##NAME##_atomic_fetch_xor(TYPE *target, TYPE value, int pe) {       \
+        return nvshmemi_atomic_fetch_xor<TYPE>(target, value, pe);                                \
+    }                                                                                             \
+    NVSHMEMI_DEV void nvshmem_##NAME##_atomic_and(TYPE *target, TYPE value, int pe) {             \
+        (void)nvshmemi_atomic_fetch_and<TYPE>(target, value, pe);                                 \
+    }                                                                                             \
+    NVSHMEMI_DEV void nvshmem_##NAME##_atomic_or(TYPE *target, TYPE value, int pe) {              \
+        (void)nvshmemi_atomic_fetch_or<TYPE>(target, value, pe);                                  \
+    }                                                                                             \
+    NVSHMEMI_DEV void nvshmem_##NAME##_atomic_xor(TYPE *target, TYPE value, int pe) {             \
+        (void)nvshmemi_atomic_fetch_xor<TYPE>(target, value, pe);                                 \
+    }
+NVSHMEMI_REPT_FOR_BITWISE_AMO_TYPES(NVSHMEMI_STAMP_AMO_BITWISE)
+#undef NVSHMEMI_STAMP_AMO_BITWISE
+
 /* ---- collectives inside a kernel: one thread group per PE ---- */
 #define NVSHMEMI_STAMP_COLL_SCOPE(NAME, TYPE, PFX, SFX, SC)                                       \
     NVSHMEMI_DEV int PFX##_##NAME##_alltoall##SFX(nvshmem_team_t team, TYPE *dest,                \

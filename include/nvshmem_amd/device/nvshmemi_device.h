@@ -435,6 +435,81 @@ NVSHMEMI_DEVICE_INLINE int nvshmemi_test(T *ivar, int cmp, T value) {
 }
 
 /* ------------------------------------------------------------------------------------------------
+ * Atomic memory operations (reference src/include/device/nvshmem_defines.h:742-1236, whose
+ * load/store branch applies atomic*_system to the translated address).  Here: relaxed agent-scope
+ * atomics on the target PE's copy; every operation works at the full width of its type (the
+ * reference narrows a few through its sub-type casts, e.g. ulong fetch_add through unsigned int,
+ * and leaves longlong / int64 / ptrdiff add and inc out).  float and double go through an integer
+ * exchange / load / store of the same width.
+ * ---------------------------------------------------------------------------------------------- */
+template <typename T> struct nvshmemi_amd_amo_word { typedef T type; };
+template <> struct nvshmemi_amd_amo_word<float> { typedef uint32_t type; };
+template <> struct nvshmemi_amd_amo_word<double> { typedef uint64_t type; };
+
+template <typename T>
+NVSHMEMI_DEVICE_INLINE typename nvshmemi_amd_amo_word<T>::type nvshmemi_amd_amo_bits(T v) {
+    typename nvshmemi_amd_amo_word<T>::type w;
+    __builtin_memcpy(&w, &v, sizeof w);
+    return w;
+}
+template <typename T>
+NVSHMEMI_DEVICE_INLINE T nvshmemi_amd_amo_value(typename nvshmemi_amd_amo_word<T>::type w) {
+    T v;
+    __builtin_memcpy(&v, &w, sizeof v);
+    return v;
+}
+template <typename T>
+NVSHMEMI_DEVICE_INLINE typename nvshmemi_amd_amo_word<T>::type *nvshmemi_amd_amo_target(const T *target, int pe) {
+    return reinterpret_cast<typename nvshmemi_amd_amo_word<T>::type *>(
+        nvshmemi_amd_remote(const_cast<T *>(target), pe));
+}
+
+template <typename T>
+NVSHMEMI_DEVICE_INLINE T nvshmemi_atomic_fetch(const T *target, int pe) {
+    return nvshmemi_amd_amo_value<T>(
+        __hip_atomic_load(nvshmemi_amd_amo_target(target, pe), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT));
+}
+template <typename T>
+NVSHMEMI_DEVICE_INLINE void nvshmemi_atomic_set(T *target, T value, int pe) {
+    __hip_atomic_store(nvshmemi_amd_amo_target(target, pe), nvshmemi_amd_amo_bits(value), __ATOMIC_RELAXED,
+                       __HIP_MEMORY_SCOPE_AGENT);
+}
+template <typename T>
+NVSHMEMI_DEVICE_INLINE T nvshmemi_atomic_swap(T *target, T value, int pe) {
+    return nvshmemi_amd_amo_value<T>(__hip_atomic_exchange(nvshmemi_amd_amo_target(target, pe),
+                                                          nvshmemi_amd_amo_bits(value), __ATOMIC_RELAXED,
+                                                          __HIP_MEMORY_SCOPE_AGENT));
+}
+/* if (*target == cond) *target = value; returns the value found */
+template <typename T>
+NVSHMEMI_DEVICE_INLINE T nvshmemi_atomic_compare_swap(T *target, T cond, T value, int pe) {
+    T expected = cond;
+    __hip_atomic_compare_exchange_strong(nvshmemi_amd_amo_target(target, pe), &expected, value,
+                                         __ATOMIC_RELAXED, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    return expected;
+}
+template <typename T>
+NVSHMEMI_DEVICE_INLINE T nvshmemi_atomic_fetch_add(T *target, T value, int pe) {
+    return __hip_atomic_fetch_add(nvshmemi_amd_amo_target(target, pe), value, __ATOMIC_RELAXED,
+                                  __HIP_MEMORY_SCOPE_AGENT);
+}
+template <typename T>
+NVSHMEMI_DEVICE_INLINE T nvshmemi_atomic_fetch_and(T *target, T value, int pe) {
+    return __hip_atomic_fetch_and(nvshmemi_amd_amo_target(target, pe), value, __ATOMIC_RELAXED,
+                                  __HIP_MEMORY_SCOPE_AGENT);
+}
+template <typename T>
+NVSHMEMI_DEVICE_INLINE T nvshmemi_atomic_fetch_or(T *target, T value, int pe) {
+    return __hip_atomic_fetch_or(nvshmemi_amd_amo_target(target, pe), value, __ATOMIC_RELAXED,
+                                 __HIP_MEMORY_SCOPE_AGENT);
+}
+template <typename T>
+NVSHMEMI_DEVICE_INLINE T nvshmemi_atomic_fetch_xor(T *target, T value, int pe) {
+    return __hip_atomic_fetch_xor(nvshmemi_amd_amo_target(target, pe), value, __ATOMIC_RELAXED,
+                                  __HIP_MEMORY_SCOPE_AGENT);
+}
+
+/* ------------------------------------------------------------------------------------------------
  * Teams (reference non_abi/device/team/nvshmemi_team_defines.cuh:95-141).  A team is the strided
  * PE set {start + i*stride, i < size}; the table holds every team as each PE sees it.
  * ---------------------------------------------------------------------------------------------- */

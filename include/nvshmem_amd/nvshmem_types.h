@@ -72,6 +72,47 @@ typedef struct { uint16_t bits; } nvshmem_half_t;
     X(size, size_t)                     \
     X(ptrdiff, ptrdiff_t)
 
+/* Atomic memory operations (reference src/include/host/nvshmem_api.h:91-112): fetch / set / swap /
+ * compare_swap / inc / add exist for the bitwise and the standard lists, fetch / set / swap also
+ * for the extended list, and / or / xor for the bitwise list only. */
+#define NVSHMEMI_REPT_FOR_BITWISE_AMO_TYPES(X) \
+    X(uint, unsigned int)                      \
+    X(ulong, unsigned long)                    \
+    X(ulonglong, unsigned long long)           \
+    X(int32, int32_t)                          \
+    X(int64, int64_t)                          \
+    X(uint32, uint32_t)                        \
+    X(uint64, uint64_t)
+#define NVSHMEMI_REPT_FOR_STANDARD_AMO_TYPES(X) \
+    NVSHMEMI_REPT_FOR_BITWISE_AMO_TYPES(X)      \
+    X(int, int)                                 \
+    X(long, long)                               \
+    X(longlong, long long)                      \
+    X(size, size_t)                             \
+    X(ptrdiff, ptrdiff_t)
+#define NVSHMEMI_REPT_FOR_EXTENDED_AMO_TYPES(X) \
+    X(float, float)                             \
+    X(double, double)
+
+/* Operation ids of the reference's nvshmemi_amo_t
+ * (src/include/device_host_transport/nvshmem_common_transport.h:41-62). */
+typedef enum {
+    NVSHMEMI_AMO_INC = 2,
+    NVSHMEMI_AMO_SET = 3,
+    NVSHMEMI_AMO_ADD = 4,
+    NVSHMEMI_AMO_AND = 5,
+    NVSHMEMI_AMO_OR = 6,
+    NVSHMEMI_AMO_XOR = 7,
+    NVSHMEMI_AMO_FETCH = 12,
+    NVSHMEMI_AMO_FETCH_INC = 13,
+    NVSHMEMI_AMO_FETCH_ADD = 14,
+    NVSHMEMI_AMO_FETCH_AND = 15,
+    NVSHMEMI_AMO_FETCH_OR = 16,
+    NVSHMEMI_AMO_FETCH_XOR = 17,
+    NVSHMEMI_AMO_SWAP = 18,
+    NVSHMEMI_AMO_COMPARE_SWAP = 19
+} nvshmemi_amo_t;
+
 /* and / or / xor. */
 #define NVSHMEMI_REPT_FOR_BITWISE_REDUCE_TYPES(X, OP) \
     X(uchar, unsigned char, u8, OP)                   \

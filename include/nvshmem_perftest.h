@@ -95,6 +95,22 @@ int nvshmem_perftest_device_reducescatter(int dtype, int op, void *dest, const v
                                           size_t nreduce, int scope, int threads, void *stream);
 int nvshmem_perftest_device_broadcast(void *dest, const void *src, size_t bytes, int root,
                                       int scope, int threads, void *stream);
+/* Atomic memory operations.  amo_matrix: every PE applies every stamped (type, operation) pair once
+ * to word k of `slots` on its right neighbour - case order: fetch, set, swap for the standard then
+ * the extended types; compare_swap, compare_swap, fetch_add, add, fetch_inc, inc for the standard
+ * types; fetch_and, and, fetch_or, or, fetch_xor, xor for the bitwise types (type lists of
+ * include/nvshmem_amd/nvshmem_types.h) - with operands val[k] / cond[k] from its own copies, and
+ * stores the returned value into its out[k]; *ncases receives the number of cases, which
+ * nvshmem_perftest_amo_matrix_cases() also returns.  All arrays are symmetric, cases + 1 words. */
+int nvshmem_perftest_amo_matrix_cases(void);
+int nvshmem_perftest_amo_matrix(uint64_t *slots, const uint64_t *val, const uint64_t *cond,
+                                uint64_t *out, int *ncases, void *stream);
+/* All blocks x threads x npes threads contend for PE `home`'s copies of words[0..8) = {ticket
+ * counter, lock, xor word, or word, and word, 32-bit sum, swap word, lock winners} and seen[ticket];
+ * chain[id] on PE `home` (symmetric, one word per thread) receives what the thread's swap
+ * returned. */
+int nvshmem_perftest_amo_contend(uint64_t *words, unsigned int *seen, unsigned long long *chain,
+                                 int home, int blocks, int threads, void *stream);
 /* In-kernel collectives on a team handle (members only; the other PEs return at once).  what:
  * 0 float sum reduce (n elements), 1 float sum reducescatter (n per member), 2 fcollectmem, 3
  * alltoallmem, 4 broadcastmem from member `root` (n bytes). */

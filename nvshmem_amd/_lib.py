@@ -129,6 +129,9 @@ def load_perftest():
         "nvshmem_perftest_ring_reduce": [vp, vp, sz, vp, sz, i32, i32, vp],
         "nvshmem_perftest_device_reduce": [i32, i32, vp, vp, sz, i32, i32, vp],
         "nvshmem_perftest_device_fcollect": [vp, vp, sz, i32, i32, vp],
+        "nvshmem_perftest_amo_matrix_cases": [],
+        "nvshmem_perftest_amo_matrix": [vp, vp, vp, vp, vp, vp],
+        "nvshmem_perftest_amo_contend": [vp, vp, vp, i32, i32, i32, vp],
         "nvshmem_perftest_device_team_coll": [i32, i32, vp, vp, sz, i32, i32, i32, vp],
         "nvshmem_perftest_team_query": [vp, i32, i32, vp],
         "nvshmem_perftest_device_team_barrier": [vp, vp, i32, i32, i32, i32, vp],

@@ -346,6 +346,34 @@ void oracle_broadcast(int npes, size_t bytes, int root, const uint8_t *src, uint
 }
 
 /* ------------------------------------------------------------------------------------------- */
+/* atomic memory operations: OpenSHMEM semantics of the calls stamped in the reference's
+ * src/include/device/nvshmem_defines.h:742-1236 (fetch_add :742-757, fetch_inc :821-836,
+ * compare_swap :907-922, fetch_and/or/xor :955-1115, swap :1135-1150, fetch :1184-1196,
+ * set :1213-1221); op ids of nvshmemi_amo_t, nvshmem_common_transport.h:41-62.                 */
+/* ------------------------------------------------------------------------------------------- */
+uint64_t oracle_amo(int op, int bits, uint64_t current, uint64_t value, uint64_t cond,
+                    uint64_t *fetched) {
+    const uint64_t mask = bits >= 64 ? ~0ull : ((1ull << bits) - 1ull);
+    current &= mask;
+    value &= mask;
+    cond &= mask;
+    if (fetched) *fetched = current;
+    uint64_t next = current;
+    switch (op) {
+        case 2: case 13: next = current + 1; break;            /* inc, fetch_inc */
+        case 3: case 18: next = value; break;                  /* set, swap */
+        case 4: case 14: next = current + value; break;        /* add, fetch_add */
+        case 5: case 15: next = current & value; break;        /* and, fetch_and */
+        case 6: case 16: next = current | value; break;        /* or, fetch_or */
+        case 7: case 17: next = current ^ value; break;        /* xor, fetch_xor */
+        case 12: break;                                        /* fetch */
+        case 19: next = current == cond ? value : current; break; /* compare_swap */
+        default: break;
+    }
+    return next & mask;
+}
+
+/* ------------------------------------------------------------------------------------------- */
 /* teams: reference nvshmemi_team_split_strided, src/host/team/team_internal.cpp:2182-2290
  * (argument checks :2197-2222, global triple :2214-2216), nvshmemi_team_split_2d :2292-2349,
  * nvshmemi_team_translate_pe :579-589 (member index wraps modulo the size; an index above the size

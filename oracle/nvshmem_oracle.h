@@ -14,6 +14,7 @@
  *   broadcast / reducescatter   brute force, the reference's known answer for broadcast
  *       (examples/ring-bcast.cu:68-72), slices of the pinned reduce for order-free operators, numpy
  *       folds and hand-evaluated NaN cases for the operand order;
+ *   atomic operations     exhaustive small-width tables and random words against Python integers;
  *   team arithmetic       PE sets enumerated by brute force from the definitions (members of the
  *       parent by index, rows and columns of the row-major grid), translate against set lookups;
  *   integer reduce        order-free closed forms, numpy, reference known answer dst[i]==i*npes
@@ -92,6 +93,13 @@ void oracle_alltoall(int npes, size_t seg_bytes, const uint8_t *src, uint8_t *ds
 int oracle_reducescatter(int dtype, int op, int npes, size_t nelems, const void *src, void *dst);
 /* dst[q][k] = src[root][k] for every q including the root; src, dst are [npes][bytes] */
 void oracle_broadcast(int npes, size_t bytes, int root, const uint8_t *src, uint8_t *dst);
+
+/* ---- atomic memory operations: op numbering of include/nvshmem_amd/nvshmem_types.h ----
+ * One operation on a word of `bits` (32 or 64) bits holding `current`: returns the new contents,
+ * *fetched receives what a fetching form returns (the old contents).  Arithmetic wraps modulo
+ * 2^bits; compare_swap stores `value` only when current == cond.  Unknown op: word unchanged. */
+uint64_t oracle_amo(int op, int bits, uint64_t current, uint64_t value, uint64_t cond,
+                    uint64_t *fetched);
 
 /* ---- teams: a team is the PE set {start + i*stride, i < size} of world PEs ---- */
 /* child of `parent` = members start, start+stride, ... (size of them) counted in parent indices.

@@ -52,6 +52,7 @@ def lib():
         "oracle_reduce": (i32, [i32, i32, i32, sz, vp, vp]),
         "oracle_reducescatter": (i32, [i32, i32, i32, sz, vp, vp]),
         "oracle_broadcast": (None, [i32, sz, i32, vp, vp]),
+        "oracle_amo": (C.c_uint64, [i32, i32, C.c_uint64, C.c_uint64, C.c_uint64, vp]),
         "oracle_team_split_strided": (i32, [vp, i32, i32, i32, i32, vp]),
         "oracle_team_translate_pe": (i32, [vp, i32, vp]),
         "oracle_team_split_2d": (None, [vp, i32, i32, vp, vp]),
@@ -134,6 +135,18 @@ def broadcast(src_bytes, root):
     out = np.empty_like(src)
     lib().oracle_broadcast(src.shape[0], src.shape[1], root, _p(src), _p(out))
     return out
+
+
+AMO = {"inc": 2, "set": 3, "add": 4, "and": 5, "or": 6, "xor": 7, "fetch": 12, "fetch_inc": 13,
+       "fetch_add": 14, "fetch_and": 15, "fetch_or": 16, "fetch_xor": 17, "swap": 18, "compare_swap": 19}
+
+
+def amo(op, bits, current, value=0, cond=0):
+    """-> (new contents, fetched value) of one atomic operation on a `bits`-bit word."""
+    fetched = C.c_uint64(0)
+    new = lib().oracle_amo(AMO[op], bits, current & (2**64 - 1), value & (2**64 - 1), cond & (2**64 - 1),
+                           C.addressof(fetched))
+    return int(new), int(fetched.value)
 
 
 def _triple(t):

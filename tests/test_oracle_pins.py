@@ -438,3 +438,33 @@ def test_team_split_2d_rows_and_columns_partition_the_parent():
                 x, y = O.team_split_2d(parent, xrange_, i)
                 assert O.team_members(x) == rows[i // xr], (parent, xrange_, i)
                 assert O.team_members(y) == cols[i % xr], (parent, xrange_, i)
+
+
+# ---------------------------------------------------------------------------------------------
+# atomic memory operations against Python integers
+# ---------------------------------------------------------------------------------------------
+def _amo_python(op, bits, cur, val, cond):
+    m = (1 << bits) - 1
+    cur, val, cond = cur & m, val & m, cond & m
+    new = {"inc": cur + 1, "fetch_inc": cur + 1, "set": val, "swap": val, "add": cur + val,
+           "fetch_add": cur + val, "and": cur & val, "fetch_and": cur & val, "or": cur | val,
+           "fetch_or": cur | val, "xor": cur ^ val, "fetch_xor": cur ^ val, "fetch": cur,
+           "compare_swap": val if cur == cond else cur}[op]
+    return new & m, cur
+
+
+def test_amo_semantics_against_python_integers():
+    rng = np.random.default_rng(21)
+    edge = [0, 1, 2, 0x7FFFFFFF, 0x80000000, 0xFFFFFFFF, 0x100000000, 2**63 - 1, 2**63, 2**64 - 1]
+    for bits in (32, 64):
+        words = edge + [int(x) for x in rng.integers(0, 2**64, 40, dtype=np.uint64)]
+        for op in O.AMO:
+            for cur in words:
+                for val in words[:12] + words[-6:]:
+                    for cond in (cur, cur ^ 1, val):
+                        assert O.amo(op, bits, cur, val, cond) == _amo_python(op, bits, cur, val, cond), \
+                            (op, bits, cur, val, cond)
+    # wrap-around and the compare_swap miss, by hand
+    assert O.amo("fetch_add", 32, 0xFFFFFFFF, 2) == (1, 0xFFFFFFFF)
+    assert O.amo("inc", 64, 2**64 - 1) == (0, 2**64 - 1)
+    assert O.amo("compare_swap", 64, 5, 9, 4) == (5, 5) and O.amo("compare_swap", 64, 5, 9, 5) == (9, 5)
