@@ -659,6 +659,209 @@ NVSHMEMI_DEVICE_INLINE T nvshmemi_amd_fold_step(int i, T acc, T x) {
 }
 
 /* ------------------------------------------------------------------------------------------------
+ * Low-latency packets for small collectives (the role of the reference's LL protocol,
+ * non_abi/device/common/nvshmemi_common_device.cuh:981-1066 packLL / recvLL, used by
+ * coll/fcollect.cuh:100-314 and coll/broadcast.cuh:40-273).
+ *
+ * Eight payload bytes travel as one 16-byte packet {lo32, flag, hi32, flag}: each 8-byte half
+ * carries its own copy of the flag, so a receiver that sees the expected flag in a half also sees
+ * that half's data.  No fence and no barrier is needed: packets are written and polled with
+ * agent-scope (write-through / L2-bypassing) accesses.  The flag is the team's call counter (never
+ * 0, buffers start zeroed), and consecutive calls rotate through three buffers.  Call f overwrites
+ * the buffer of call f-3, so every member must have finished reading f-3 by then.  A PE that
+ * completed an fcollect or reduce f-1 has received packets of f-1 from every member, each of which
+ * had finished reading f-2 before it sent them.  A broadcast gives its root no such knowledge, so a
+ * root waits until every receiver has published `done >= f-2`; a receiver that then completes the
+ * broadcast f-1 inherits "everybody finished f-3".
+ *
+ * An agent-scope access costs about a memory round trip per instruction, whether one lane is active
+ * or 64, so the packets of a call are spread over the lanes - one per lane - and the path is only
+ * taken while that is possible; longer messages are faster through the copy engine and a barrier.
+ * ---------------------------------------------------------------------------------------------- */
+NVSHMEMI_DEVICE_INLINE char *nvshmemi_amd_ll_buffer(nvshmem_team_t team, int pe, uint32_t flag) {
+    const size_t buf = 2 * (size_t)NVSHMEMI_AMD_LL_PAYLOAD_BYTES;
+    return nvshmemi_device_state_d.ll_buffers +
+           (((size_t)team * (size_t)nvshmemi_device_state_d.npes + (size_t)pe) * NVSHMEMI_AMD_LL_BUFFERS +
+            flag % NVSHMEMI_AMD_LL_BUFFERS) * buf;
+}
+NVSHMEMI_DEVICE_INLINE uint64_t *nvshmemi_amd_ll_word(nvshmem_team_t team, int pe, int word) {
+    return nvshmemi_device_state_d.team_sync +
+           ((size_t)team * NVSHMEMI_AMD_MAX_PES + (size_t)pe) * NVSHMEMI_AMD_TEAM_SYNC_WORDS + word;
+}
+NVSHMEMI_DEVICE_INLINE unsigned nvshmemi_amd_ll_packets(size_t nbytes) { return (unsigned)((nbytes + 7) >> 3); }
+
+/* Packets one call may receive per PE: one per lane of the thread group; a single thread takes a
+ * few, one after the other, which still beats its barrier. */
+template <int SCOPE>
+NVSHMEMI_DEVICE_INLINE unsigned nvshmemi_amd_ll_lanes() {
+    const unsigned nthr = (unsigned)nvshmemi_threadgroup_size<SCOPE>();
+    return nthr < 8 ? 8 : nthr;
+}
+NVSHMEMI_DEVICE_INLINE bool nvshmemi_amd_ll_available() { return nvshmemi_device_state_d.ll_buffers != nullptr; }
+
+/* Next flag of the calling PE for `team`; all threads of the group return the same value. */
+template <int SCOPE>
+NVSHMEMI_DEVICE_INLINE uint32_t nvshmemi_amd_ll_next_flag(nvshmem_team_t team) {
+    uint64_t *count = nvshmemi_amd_ll_word(team, nvshmemi_amd_my_pe(), NVSHMEMI_AMD_LL_COUNT_WORD);
+    nvshmemi_threadgroup_sync<SCOPE>();
+    uint32_t flag = (uint32_t)(*reinterpret_cast<volatile uint64_t *>(count)) + 1u;
+    if (flag == 0) flag = 1; /* 0 is what an empty buffer holds */
+    nvshmemi_threadgroup_sync<SCOPE>();
+    if (nvshmemi_thread_id_in_threadgroup<SCOPE>() == 0) *reinterpret_cast<volatile uint64_t *>(count) = flag;
+    return flag;
+}
+
+NVSHMEMI_DEVICE_INLINE uint64_t nvshmemi_amd_ll_load_payload(const char *src, size_t left) {
+    uint64_t w = 0;
+    if (left >= 8 && (((uintptr_t)src) & 7) == 0) return *reinterpret_cast<const uint64_t *>(src);
+    const size_t n = left < 8 ? left : 8;
+    for (size_t b = 0; b < n; ++b) w |= (uint64_t)(unsigned char)src[b] << (8 * b);
+    return w;
+}
+NVSHMEMI_DEVICE_INLINE void nvshmemi_amd_ll_store_payload(char *dst, uint64_t w, size_t left) {
+    if (left >= 8 && (((uintptr_t)dst) & 7) == 0) {
+        *reinterpret_cast<uint64_t *>(dst) = w;
+        return;
+    }
+    const size_t n = left < 8 ? left : 8;
+    for (size_t b = 0; b < n; ++b) dst[b] = (char)(w >> (8 * b));
+}
+/* One packet, written with a single 16-byte agent-scope store so that a wavefront's packets fill
+ * whole cache lines; only the two 8-byte halves have to arrive untorn. */
+NVSHMEMI_DEVICE_INLINE void nvshmemi_amd_ll_store_packet(char *packet, uint64_t w, uint32_t flag) {
+    nvshmemi_v4u v;
+    v.x = (uint32_t)w;
+    v.y = flag;
+    v.z = (uint32_t)(w >> 32);
+    v.w = flag;
+    asm volatile("global_store_dwordx4 %0, %1, off sc1" : : "v"(packet), "v"(v) : "memory");
+}
+/* Waits until both halves of the packet carry `flag` and returns its 8 payload bytes.  A bounded
+ * wait that gives up records the timeout like nvshmemi_wait_until and returns what it last saw. */
+NVSHMEMI_DEVICE_INLINE uint64_t nvshmemi_amd_ll_recv_packet(const char *packet, uint32_t flag) {
+    const uint64_t limit = nvshmemi_device_state_d.spin_limit;
+    uint64_t polls = 0;
+    nvshmemi_v4u v;
+    for (;;) {
+        asm volatile("global_load_dwordx4 %0, %1, off sc1\n\ts_waitcnt vmcnt(0)" : "=v"(v) : "v"(packet) : "memory");
+        if (v.y == flag && v.w == flag) break;
+        if (limit && ++polls > limit) {
+            nvshmemi_amd_record_timeout(packet, v.y, flag);
+            break;
+        }
+        __builtin_amdgcn_s_sleep(1);
+    }
+    return (uint64_t)v.x | ((uint64_t)v.z << 32);
+}
+/* Sends the npk chunks of src to the other members of the team, chunk j into slot slot0 + j of
+ * their buffers; the (member, chunk) pairs are spread over the lanes. */
+template <int SCOPE>
+NVSHMEMI_DEVICE_INLINE void nvshmemi_amd_ll_send_to_all(nvshmem_team_t team, const nvshmemi_amd_team_view_t &tv,
+                                                        const char *src, size_t nbytes, unsigned npk,
+                                                        unsigned slot0, uint32_t flag) {
+    const unsigned nthr = (unsigned)nvshmemi_threadgroup_size<SCOPE>();
+    const unsigned total = (unsigned)(tv.size - 1) * npk;
+    for (unsigned w = (unsigned)nvshmemi_thread_id_in_threadgroup<SCOPE>(); w < total; w += nthr) {
+        const unsigned off = w / npk, j = w - off * npk;
+        int idx = tv.my_pe + 1 + (int)off;
+        if (idx >= tv.size) idx -= tv.size;
+        nvshmemi_amd_ll_store_packet(
+            nvshmemi_amd_ll_buffer(team, nvshmemi_amd_team_pe(tv, idx), flag) + (size_t)(slot0 + j) * 16,
+            nvshmemi_amd_ll_load_payload(src + 8 * (size_t)j, nbytes - 8 * (size_t)j), flag);
+    }
+}
+/* Tells the other PEs that this PE has read everything of call `flag`. */
+template <int SCOPE>
+NVSHMEMI_DEVICE_INLINE void nvshmemi_amd_ll_publish_done(nvshmem_team_t team, uint32_t flag) {
+    nvshmemi_threadgroup_sync<SCOPE>();
+    if (nvshmemi_thread_id_in_threadgroup<SCOPE>() == 0)
+        __hip_atomic_store(nvshmemi_amd_ll_word(team, nvshmemi_amd_my_pe(), NVSHMEMI_AMD_LL_DONE_WORD),
+                           (uint64_t)flag, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+/* fcollect / reduce: a contribution of nbytes from each of `size` members */
+template <int SCOPE>
+NVSHMEMI_DEVICE_INLINE bool nvshmemi_amd_ll_fits(size_t nbytes, int size) {
+    const size_t npk = (nbytes + 7) >> 3;
+    return nbytes > 0 && nbytes <= NVSHMEMI_AMD_LL_MAX_BYTES && nvshmemi_amd_ll_available() &&
+           npk * 8 * (size_t)size <= NVSHMEMI_AMD_LL_PAYLOAD_BYTES &&
+           npk * (size_t)(size - 1) <= nvshmemi_amd_ll_lanes<SCOPE>();
+}
+
+/* Small allreduce in one hop: every member sends its source to every other member as packets and
+ * folds the contributions itself, in member order.  Wavefront and block scope: lane (chunk j,
+ * member p) fetches one packet (its own source for p == me), then the lanes of a chunk - adjacent,
+ * in a group of G = npes rounded up to a power of two - pass their values to each other with
+ * cross-lane reads and the first lane of the group stores the result. */
+template <typename T, int OP, int SCOPE>
+NVSHMEMI_DEVICE_INLINE void nvshmemi_amd_ll_reduce(nvshmem_team_t team, const nvshmemi_amd_team_view_t &tv,
+                                                   T *dest, const T *source, size_t nreduce, unsigned group) {
+    constexpr size_t PER = 8 / sizeof(T);
+    const int me = tv.my_pe, npes = tv.size;
+    const unsigned tid = (unsigned)nvshmemi_thread_id_in_threadgroup<SCOPE>();
+    const size_t nbytes = nreduce * sizeof(T);
+    const uint32_t flag = nvshmemi_amd_ll_next_flag<SCOPE>(team);
+    const unsigned npk = nvshmemi_amd_ll_packets(nbytes);
+    const char *src = nvshmemi_amd_local(source);
+    char *dst = nvshmemi_amd_local(dest);
+    nvshmemi_amd_ll_send_to_all<SCOPE>(team, tv, src, nbytes, npk, (unsigned)me * npk, flag);
+    /* dest may be source: everything is sent before any result is stored */
+    nvshmemi_threadgroup_sync<SCOPE>();
+    const char *mine = nvshmemi_amd_ll_buffer(team, nvshmemi_amd_my_pe(), flag);
+    if (SCOPE == NVSHMEMI_THREADGROUP_THREAD) {
+        for (unsigned j = 0; j < npk; ++j) {
+            T acc[PER];
+            for (int p = 0; p < npes; ++p) {
+                const uint64_t v = p == me ? nvshmemi_amd_ll_load_payload(src + 8 * (size_t)j, nbytes - 8 * (size_t)j)
+                                           : nvshmemi_amd_ll_recv_packet(mine + ((size_t)p * npk + j) * 16, flag);
+                T x[PER];
+                __builtin_memcpy(x, &v, 8);
+#pragma unroll
+                for (size_t k = 0; k < PER; ++k) acc[k] = p == 0 ? x[k] : nvshmemi_amd_fold_step<T, OP>(p, acc[k], x[k]);
+            }
+            uint64_t r;
+            __builtin_memcpy(&r, acc, 8);
+            nvshmemi_amd_ll_store_payload(dst + 8 * (size_t)j, r, nbytes - 8 * (size_t)j);
+        }
+    } else {
+        /* group * npk <= nthr: every (chunk, member) pair has a lane; whole wavefronts take part in
+         * the cross-lane reads, lanes without a pair carry zeros */
+        const unsigned gshift = 31u - (unsigned)__builtin_clz(group);
+        const unsigned j = tid >> gshift, p = tid & (group - 1);
+        const bool wave_active = (tid & ~63u) < group * npk;
+        if (wave_active) {
+            uint64_t v = 0;
+            if (j < npk && (int)p < npes)
+                v = (int)p == me ? nvshmemi_amd_ll_load_payload(src + 8 * (size_t)j, nbytes - 8 * (size_t)j)
+                                 : nvshmemi_amd_ll_recv_packet(mine + ((size_t)p * npk + j) * 16, flag);
+            const int base = (int)((tid & 63u) & ~(group - 1));
+            T acc[PER];
+            for (int q = 0; q < npes; ++q) {
+                const uint64_t xv = (uint64_t)__shfl((unsigned long long)v, base + q, 64);
+                T x[PER];
+                __builtin_memcpy(x, &xv, 8);
+#pragma unroll
+                for (size_t k = 0; k < PER; ++k) acc[k] = q == 0 ? x[k] : nvshmemi_amd_fold_step<T, OP>(q, acc[k], x[k]);
+            }
+            if (p == 0 && j < npk) {
+                uint64_t r;
+                __builtin_memcpy(&r, acc, 8);
+                nvshmemi_amd_ll_store_payload(dst + 8 * (size_t)j, r, nbytes - 8 * (size_t)j);
+            }
+        }
+    }
+    nvshmemi_amd_ll_publish_done<SCOPE>(team, flag);
+}
+/* the group width of nvshmemi_amd_ll_reduce, or 0 when the call does not qualify */
+template <int SCOPE>
+NVSHMEMI_DEVICE_INLINE unsigned nvshmemi_amd_ll_reduce_group(size_t nbytes, int size) {
+    if (!nvshmemi_amd_ll_fits<SCOPE>(nbytes, size)) return 0;
+    if (SCOPE == NVSHMEMI_THREADGROUP_THREAD) return 1;
+    unsigned group = 1;
+    while ((int)group < size) group <<= 1;
+    return group * (unsigned)((nbytes + 7) >> 3) <= (unsigned)nvshmemi_threadgroup_size<SCOPE>() ? group : 0;
+}
+
+/* ------------------------------------------------------------------------------------------------
  * Collectives called from inside a user kernel, one thread group per PE
  * (reference coll/reduce.cuh:1158-1196 get-based reduce, coll/fcollect.cuh:331-344,
  * coll/alltoall.cuh:122-143).  Each ends with barrier semantics.
@@ -687,6 +890,10 @@ NVSHMEMI_DEVICE_INLINE int nvshmemi_reduce_threadgroup(nvshmem_team_t team, T *d
     const int npes = tv.size;
     const size_t tid = (size_t)nvshmemi_thread_id_in_threadgroup<SCOPE>();
     const size_t nthr = (size_t)nvshmemi_threadgroup_size<SCOPE>();
+    if (const unsigned group = nvshmemi_amd_ll_reduce_group<SCOPE>(nreduce * sizeof(T), npes)) {
+        nvshmemi_amd_ll_reduce<T, OP, SCOPE>(team, tv, dest, source, nreduce, group);
+        return 0;
+    }
     /* every PE's source is complete and visible before anyone reads it */
     nvshmemi_barrier_threadgroup<SCOPE>(team);
     /* member 0's copies; member i's are i * pe_stride elements further */
@@ -732,6 +939,30 @@ NVSHMEMI_DEVICE_INLINE int nvshmemi_fcollect_threadgroup(nvshmem_team_t team, T 
     if (tv.size <= 0) return 1;
     const int me = tv.my_pe;
     const int npes = tv.size;
+    const size_t nbytes = nelems * sizeof(T);
+    if (nvshmemi_amd_ll_fits<SCOPE>(nbytes, npes)) {
+        /* small contributions: packets to every member's buffer, then unpack what arrived here;
+         * the (member, chunk) pairs are spread over the lanes both ways */
+        const unsigned tid = (unsigned)nvshmemi_thread_id_in_threadgroup<SCOPE>();
+        const unsigned nthr = (unsigned)nvshmemi_threadgroup_size<SCOPE>();
+        const uint32_t flag = nvshmemi_amd_ll_next_flag<SCOPE>(team);
+        const unsigned npk = nvshmemi_amd_ll_packets(nbytes);
+        const unsigned total = (unsigned)(npes - 1) * npk;
+        const char *src = nvshmemi_amd_local(source);
+        char *dst = nvshmemi_amd_local(dest);
+        nvshmemi_amd_ll_send_to_all<SCOPE>(team, tv, src, nbytes, npk, (unsigned)me * npk, flag);
+        for (size_t b = tid; b < nbytes; b += nthr) dst[(size_t)me * nbytes + b] = src[b];
+        const char *mine = nvshmemi_amd_ll_buffer(team, nvshmemi_amd_my_pe(), flag);
+        for (unsigned w = tid; w < total; w += nthr) {
+            const unsigned off = w / npk, j = w - off * npk;
+            int idx = me + 1 + (int)off;
+            if (idx >= npes) idx -= npes;
+            const uint64_t v = nvshmemi_amd_ll_recv_packet(mine + ((size_t)idx * npk + j) * 16, flag);
+            nvshmemi_amd_ll_store_payload(dst + (size_t)idx * nbytes + 8 * (size_t)j, v, nbytes - 8 * (size_t)j);
+        }
+        nvshmemi_amd_ll_publish_done<SCOPE>(team, flag);
+        return 0;
+    }
     nvshmemi_threadgroup_sync<SCOPE>();
     for (int ii = 0; ii < npes; ++ii) {
         const int peer = nvshmemi_amd_team_pe(tv, (me + ii) % npes);
@@ -771,6 +1002,39 @@ NVSHMEMI_DEVICE_INLINE int nvshmemi_broadcast_threadgroup(nvshmem_team_t team, T
     if (tv.size <= 0) return 1;
     const int me = tv.my_pe;
     const int npes = tv.size;
+    const size_t nbytes = nelems * sizeof(T);
+    /* a single thread also sends one after the other, so all its packets count */
+    if (nbytes > 0 && nbytes <= NVSHMEMI_AMD_LL_BCAST_MAX_BYTES && nvshmemi_amd_ll_available() &&
+        ((nbytes + 7) >> 3) * (size_t)(SCOPE == NVSHMEMI_THREADGROUP_THREAD ? npes - 1 : 1) <=
+            nvshmemi_amd_ll_lanes<SCOPE>()) {
+        const unsigned tid = (unsigned)nvshmemi_thread_id_in_threadgroup<SCOPE>();
+        const unsigned nthr = (unsigned)nvshmemi_threadgroup_size<SCOPE>();
+        const uint32_t flag = nvshmemi_amd_ll_next_flag<SCOPE>(team);
+        const unsigned npk = nvshmemi_amd_ll_packets(nbytes);
+        if (me == PE_root) {
+            const char *src = nvshmemi_amd_local(source);
+            char *dst = nvshmemi_amd_local(dest);
+            /* nothing else orders a root against its receivers: all of them must have finished
+             * reading call flag - 2 before anybody may be sent call flag */
+            for (unsigned i = tid; i < (unsigned)npes; i += nthr)
+                if ((int)i != me && flag > 2)
+                    nvshmemi_wait_until<uint64_t>(
+                        nvshmemi_amd_ll_word(team, nvshmemi_amd_team_pe(tv, (int)i), NVSHMEMI_AMD_LL_DONE_WORD),
+                        NVSHMEM_CMP_GE, (uint64_t)(flag - 2));
+            nvshmemi_threadgroup_sync<SCOPE>();
+            nvshmemi_amd_ll_send_to_all<SCOPE>(team, tv, src, nbytes, npk, 0, flag);
+            if (dst != src)
+                for (size_t b = tid; b < nbytes; b += nthr) dst[b] = src[b];
+        } else {
+            char *dst = nvshmemi_amd_local(dest);
+            const char *mine = nvshmemi_amd_ll_buffer(team, nvshmemi_amd_my_pe(), flag);
+            for (unsigned j = tid; j < npk; j += nthr)
+                nvshmemi_amd_ll_store_payload(dst + 8 * (size_t)j, nvshmemi_amd_ll_recv_packet(mine + (size_t)j * 16, flag),
+                                              nbytes - 8 * (size_t)j);
+        }
+        nvshmemi_amd_ll_publish_done<SCOPE>(team, flag);
+        return 0;
+    }
     if (me == PE_root) {
         const void *from = nvshmemi_amd_local(source);
         for (int ii = 0; ii < npes; ++ii) {

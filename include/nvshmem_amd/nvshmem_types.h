@@ -204,6 +204,19 @@ typedef struct {
  * index, then the PE's epoch; one such row per (team, PE). */
 #define NVSHMEMI_AMD_TEAM_SYNC_WORDS (NVSHMEMI_AMD_MAX_PES + 8)
 
+/* Low-latency collectives: every (team, PE) owns NVSHMEMI_AMD_LL_BUFFERS packet buffers (used in
+ * rotation, by the team's call counter) that hold 16-byte packets for NVSHMEMI_AMD_LL_PAYLOAD_BYTES bytes of
+ * payload each.  A PE's contribution travels that way when it is at most
+ * NVSHMEMI_AMD_LL_MAX_BYTES long and all contributions of the team fit one buffer.  Word
+ * NVSHMEMI_AMD_LL_COUNT_WORD of a PE's team sync row counts the team's low-latency calls,
+ * NVSHMEMI_AMD_LL_DONE_WORD publishes the last one the PE has finished reading. */
+#define NVSHMEMI_AMD_LL_BUFFERS 3
+#define NVSHMEMI_AMD_LL_PAYLOAD_BYTES 16384
+#define NVSHMEMI_AMD_LL_MAX_BYTES 2048
+#define NVSHMEMI_AMD_LL_BCAST_MAX_BYTES 16384 /* broadcast: one contribution, up to a whole buffer */
+#define NVSHMEMI_AMD_LL_COUNT_WORD (NVSHMEMI_AMD_MAX_PES + 1)
+#define NVSHMEMI_AMD_LL_DONE_WORD (NVSHMEMI_AMD_MAX_PES + 2)
+
 typedef struct nvshmemi_device_state {
     uint32_t version;     /* (1 << 16) + sizeof(struct) */
     int32_t mype;         /* PE a kernel acts as when its grid is not PE-multiplexed */
@@ -216,7 +229,9 @@ typedef struct nvshmemi_device_state {
     uint64_t spin_limit;  /* 0 = wait forever; else a bounded wait gives up after this many polls */
     uint64_t *timeout_record; /* canonical address: 4 words {flag, addr, found, expected} */
     const nvshmemi_amd_team_view_t *team_views; /* [NVSHMEMI_AMD_MAX_TEAMS][NVSHMEMI_AMD_MAX_PES] */
-    uint64_t *team_sync; /* [MAX_TEAMS][MAX_PES][NVSHMEMI_AMD_TEAM_SYNC_WORDS], teams other than WORLD */
+    uint64_t *team_sync; /* [MAX_TEAMS][MAX_PES][NVSHMEMI_AMD_TEAM_SYNC_WORDS]: barrier rows of the teams
+                            other than WORLD, low-latency counters of all teams */
+    char *ll_buffers;    /* [MAX_TEAMS][npes][NVSHMEMI_AMD_LL_BUFFERS][2 * NVSHMEMI_AMD_LL_PAYLOAD_BYTES] */
 } nvshmemi_device_state_t;
 
 #endif

@@ -111,11 +111,24 @@ int nvshmem_perftest_amo_matrix(uint64_t *slots, const uint64_t *val, const uint
  * returned. */
 int nvshmem_perftest_amo_contend(uint64_t *words, unsigned int *seen, unsigned long long *chain,
                                  int home, int blocks, int threads, void *stream);
+/* `rounds` rounds of {int32 sum reduce of n elements, broadcast of those n elements from PE
+ * r % npes, fcollect of fc_bytes (a multiple of 4, at most 4n) per PE} back to back inside one
+ * kernel, all on NVSHMEM_TEAM_WORLD into dst, with no barrier in between unless sync_between is
+ * set.  Round r sends src[i] = (me*1000003 + r*7919 + i*31) & 0x7fffffff.  After every collective
+ * each PE folds dst into its check[0]: h = h*1000003 + sum_i (uint32)dst[i] * (2i+1) (mod 2^64),
+ * over the n (reduce, broadcast) or fc_bytes*npes/4 (fcollect) words the call produced. */
+int nvshmem_perftest_coll_sequence(int32_t *src, int32_t *dst, uint64_t *check, int n, int fc_bytes,
+                                   int rounds, int sync_between, int scope, int threads, void *stream);
 /* In-kernel collectives on a team handle (members only; the other PEs return at once).  what:
  * 0 float sum reduce (n elements), 1 float sum reducescatter (n per member), 2 fcollectmem, 3
  * alltoallmem, 4 broadcastmem from member `root` (n bytes). */
 int nvshmem_perftest_device_team_coll(int what, int team, void *dest, const void *src, size_t n,
                                       int root, int scope, int threads, void *stream);
+/* The same call repeated `iters` times inside one kernel (the launch is paid once), for latency
+ * measurements; what = 5 adds nvshmem_barrier(team). */
+int nvshmem_perftest_device_team_coll_loop(int what, int team, void *dest, const void *src,
+                                           size_t n, int root, int iters, int scope, int threads,
+                                           void *stream);
 /* Every PE writes into its copy of `out` (4 + 64 ints): team_my_pe(a), team_n_pes(a),
  * team_my_pe(b), team_n_pes(b), then team_translate_pe(a, i, b) for i = 0..63, all evaluated in
  * device code. */

@@ -132,7 +132,9 @@ def load_perftest():
         "nvshmem_perftest_amo_matrix_cases": [],
         "nvshmem_perftest_amo_matrix": [vp, vp, vp, vp, vp, vp],
         "nvshmem_perftest_amo_contend": [vp, vp, vp, i32, i32, i32, vp],
+        "nvshmem_perftest_coll_sequence": [vp, vp, vp, i32, i32, i32, i32, i32, i32, vp],
         "nvshmem_perftest_device_team_coll": [i32, i32, vp, vp, sz, i32, i32, i32, vp],
+        "nvshmem_perftest_device_team_coll_loop": [i32, i32, vp, vp, sz, i32, i32, i32, i32, vp],
         "nvshmem_perftest_team_query": [vp, i32, i32, vp],
         "nvshmem_perftest_device_team_barrier": [vp, vp, i32, i32, i32, i32, vp],
         "nvshmem_perftest_device_reducescatter": [i32, i32, vp, vp, sz, i32, i32, vp],

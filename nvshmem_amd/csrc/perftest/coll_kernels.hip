@@ -78,13 +78,16 @@ __global__ void barrier_kernel(uint64_t *counter, uint64_t *errors, int rounds) 
 }
 
 // Collectives and queries on a team handle; PEs that are not members of `team` return at once.
-enum { kTeamReduce = 0, kTeamReducescatter = 1, kTeamFcollect = 2, kTeamAlltoall = 3, kTeamBroadcast = 4 };
+enum { kTeamReduce = 0, kTeamReducescatter = 1, kTeamFcollect = 2, kTeamAlltoall = 3, kTeamBroadcast = 4,
+       kTeamBarrier = 5 };
 
+// `iters` > 1 repeats the call inside the kernel, which is how the reference's device perftests
+// time a collective (perftest/device/coll/*_latency.cu): the launch is paid once.
 template <int SCOPE>
 __global__ void team_coll_kernel(int what, nvshmem_team_t team, void *dest, const void *src, size_t n,
-                                 int root) {
+                                 int root, int iters) {
     if (nvshmem_team_my_pe(team) < 0) return;
-    switch (what) {
+    for (int it = 0; it < iters; ++it) switch (what) {
         case kTeamReduce:
             SCOPED_CALL(SCOPE, float_sum_reduce, team, (float *)dest, (const float *)src, n);
             break;
@@ -93,6 +96,7 @@ __global__ void team_coll_kernel(int what, nvshmem_team_t team, void *dest, cons
             break;
         case kTeamFcollect: SCOPED_CALL(SCOPE, fcollectmem, team, dest, src, n); break;
         case kTeamAlltoall: SCOPED_CALL(SCOPE, alltoallmem, team, dest, src, n); break;
+        case kTeamBarrier: SCOPED_CALL(SCOPE, barrier, team); break;
         default: SCOPED_CALL(SCOPE, broadcastmem, team, dest, src, n, root); break;
     }
 }
@@ -127,6 +131,47 @@ __global__ void team_barrier_kernel(uint64_t *counter, uint64_t *errors, int rou
         SCOPED_CALL(SCOPE, team_sync, team);
     }
     if (threadIdx.x == 0) *(uint64_t *)nvshmem_ptr(errors, me) += bad;
+}
+
+// Many collectives back to back without any barrier in between (sync_between = 0) or with one
+// after every check (1): round r fills src[i] = gen(me, r, i), then runs an int32 sum reduce of n
+// elements, a broadcast of the same n elements from member r % npes and an fcollect of fc_bytes per
+// PE, all into dst, and folds a position-weighted checksum of dst into check[0] after each.
+__device__ inline int32_t ll_gen(int me, int r, int i) {
+    return (int32_t)(((uint32_t)me * 1000003u + (uint32_t)r * 7919u + (uint32_t)i * 31u) & 0x7fffffffu);
+}
+__device__ inline uint64_t ll_checksum(uint64_t h, const int32_t *words, size_t n) {
+    uint64_t s = 0;
+    for (size_t i = 0; i < n; ++i) s += (uint64_t)(uint32_t)words[i] * (2 * (uint64_t)i + 1);
+    return h * 1000003ull + s;
+}
+template <int SCOPE>
+__global__ void coll_sequence_kernel(int32_t *src, int32_t *dst, uint64_t *check, int n, int fc_bytes,
+                                     int rounds, int sync_between) {
+    const int me = nvshmem_my_pe(), np = nvshmem_n_pes();
+    int32_t *my_src = (int32_t *)nvshmem_ptr(src, me);
+    const int32_t *my_dst = (const int32_t *)nvshmem_ptr(dst, me);
+    uint64_t h = 0;
+    for (int r = 0; r < rounds; ++r) {
+        for (int i = threadIdx.x; i < n; i += blockDim.x) my_src[i] = ll_gen(me, r, i);
+        __syncthreads();
+        SCOPED_CALL(SCOPE, int32_sum_reduce, NVSHMEM_TEAM_WORLD, dst, src, (size_t)n);
+        __syncthreads();
+        if (threadIdx.x == 0) h = ll_checksum(h, my_dst, (size_t)n);
+        __syncthreads();
+        if (sync_between) SCOPED_CALL(SCOPE, barrier_all);
+        SCOPED_CALL(SCOPE, broadcastmem, NVSHMEM_TEAM_WORLD, dst, src, (size_t)n * 4, r % np);
+        __syncthreads();
+        if (threadIdx.x == 0) h = ll_checksum(h, my_dst, (size_t)n);
+        __syncthreads();
+        if (sync_between) SCOPED_CALL(SCOPE, barrier_all);
+        SCOPED_CALL(SCOPE, fcollectmem, NVSHMEM_TEAM_WORLD, dst, src, (size_t)fc_bytes);
+        __syncthreads();
+        if (threadIdx.x == 0) h = ll_checksum(h, my_dst, (size_t)fc_bytes * np / 4);
+        __syncthreads();
+        if (sync_between) SCOPED_CALL(SCOPE, barrier_all);
+    }
+    if (threadIdx.x == 0) *(uint64_t *)nvshmem_ptr(check, me) = h;
 }
 
 template <typename... Args>
@@ -244,16 +289,24 @@ int nvshmem_perftest_device_barrier(uint64_t *counter, uint64_t *errors, int rou
         barrier_kernel<NVSHMEM_PERFTEST_SCOPE_THREAD>, threads, stream, counter, errors, rounds);
 }
 
-int nvshmem_perftest_device_team_coll(int what, int team, void *dest, const void *src, size_t n,
-                                      int root, int scope, int threads, void *stream) {
-    if (!perftest::ready() || scope < 0 || scope > 2 || what < kTeamReduce || what > kTeamBroadcast ||
-        !perftest::check_launch(1, threads) || !perftest::check_range(dest, 1) ||
+int nvshmem_perftest_device_team_coll_loop(int what, int team, void *dest, const void *src,
+                                           size_t n, int root, int iters, int scope, int threads,
+                                           void *stream) {
+    if (!perftest::ready() || scope < 0 || scope > 2 || what < kTeamReduce || what > kTeamBarrier ||
+        iters < 1 || !perftest::check_launch(1, threads) || !perftest::check_range(dest, 1) ||
         !perftest::check_range(src, 1))
         return NVSHMEMX_ERROR_INVALID_VALUE;
-    return launch_scoped<int, nvshmem_team_t, void *, const void *, size_t, int>(
+    return launch_scoped<int, nvshmem_team_t, void *, const void *, size_t, int, int>(
         scope, team_coll_kernel<NVSHMEM_PERFTEST_SCOPE_BLOCK>, team_coll_kernel<NVSHMEM_PERFTEST_SCOPE_WARP>,
         team_coll_kernel<NVSHMEM_PERFTEST_SCOPE_THREAD>, threads, stream, what, (nvshmem_team_t)team,
-        dest, src, n, root);
+        dest, src, n, root, iters);
+}
+
+int nvshmem_perftest_device_team_coll(int what, int team, void *dest, const void *src, size_t n,
+                                      int root, int scope, int threads, void *stream) {
+    if (what == kTeamBarrier) return NVSHMEMX_ERROR_INVALID_VALUE;
+    return nvshmem_perftest_device_team_coll_loop(what, team, dest, src, n, root, 1, scope, threads,
+                                                  stream);
 }
 
 int nvshmem_perftest_team_query(int *out, int team_a, int team_b, void *stream) {
@@ -276,6 +329,22 @@ int nvshmem_perftest_device_team_barrier(uint64_t *counter, uint64_t *errors, in
         scope, team_barrier_kernel<NVSHMEM_PERFTEST_SCOPE_BLOCK>,
         team_barrier_kernel<NVSHMEM_PERFTEST_SCOPE_WARP>, team_barrier_kernel<NVSHMEM_PERFTEST_SCOPE_THREAD>,
         threads, stream, counter, errors, rounds, (nvshmem_team_t)team);
+}
+
+int nvshmem_perftest_coll_sequence(int32_t *src, int32_t *dst, uint64_t *check, int n, int fc_bytes,
+                                   int rounds, int sync_between, int scope, int threads, void *stream) {
+    const size_t np = (size_t)nvshmem_n_pes();
+    if (!perftest::ready() || scope < 0 || scope > 2 || n < 1 || fc_bytes < 4 || fc_bytes % 4 ||
+        rounds < 1 || !perftest::check_launch(1, threads) ||
+        !perftest::check_range(src, (size_t)n * 4 > (size_t)fc_bytes ? (size_t)n * 4 : (size_t)fc_bytes) ||
+        !perftest::check_range(dst, (size_t)n * 4 > fc_bytes * np ? (size_t)n * 4 : fc_bytes * np) ||
+        !perftest::check_range(check, sizeof(uint64_t)))
+        return NVSHMEMX_ERROR_INVALID_VALUE;
+    if ((size_t)fc_bytes > (size_t)n * 4) return NVSHMEMX_ERROR_INVALID_VALUE;  // fcollect sends src[0, fc_bytes)
+    return launch_scoped<int32_t *, int32_t *, uint64_t *, int, int, int, int>(
+        scope, coll_sequence_kernel<NVSHMEM_PERFTEST_SCOPE_BLOCK>,
+        coll_sequence_kernel<NVSHMEM_PERFTEST_SCOPE_WARP>, coll_sequence_kernel<NVSHMEM_PERFTEST_SCOPE_THREAD>,
+        threads, stream, src, dst, check, n, fc_bytes, rounds, sync_between);
 }
 
 }  // extern "C"

@@ -27,6 +27,7 @@ struct TeamTable {
     nvshmem_team_config_t config[NVSHMEMI_AMD_MAX_TEAMS];
     long config_mask[NVSHMEMI_AMD_MAX_TEAMS];
     char *dev = nullptr;
+    char *ll = nullptr;  // packet buffers of the low-latency collectives, per (team, PE)
     nvshmemi_amd_team_view_t *dev_views() const { return (nvshmemi_amd_team_view_t *)dev; }
     nvshmemi_amd_team_view_t *dev_groups() const {
         return dev_views() + NVSHMEMI_AMD_MAX_TEAMS * NVSHMEMI_AMD_MAX_PES;

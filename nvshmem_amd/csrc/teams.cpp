@@ -5,6 +5,7 @@
 // every (handle, PE) pair, and one handle can name a family of disjoint teams (all rows of a 2-D
 // split).  No per-team scratch is carved from the heap: the only per-team state the load/store
 // collectives need is one row of barrier arrival words per PE.
+#include <cstdlib>
 #include <cstring>
 
 #include "nvshmem.h"
@@ -20,6 +21,10 @@ const nvshmemi_amd_team_view_t kNotMember = {0, 1, 0, -1};
 
 bool handle_ok(const Runtime &rt, nvshmem_team_t team) {
     return team >= 0 && team < kMaxTeams && rt.teams.used[team];
+}
+
+size_t ll_bytes_per_team(const Runtime &rt) {
+    return (size_t)rt.npes * NVSHMEMI_AMD_LL_BUFFERS * 2 * NVSHMEMI_AMD_LL_PAYLOAD_BYTES;
 }
 
 // distinct member sets of the handle, in order of their first PE
@@ -49,6 +54,9 @@ bool upload_team(Runtime &rt, int team) {
     if (e == hipSuccess)
         e = hipMemset(tt.dev_sync() + (size_t)team * kMaxPes * NVSHMEMI_AMD_TEAM_SYNC_WORDS, 0,
                       sizeof(uint64_t) * kMaxPes * NVSHMEMI_AMD_TEAM_SYNC_WORDS);
+    // ... nor packets whose flags its restarted call counter would accept
+    if (e == hipSuccess && tt.ll)
+        e = hipMemset(tt.ll + (size_t)team * ll_bytes_per_team(rt), 0, ll_bytes_per_team(rt));
     if (e != hipSuccess) {
         set_error("team table upload failed: %s", hipGetErrorString(e));
         return false;
@@ -125,6 +133,24 @@ bool teams_init(Runtime &rt) {
         set_error("team table: hipMemset failed");
         return false;
     }
+    // packet buffers of the low-latency collectives; NVSHMEM_AMD_DISABLE_LL=1 leaves them out and
+    // every in-kernel collective takes its copy-and-barrier path
+    const char *no_ll = getenv("NVSHMEM_AMD_DISABLE_LL");
+    if (!(no_ll && no_ll[0] == '1')) {
+        const size_t ll_bytes = ll_bytes_per_team(rt) * kMaxTeams;
+        e = hipMalloc(&mem, ll_bytes);
+        if (e != hipSuccess || !mem) {
+            (void)hipGetLastError();
+            set_error("team table: hipMalloc of %zu bytes of packet buffers failed: %s", ll_bytes,
+                      hipGetErrorString(e));
+            return false;
+        }
+        tt.ll = (char *)mem;
+        if (hipMemset(mem, 0, ll_bytes) != hipSuccess) {
+            set_error("team table: hipMemset failed");
+            return false;
+        }
+    }
     for (int t = 0; t < kMaxTeams; ++t) {
         tt.used[t] = false;
         tt.ngroups[t] = 0;
@@ -146,12 +172,15 @@ bool teams_init(Runtime &rt) {
         if (!upload_team(rt, t)) return false;
     rt.dev.team_views = tt.dev_views();
     rt.dev.team_sync = tt.dev_sync();
+    rt.dev.ll_buffers = tt.ll;
     return true;
 }
 
 void teams_finalize(Runtime &rt) {
     if (rt.teams.dev) (void)hipFree(rt.teams.dev);
+    if (rt.teams.ll) (void)hipFree(rt.teams.ll);
     rt.teams.dev = nullptr;
+    rt.teams.ll = nullptr;
     for (int t = 0; t < kMaxTeams; ++t) rt.teams.used[t] = false;
 }
 
