@@ -9,6 +9,10 @@
 // the default scope is one row per wavefront with no block-wide synchronisation in the loop.
 #include <hip/hip_runtime.h>
 
+// A row is 14 vectors per lane: rounds of 8 + 4 + 2 keep more loads in flight than the default
+// 4 + 4 + 4 + 2 (measured 5 % faster for dispatch and combine).
+#define NVSHMEMI_AMD_COPY_UNROLL 8
+
 #include "nvshmem_perftest.h"
 #include "nvshmemx.h"
 #include "perftest_common.hpp"
