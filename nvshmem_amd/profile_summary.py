@@ -45,13 +45,14 @@ def counter_avg(directory, counter):
     return {_short(n): (v, c) for n, v, c in rows}
 
 
-# workloads of nvshmem_amd/profile_workloads.py: kernel -> (file name, description, algorithmic bytes)
+# workloads of nvshmem_amd/profile_workloads.py:
+# leading part of the kernel name as the trace prints it -> (file name, description, algorithmic bytes)
 WORKLOADS = {
     "ring_rma_kernel<2, false>": (
         "ring_rma_kernel_put_block_8pe_256MiB.txt",
         "put_block: nvshmemx_putmem_block ring, 8 logical PEs x 256 MiB, 65536 blocks x 128 threads per PE.\n"
         "Algorithmic bytes per launch: 8 x 256 MiB read + 8 x 256 MiB written = 4 GiB.", 4 << 30),
-    "reduce_vector_kernel<float, 5, 8, true>": (
+    "reduce_vector_kernel<float, 5, 8, true, false,": (
         "reduce_vector_kernel_float_sum_8pe_64Mi.txt",
         "sum_reduce: nvshmemx_float_sum_reduce_on_stream, 8 logical PEs x 2^26 fp32.\n"
         "Algorithmic bytes per launch: 8 sources read once + 8 destinations written once = 4 GiB.", 4 << 30),
@@ -66,6 +67,16 @@ WORKLOADS = {
         "segment_copy_kernel_fcollect_16pe_4Mi_fp32.txt",
         "fcollect: nvshmemx_float_fcollect_on_stream, 16 logical PEs x 2^22 fp32.\n"
         "Algorithmic bytes per launch: 256 MiB read + 16 x 256 MiB written = 4.25 GiB.", (17 * 256) << 20),
+    "reduce_vector_kernel<float, 5, 8, true, true,": (
+        "reduce_vector_kernel_float_sum_reducescatter_8pe_8Mi.txt",
+        "reducescatter: nvshmemx_float_sum_reducescatter_on_stream, 8 logical PEs, source 8 x 2^23 fp32\n"
+        "(256 MiB) per PE, result 2^23 fp32 (32 MiB) per PE.\n"
+        "Algorithmic bytes per launch: 8 sources of 256 MiB read once + 8 results of 32 MiB written = 2.25 GiB.",
+        (9 * 256) << 20),
+    "segment_copy_kernel<2, 1, false>": (
+        "segment_copy_kernel_broadcast_8pe_256MiB.txt",
+        "broadcast: nvshmemx_broadcastmem_on_stream, 8 logical PEs, 256 MiB from PE 3.\n"
+        "Algorithmic bytes per launch: 256 MiB read + 8 x 256 MiB written = 2.25 GiB.", (9 * 256) << 20),
     "plain_copy_kernel": (
         "plain_copy_kernel_calibration_1GiB.txt",
         "Counter calibration: plain one-vector-per-thread copy, 1 GiB read + 1 GiB written.", 2 << 30),
@@ -83,14 +94,20 @@ Hardware: one MI355X (gfx950), ROCm 7.2.  Durations are per dispatch from the ke
 
 def write_profiles(directory, stats, fetch, write, fscale, wscale):
     os.makedirs(directory, exist_ok=True)
+    def find(table, prefix):
+        hits = [k for k in table if k.startswith(prefix)]
+        return hits[0] if len(hits) == 1 else None
+
     by_name = {s[0]: s for s in stats}
-    for kernel, (fname, desc, alg) in WORKLOADS.items():
-        if kernel not in by_name:
+    for prefix, (fname, desc, alg) in WORKLOADS.items():
+        kernel = find(by_name, prefix)
+        if kernel is None:
             continue
         name, calls, avg, lo, hi = by_name[kernel]
         lines = [desc, "", COMMANDS, "",
                  "%-46s %6s %12s %12s %12s" % ("kernel", "calls", "avg us", "min us", "max us"),
-                 "%-46s %6d %12.2f %12.2f %12.2f" % (name[:46], calls, avg, lo, hi), ""]
+                 "%-46s %6d %12.2f %12.2f %12.2f" % (name[:46], calls, avg, lo, hi), "",
+                 "full kernel name: " + name, ""]
         if fscale and wscale and kernel in fetch and kernel in write:
             f, w = fetch[kernel][0], write[kernel][0]
             lines += ["counters (KiB per dispatch): FETCH_SIZE %.1f  WRITE_SIZE %.1f" % (f, w),

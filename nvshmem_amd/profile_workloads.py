@@ -5,8 +5,9 @@
     rocprofv3 --pmc WRITE_SIZE -d <out> -- python3 nvshmem_amd/profile_workloads.py
 
 Workloads (same shapes as bench.py): plain_copy calibration (1 GiB read + 1 GiB written),
-put_block (8 PEs x 256 MiB), float sum reduce (8 PEs x 2^26), then with 16 PEs alltoall and
-fcollect (2^22 fp32 per PE).  Buffers are zero-filled: only traffic and time matter here.
+put_block (8 PEs x 256 MiB), float sum reduce (8 PEs x 2^26), float sum reducescatter (8 PEs, 256 MiB
+source per PE), broadcast (8 PEs x 256 MiB), then with 16 PEs alltoall and fcollect (2^22 fp32 per
+PE).  Buffers are zero-filled: only traffic and time matter here.
 """
 import argparse
 import os
@@ -51,6 +52,26 @@ def main():
     red = _lib.typed_coll(rt.lib, "nvshmemx_float_sum_reduce_on_stream", True)
     for _ in range(args.iters):
         assert red(N.TEAM_WORLD, dst, src, n, None) == 0
+    hip.synchronize()
+    rt.finalize()
+
+    # reducescatter (source 8 blocks of 2^23 fp32 per PE) and broadcast (256 MiB from PE 3)
+    n = 1 << 23
+    rt = N.Runtime(npes=8, symmetric_size=9 * n * 4 + (64 << 20))
+    src = rt.calloc(8 * n, 4)
+    dst = rt.calloc(n, 4)
+    for _ in range(args.iters):
+        rt.reducescatter("float", "sum", dst, src, n, stream=None)
+    hip.synchronize()
+    rt.free(dst)
+    dst = None
+    rt.finalize()
+    S = 1 << 28
+    rt = N.Runtime(npes=8, symmetric_size=2 * S + (64 << 20))
+    src = rt.calloc(S, 1)
+    dst = rt.calloc(S, 1)
+    for _ in range(args.iters):
+        rt.broadcastmem(dst, src, S, 3)
     hip.synchronize()
     rt.finalize()
 
