@@ -8,7 +8,8 @@ sweep: every one of 8 logical PEs moves 256 MiB to its right neighbour with
 nvshmemx_putmem_block; a "step" is one such exchange (one kernel launch carrying all PEs).
 `value` is algorithmic bytes (payload read once + written once, all PEs) per second, inputs
 already resident in HBM.  sum_reduce (fp32, 8 PEs x 2^26 elements) and alltoall (fp32, 16 PEs x 2^22
-elements) are measured the same way and reported under "workloads".  The CPU oracle is timed on
+elements), a 1 GiB alltoall, reducescatter and broadcast are measured the same way and reported under
+"workloads".  The CPU oracle is timed on
 a bounded sample of each workload on this host's cores as a reported baseline.
 """
 import argparse
@@ -31,6 +32,8 @@ MEASURED_TRAFFIC_BYTES = {
     "sum_reduce": (2048 + 2048) << 20,   # profiles/reduce_vector_kernel_float_sum_8pe_64Mi.txt
     "alltoall": (256 + 256) << 20,       # profiles/segment_copy_kernel_alltoall_16pe_4Mi_fp32.txt
     "alltoall_1GiB": None,              # not profiled
+    "reducescatter": (2048 + 256) << 20,  # profiles/reduce_vector_kernel_float_sum_reducescatter_8pe_8Mi.txt
+    "broadcast": (256 + 2048) << 20,      # profiles/segment_copy_kernel_broadcast_8pe_256MiB.txt
 }
 
 # put_block launch shape: each block moves a contiguous 4 KiB slice (short-lived blocks keep the
@@ -190,6 +193,77 @@ def bench_alltoall(N, O, hip, np, steps, warmup, cpu_budget, n=1 << 22, name="al
     }
 
 
+def bench_reducescatter(N, O, hip, np, steps, warmup, cpu_budget):
+    npes, n = 8, 1 << 23
+    with _runtime(N, npes, 9 * n * 4 + (64 << 20)) as rt:
+        src = rt.malloc(npes * n * 4); dst = rt.malloc(n * 4)
+        data = O.fill_all("f32", npes, npes * n, 9)
+        rt.upload_all(src, data)
+        from nvshmem_amd import _lib
+        fn = _lib.typed_coll(rt.lib, "nvshmemx_float_sum_reducescatter_on_stream", True)
+
+        def step():
+            rc = fn(N.TEAM_WORLD, dst, src, n, None)
+            if rc != 0:
+                raise RuntimeError("reducescatter failed: %d %s" % (rc, rt.last_error()))
+        wall, ev = _time_steps(step, steps, warmup, hip)
+        sample = 1 << 20
+        pe = 5
+        want = O.reducescatter("f32", "sum", np.ascontiguousarray(
+            data.reshape(npes, npes, n)[:, :, :sample].reshape(npes, npes * sample)))[pe]
+        got = rt.download(dst, pe, (sample,), np.float32)
+        ok = bool(np.array_equal(got.view(np.uint32), want.view(np.uint32)))
+        rt.free(src); rt.free(dst)
+    alg = (npes + 1) * npes * n * 4
+    cores = min(16, O.lib().oracle_get_threads())
+    O.lib().oracle_set_threads(cores)
+    cs = 1 << 20
+    host = np.ascontiguousarray(data[:, :npes * cs])
+    best, passes = _cpu_time(lambda: O.reducescatter("f32", "sum", host), cpu_budget, 20)
+    cpu = {"value": round((npes + 1) * npes * cs * 4 / best / 1e9, 2), "unit": "GB/s", "cores": cores,
+           "kind": "port", "sample": "oracle_reducescatter f32 sum, 8 PEs x 8 x 2^20 elements, best of %d "
+                                     "passes" % passes}
+    return {
+        "name": "reducescatter", "dtype": "f32", "verified": ok, "algorithmic_bytes": alg,
+        "wall_ms": wall, "kernel_ms": ev,
+        "config": {"workload": "reducescatter: nvshmemx_float_sum_reducescatter_on_stream, 8 logical PEs, "
+                               "source 8 x 2^23 fp32 (256 MiB) per PE, result 2^23 fp32 per PE",
+                   "npes": npes, "nreduce": n},
+        "kernel": "reduce_vector_kernel<float, sum, 8, scatter>",
+        "cpu_baseline": cpu,
+    }
+
+
+def bench_broadcast(N, O, hip, np, steps, warmup, cpu_budget):
+    npes, nbytes, root = 8, 1 << 28, 3
+    with _runtime(N, npes, 2 * nbytes + (64 << 20)) as rt:
+        src = rt.malloc(nbytes); dst = rt.malloc(nbytes)
+        rows = [O.fill("bytes", nbytes, 12, pe) if pe == root else np.zeros(1, np.uint8) for pe in range(npes)]
+        rt.upload(src, root, rows[root])
+
+        def step():
+            rc = rt.lib.nvshmemx_broadcastmem_on_stream(N.TEAM_WORLD, dst, src, nbytes, root, None)
+            if rc != 0:
+                raise RuntimeError("broadcast failed: %d %s" % (rc, rt.last_error()))
+        wall, ev = _time_steps(step, steps, warmup, hip)
+        ok = all(bool(np.array_equal(rt.download(dst, pe, (nbytes,), np.uint8), rows[root])) for pe in (0, 3, 7))
+        rt.free(src); rt.free(dst)
+    alg = (npes + 1) * nbytes
+    sample = 1 << 26
+    host = np.ascontiguousarray(np.broadcast_to(rows[root][:sample], (npes, sample)))
+    best, passes = _cpu_time(lambda: O.broadcast(host, root), cpu_budget, 20)
+    cpu = {"value": round((npes + 1) * sample / best / 1e9, 2), "unit": "GB/s", "cores": 1, "kind": "port",
+           "sample": "oracle_broadcast (memcpy per PE), 8 PEs x 64 MiB, best of %d passes" % passes}
+    return {
+        "name": "broadcast", "dtype": "u8", "verified": ok, "algorithmic_bytes": alg,
+        "wall_ms": wall, "kernel_ms": ev,
+        "config": {"workload": "broadcast: nvshmemx_broadcastmem_on_stream, 8 logical PEs, 256 MiB from PE 3",
+                   "npes": npes, "bytes": nbytes, "root": root},
+        "kernel": "segment_copy_kernel<broadcast>",
+        "cpu_baseline": cpu,
+    }
+
+
 class _runtime:
     def __init__(self, N, npes, size):
         self.N, self.npes, self.size = N, npes, size
@@ -242,6 +316,8 @@ def main():
     a2a = bench_alltoall(N, O, hip, np, args.steps, args.warmup, args.cpu_seconds)
     a2a_big = bench_alltoall(N, O, hip, np, args.steps, args.warmup, 1.0, n=1 << 24,
                              name="alltoall_1GiB")
+    rsc = bench_reducescatter(N, O, hip, np, args.steps, args.warmup, 1.0)
+    bca = bench_broadcast(N, O, hip, np, args.steps, args.warmup, 1.0)
 
     head = put
     value = head["algorithmic_bytes"] / head["wall_ms"] / 1e6
@@ -264,9 +340,11 @@ def main():
                      "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBS, 4),
                      "traffic": MEASURED_TRAFFIC_BYTES[head["name"]], "kernel": head["kernel"]},
         "cpu_baseline": head["cpu_baseline"],
-        "verified": bool(put["verified"] and red["verified"] and a2a["verified"] and a2a_big["verified"]),
+        "verified": bool(put["verified"] and red["verified"] and a2a["verified"] and a2a_big["verified"]
+                         and rsc["verified"] and bca["verified"]),
         "workloads": {"put_block": _summarise(put), "sum_reduce": _summarise(red),
-                      "alltoall": _summarise(a2a), "alltoall_1GiB": _summarise(a2a_big)},
+                      "alltoall": _summarise(a2a), "alltoall_1GiB": _summarise(a2a_big),
+                      "reducescatter": _summarise(rsc), "broadcast": _summarise(bca)},
     }
     print(json.dumps(line))
     return 0 if line["verified"] else 1
