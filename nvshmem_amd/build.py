@@ -55,10 +55,15 @@ def _link(objs, out, extra=()):
     _run([HIPCC, "--offload-arch=gfx950", "-shared", "-fPIC", "-o", out] + objs + list(extra))
 
 
+BINDIR = os.path.join(ROOT, "nvshmem_amd", "bin")
+DRIVER_SOURCE = "perftest/perftest_main.cpp"   # command-line driver over both libraries
+
+
 def build_native(jobs=8):
     os.makedirs(LIBDIR, exist_ok=True)
     os.makedirs(OBJDIR, exist_ok=True)
-    sources = RUNTIME_SOURCES + [s for s in PERFTEST_SOURCES
+    os.makedirs(BINDIR, exist_ok=True)
+    sources = RUNTIME_SOURCES + [s for s in PERFTEST_SOURCES + [DRIVER_SOURCE]
                                  if os.path.exists(os.path.join(CSRC, s))]
     with ThreadPoolExecutor(max_workers=jobs) as pool:
         objs = dict(zip(sources, pool.map(_compile, sources)))
@@ -68,6 +73,10 @@ def build_native(jobs=8):
     if perf:
         _link(perf, os.path.join(LIBDIR, "libnvshmem_amd_perftest.so"),
               ["-L" + LIBDIR, "-lnvshmem_amd", "-Wl,-rpath,$ORIGIN"])
+    if perf and DRIVER_SOURCE in objs:
+        _run([HIPCC, "--offload-arch=gfx950", "-o", os.path.join(BINDIR, "nvshmem_perftest"),
+              objs[DRIVER_SOURCE], "-L" + LIBDIR, "-lnvshmem_amd_perftest", "-lnvshmem_amd",
+              "-Wl,-rpath,$ORIGIN/../lib"])
     return runtime
 
 

@@ -1,0 +1,266 @@
+// Command-line performance driver over the public C ABI, with the conventions of the reference's
+// perftest programs (perftest/common/utils.cu:661-689 table layout; warm-up then timed iterations
+// between events; sizes doubling from --min to --max; bandwidth = payload bytes / time as in
+// perftest/device/pt-to-pt/shmem_put_bw.cu:118-128, latency in microseconds as in
+// perftest/device/coll/*_latency.cu).
+//
+//   nvshmem_perftest <test> [--npes N] [--min BYTES] [--max BYTES] [--iters K] [--warmup W]
+//                           [--blocks B] [--threads T] [--scope thread|warp|block]
+//
+// tests: put_bw get_bw                      device put/get, every PE to its right neighbour
+//        reduce reducescatter fcollect alltoall broadcast
+//                                           host-launched collectives on a stream (fp32 sum for the
+//                                           reductions); size = bytes each PE contributes
+//        coll_latency                       the same five calls made inside a kernel, the call
+//                                           repeated --iters times in one launch
+//        barrier_latency                    nvshmem_barrier_all inside a kernel
+#include <hip/hip_runtime.h>
+
+#include <cstdio>
+#include <cstdlib>
+#include <cstring>
+#include <string>
+#include <vector>
+
+#include "nvshmem.h"
+#include "nvshmem_perftest.h"
+
+namespace {
+
+struct Options {
+    std::string test;
+    int npes = 8;
+    size_t min_bytes = 8, max_bytes = (size_t)64 << 20;
+    int iters = 20, warmup = 5;
+    int blocks = 0, threads = 0;  // 0: a shape that fills the GPU
+    int scope = NVSHMEM_PERFTEST_SCOPE_BLOCK;
+};
+
+[[noreturn]] void usage(const char *why) {
+    fprintf(stderr, "nvshmem_perftest: %s\nusage: nvshmem_perftest <put_bw|get_bw|reduce|reducescatter|fcollect|"
+                    "alltoall|broadcast|coll_latency|barrier_latency> [--npes N] [--min B] [--max B] [--iters K] "
+                    "[--warmup W] [--blocks B] [--threads T] [--scope thread|warp|block]\n", why);
+    exit(2);
+}
+
+size_t parse_size(const char *s) {
+    char *end = nullptr;
+    double v = strtod(s, &end);
+    if (end == s || v < 0) usage("bad size");
+    switch (*end) {
+        case 'k': case 'K': v *= 1024.0; break;
+        case 'm': case 'M': v *= 1024.0 * 1024.0; break;
+        case 'g': case 'G': v *= 1024.0 * 1024.0 * 1024.0; break;
+        default: break;
+    }
+    return (size_t)v;
+}
+
+Options parse(int argc, char **argv) {
+    if (argc < 2) usage("no test named");
+    Options o;
+    o.test = argv[1];
+    for (int i = 2; i < argc; ++i) {
+        const std::string a = argv[i];
+        auto next = [&]() -> const char * {
+            if (i + 1 >= argc) usage(("missing value after " + a).c_str());
+            return argv[++i];
+        };
+        if (a == "--npes") o.npes = atoi(next());
+        else if (a == "--min") o.min_bytes = parse_size(next());
+        else if (a == "--max") o.max_bytes = parse_size(next());
+        else if (a == "--iters") o.iters = atoi(next());
+        else if (a == "--warmup") o.warmup = atoi(next());
+        else if (a == "--blocks") o.blocks = atoi(next());
+        else if (a == "--threads") o.threads = atoi(next());
+        else if (a == "--scope") {
+            const std::string s = next();
+            if (s == "thread") o.scope = NVSHMEM_PERFTEST_SCOPE_THREAD;
+            else if (s == "warp") o.scope = NVSHMEM_PERFTEST_SCOPE_WARP;
+            else if (s == "block") o.scope = NVSHMEM_PERFTEST_SCOPE_BLOCK;
+            else usage("bad scope");
+        } else usage(("unknown option " + a).c_str());
+    }
+    if (o.iters < 1 || o.warmup < 0 || o.min_bytes < 1 || o.max_bytes < o.min_bytes) usage("bad range");
+    return o;
+}
+
+const char *scope_name(int scope) {
+    return scope == NVSHMEM_PERFTEST_SCOPE_THREAD ? "thread" : scope == NVSHMEM_PERFTEST_SCOPE_WARP ? "warp" : "block";
+}
+
+#define CHECK_HIP(x)                                                                         \
+    do {                                                                                     \
+        hipError_t e_ = (x);                                                                 \
+        if (e_ != hipSuccess) {                                                              \
+            fprintf(stderr, "%s failed: %s (%s:%d)\n", #x, hipGetErrorString(e_), __FILE__, __LINE__); \
+            exit(1);                                                                         \
+        }                                                                                    \
+    } while (0)
+
+// average milliseconds of one call of fn: `warmup` untimed calls, then `iters` between two events
+template <typename Fn>
+double time_ms(Fn fn, int iters, int warmup) {
+    for (int i = 0; i < warmup; ++i)
+        if (fn() != 0) {
+            fprintf(stderr, "nvshmem_perftest: call failed: %s\n", nvshmemx_amd_last_error());
+            exit(1);
+        }
+    CHECK_HIP(hipDeviceSynchronize());
+    hipEvent_t a, b;
+    CHECK_HIP(hipEventCreate(&a));
+    CHECK_HIP(hipEventCreate(&b));
+    CHECK_HIP(hipEventRecord(a, nullptr));
+    for (int i = 0; i < iters; ++i) (void)fn();
+    CHECK_HIP(hipEventRecord(b, nullptr));
+    CHECK_HIP(hipEventSynchronize(b));
+    float ms = 0;
+    CHECK_HIP(hipEventElapsedTime(&ms, a, b));
+    CHECK_HIP(hipEventDestroy(a));
+    CHECK_HIP(hipEventDestroy(b));
+    return (double)ms / iters;
+}
+
+void print_table(const char *job, const char *scope, const char *what, const char *units,
+                 const std::vector<size_t> &sizes, const std::vector<double> &values) {
+    char head[64];
+    snprintf(head, sizeof head, "%s (%s)", what, units);
+    printf("#%10s\n%-10s  %-8s  %-16s\n", job, "size(B)", "scope", head);
+    for (size_t i = 0; i < sizes.size(); ++i) printf("%-10zu  %-8s  %-16.6f\n", sizes[i], scope, values[i]);
+}
+
+std::vector<size_t> sweep(const Options &o, size_t multiple) {
+    std::vector<size_t> out;
+    for (size_t s = o.min_bytes; s <= o.max_bytes; s *= 2) {
+        const size_t r = (s + multiple - 1) / multiple * multiple;
+        if (out.empty() || out.back() != r) out.push_back(r);
+    }
+    return out;
+}
+
+int run_rma(const Options &o, bool is_get) {
+    void *src = nvshmem_malloc(o.max_bytes), *dst = nvshmem_malloc(o.max_bytes);
+    if (!src || !dst) return 1;
+    std::vector<size_t> sizes = sweep(o, 1);
+    std::vector<double> gbs;
+    for (size_t bytes : sizes) {
+        // default: 4 KiB per block of 128 threads, the shape that fills the GPU (bounded below by 1)
+        int threads = o.threads ? o.threads : 128;
+        long blocks = o.blocks ? o.blocks : (long)((bytes + 4095) / 4096);
+        if (blocks < 1) blocks = 1;
+        if (blocks > (1 << 22)) blocks = 1 << 22;
+        const double ms = time_ms([&] {
+            return nvshmem_perftest_ring_rma(dst, src, bytes, (int)blocks, threads, o.scope, is_get ? 1 : 0, 1, nullptr);
+        }, o.iters, o.warmup);
+        gbs.push_back((double)bytes / ms / 1e6);  // payload of one PE, as the reference reports it
+    }
+    print_table(is_get ? "shmem_get_bw" : "shmem_put_bw", scope_name(o.scope), "BW", "GB/s per PE", sizes, gbs);
+    printf("# %d PEs move that payload at once: aggregate payload = npes x BW, HBM traffic = 2 x that\n", o.npes);
+    nvshmem_free(src);
+    nvshmem_free(dst);
+    return 0;
+}
+
+enum { kReduce, kReducescatter, kFcollect, kAlltoall, kBroadcast };
+
+int run_host_collective(const Options &o, int what) {
+    const size_t n = (size_t)o.npes;
+    // bytes = what one PE contributes; the larger of source and dest per PE is npes times that
+    void *src = nvshmem_malloc(o.max_bytes * n), *dst = nvshmem_malloc(o.max_bytes * n);
+    if (!src || !dst) return 1;
+    std::vector<size_t> sizes = sweep(o, 4);
+    std::vector<double> us, gbs;
+    for (size_t bytes : sizes) {
+        double alg = 0;
+        const double ms = time_ms([&]() -> int {
+            switch (what) {
+                case kReduce:
+                    alg = 2.0 * n * bytes;
+                    return nvshmemx_float_sum_reduce_on_stream(NVSHMEM_TEAM_WORLD, (float *)dst, (const float *)src, bytes / 4, nullptr);
+                case kReducescatter:  // every PE holds npes blocks of `bytes`
+                    alg = (double)(n + 1) * n * bytes;
+                    return nvshmemx_float_sum_reducescatter_on_stream(NVSHMEM_TEAM_WORLD, (float *)dst, (const float *)src, bytes / 4, nullptr);
+                case kFcollect:
+                    alg = (double)(n + 1) * n * bytes;
+                    return nvshmemx_fcollectmem_on_stream(NVSHMEM_TEAM_WORLD, dst, src, bytes, nullptr);
+                case kAlltoall:  // `bytes` per destination
+                    alg = 2.0 * n * n * bytes;
+                    return nvshmemx_alltoallmem_on_stream(NVSHMEM_TEAM_WORLD, dst, src, bytes, nullptr);
+                default:
+                    alg = (double)(n + 1) * bytes;
+                    return nvshmemx_broadcastmem_on_stream(NVSHMEM_TEAM_WORLD, dst, src, bytes, 0, nullptr);
+            }
+        }, o.iters, o.warmup);
+        us.push_back(ms * 1e3);
+        gbs.push_back(alg / ms / 1e6);
+    }
+    static const char *names[] = {"reduction_on_stream", "reducescatter_on_stream", "fcollect_on_stream",
+                                  "alltoall_on_stream", "bcast_on_stream"};
+    print_table(names[what], "stream", "latency", "us", sizes, us);
+    print_table(names[what], "stream", "algorithmic BW", "GB/s", sizes, gbs);
+    nvshmem_free(src);
+    nvshmem_free(dst);
+    return 0;
+}
+
+int run_device_latency(const Options &o, bool barrier_only) {
+    const size_t n = (size_t)o.npes;
+    const size_t cap = barrier_only ? 64 : o.max_bytes;
+    void *src = nvshmem_malloc(cap * n), *dst = nvshmem_malloc(cap * n);
+    if (!src || !dst) return 1;
+    const int threads = o.threads ? o.threads : 256;
+    // per-call time = (launch with K + 1 calls - launch with 1 call) / K: the launch is paid once
+    auto latency_us = [&](int what, size_t count) {
+        auto one = [&] { return nvshmem_perftest_device_team_coll_loop(what, NVSHMEM_TEAM_WORLD, dst, src, count, 0, 1, o.scope, threads, nullptr); };
+        auto many = [&] { return nvshmem_perftest_device_team_coll_loop(what, NVSHMEM_TEAM_WORLD, dst, src, count, 0, o.iters + 1, o.scope, threads, nullptr); };
+        const double t1 = time_ms(one, 5, 2), tk = time_ms(many, 5, 2);
+        return (tk - t1) * 1e3 / o.iters;
+    };
+    if (barrier_only) {
+        printf("#barrier_latency\n%-8s  %-16s\n%-8s  %-16.6f\n", "scope", "latency (us)", scope_name(o.scope),
+               latency_us(5, 0));
+    } else {
+        std::vector<size_t> sizes = sweep(o, 4);
+        static const struct { int what; const char *job; } calls[] = {
+            {0, "reduction_latency"}, {1, "reducescatter_latency"}, {2, "fcollect_latency"},
+            {3, "alltoall_latency"}, {4, "bcast_latency"}};
+        for (const auto &c : calls) {
+            std::vector<double> us;
+            for (size_t bytes : sizes) us.push_back(latency_us(c.what, c.what <= 1 ? bytes / 4 : bytes));
+            print_table(c.job, scope_name(o.scope), "latency", "us", sizes, us);
+        }
+    }
+    nvshmem_free(src);
+    nvshmem_free(dst);
+    return 0;
+}
+
+}  // namespace
+
+int main(int argc, char **argv) {
+    const Options o = parse(argc, argv);
+    const bool device_lat = o.test == "coll_latency" || o.test == "barrier_latency";
+    // heap: source and dest of the largest size, times npes for the collectives
+    const bool rma = o.test == "put_bw" || o.test == "get_bw";
+    Options eff = o;
+    if (device_lat && o.max_bytes > ((size_t)1 << 20)) eff.max_bytes = (size_t)1 << 20;
+    const size_t per_pe = (rma ? 2 * eff.max_bytes : 2 * eff.max_bytes * (size_t)eff.npes) + ((size_t)16 << 20);
+    if (nvshmemx_amd_init(eff.npes, per_pe) != 0) {
+        fprintf(stderr, "nvshmem_perftest: init failed: %s\n", nvshmemx_amd_last_error());
+        return 1;
+    }
+    int rc;
+    if (o.test == "put_bw") rc = run_rma(eff, false);
+    else if (o.test == "get_bw") rc = run_rma(eff, true);
+    else if (o.test == "reduce") rc = run_host_collective(eff, kReduce);
+    else if (o.test == "reducescatter") rc = run_host_collective(eff, kReducescatter);
+    else if (o.test == "fcollect") rc = run_host_collective(eff, kFcollect);
+    else if (o.test == "alltoall") rc = run_host_collective(eff, kAlltoall);
+    else if (o.test == "broadcast") rc = run_host_collective(eff, kBroadcast);
+    else if (o.test == "coll_latency") rc = run_device_latency(eff, false);
+    else if (o.test == "barrier_latency") rc = run_device_latency(eff, true);
+    else usage("unknown test");
+    if (rc != 0) fprintf(stderr, "nvshmem_perftest: %s\n", nvshmemx_amd_last_error());
+    nvshmem_finalize();
+    return rc;
+}

@@ -1,0 +1,58 @@
+"""The command-line performance driver: runs in a child process against the built libraries and
+prints tables in the reference's perftest layout; the numbers are only checked for sanity here."""
+import os
+import subprocess
+
+import pytest
+
+pytestmark = pytest.mark.gpu
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+DRIVER = os.path.join(ROOT, "nvshmem_amd", "bin", "nvshmem_perftest")
+
+
+def _run(*args):
+    assert os.path.exists(DRIVER), "run `python -m nvshmem_amd.build` first"
+    proc = subprocess.run([DRIVER] + list(args), stdout=subprocess.PIPE, stderr=subprocess.PIPE, timeout=100)
+    assert proc.returncode == 0, proc.stderr.decode()
+    return proc.stdout.decode()
+
+
+def _rows(text, job):
+    """[(size, scope, value)] of the first table of `job`."""
+    lines = text.splitlines()
+    start = next(i for i, l in enumerate(lines) if l.strip() == "#" + job or l.split() == ["#" + job])
+    rows = []
+    for l in lines[start + 2:]:
+        if l.startswith("#") or not l.strip():
+            break
+        size, scope, value = l.split()
+        rows.append((int(size), scope, float(value)))
+    return rows
+
+
+def test_put_bw_and_collective_tables():
+    out = _run("put_bw", "--min", "1k", "--max", "16m", "--iters", "10")
+    rows = _rows(out, "shmem_put_bw")
+    assert [r[0] for r in rows] == [1024 << i for i in range(15)] and all(r[1] == "block" for r in rows)
+    assert rows[-1][2] > 100.0            # GB/s per PE at 16 MiB
+    out = _run("reduce", "--min", "4k", "--max", "4m", "--iters", "10", "--npes", "8")
+    lat = _rows(out, "reduction_on_stream")
+    assert len(lat) == 11 and all(v > 0 for _, _, v in lat)
+    out = _run("broadcast", "--min", "64", "--max", "64k", "--iters", "5", "--npes", "4")
+    assert len(_rows(out, "bcast_on_stream")) == 11
+
+
+def test_device_latency_tables():
+    out = _run("coll_latency", "--min", "8", "--max", "512", "--iters", "50", "--scope", "warp")
+    for job in ("reduction_latency", "reducescatter_latency", "fcollect_latency", "alltoall_latency", "bcast_latency"):
+        rows = _rows(out, job)
+        assert [r[0] for r in rows] == [8, 16, 32, 64, 128, 256, 512] and all(r[1] == "warp" for r in rows)
+        assert all(0.0 < v < 1000.0 for _, _, v in rows), (job, rows)
+    out = _run("barrier_latency", "--iters", "100")
+    assert "barrier_latency" in out
+
+
+def test_bad_arguments_are_refused():
+    proc = subprocess.run([DRIVER, "nonsense"], stdout=subprocess.PIPE, stderr=subprocess.PIPE, timeout=100)
+    assert proc.returncode == 2 and b"usage" in proc.stderr
