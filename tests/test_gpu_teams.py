@@ -276,11 +276,12 @@ def test_team_argument_errors(rt):
 # ---------------------------------------------------------------------------------------------
 # in-kernel collectives and barriers on teams
 # ---------------------------------------------------------------------------------------------
+# n = 517: copy-and-barrier paths; n = 12: the packet paths (one packet per lane) on every team
+@pytest.mark.parametrize("n", [517, 12])
 @pytest.mark.parametrize("scope,threads", [(N.SCOPE_THREAD, 64), (N.SCOPE_WARP, 128), (N.SCOPE_BLOCK, 256)])
-def test_device_scope_collectives_on_teams(rt, scope, threads):
+def test_device_scope_collectives_on_teams(rt, scope, threads, n):
     perf = rt.perftest()
-    rng = np.random.default_rng(50 + scope)
-    n = 517
+    rng = np.random.default_rng(50 + scope + n)
     x, y = rt.team_split_2d(N.TEAM_WORLD, 4)
     odd = rt.team_split_strided(N.TEAM_WORLD, 1, 2, 8)
     want2d = [O.team_split_2d(WORLD, 4, pe) for pe in range(NPES)]
@@ -345,3 +346,42 @@ def test_device_scope_collectives_on_teams(rt, scope, threads):
     rt.free(src); rt.free(dst)
     for t in (x, y, odd):
         rt.team_destroy(t)
+
+
+def test_a_reused_handle_starts_clean(rt):
+    """Packet flags and barrier epochs restart when a handle is reused by other members."""
+    perf = rt.perftest()
+    rng = np.random.default_rng(77)
+    n = 8
+    src = rt.malloc(4096); dst = rt.malloc(4096)
+    for round_, (start, stride, size) in enumerate(((0, 1, 4), (2, 3, 5), (1, 1, 15), (0, 2, 8))):
+        t = rt.team_split_strided(N.TEAM_WORLD, start, stride, size)
+        assert t == 6                                  # always the same, lowest free handle
+        members = [start + i * stride for i in range(size)]
+        for rep in range(3 + round_):                  # a different number of calls per life
+            data = rng.standard_normal((NPES, n)).astype(np.float32)
+            rt.upload_all(src, data)
+            rt.fill(dst, 0xCD, 4096)
+            note("reused handle round=%d rep=%d" % (round_, rep))
+            assert perf.nvshmem_perftest_device_team_coll(0, t, dst, src, n, 0, N.SCOPE_BLOCK, 256, None) == 0
+            rt.sync()
+            want = O.reduce("f32", "sum", data[members])
+            for pe in range(NPES):
+                got = rt.download(dst, pe, (n,), np.float32)
+                if pe in members:
+                    assert bits_equal(got, want), (round_, rep, pe)
+                else:
+                    assert (got.view(np.uint32) == 0xCDCDCDCD).all()
+            root = rep % size
+            assert perf.nvshmem_perftest_device_team_coll(4, t, dst, src, n * 4, root, N.SCOPE_WARP, 64, None) == 0
+            rt.sync()
+            for pe in members:
+                assert bits_equal(rt.download(dst, pe, (n,), np.float32), data[members[root]])
+        counter = rt.calloc(1, 8); errors = rt.calloc(1, 8)
+        assert perf.nvshmem_perftest_device_team_barrier(counter, errors, 5 + round_, t, N.SCOPE_BLOCK, 128, None) == 0
+        rt.sync()
+        assert (rt.download_all(errors, (1,), np.uint64) == 0).all()
+        rt.free(counter); rt.free(errors)
+        rt.team_destroy(t)
+    assert rt.read_timeout(0)[0] == 0
+    rt.free(src); rt.free(dst)
