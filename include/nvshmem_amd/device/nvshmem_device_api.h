@@ -198,7 +198,7 @@ NVSHMEMI_DEV uint64_t nvshmem_signal_wait_until(uint64_t *sig_addr, int cmp, uin
     return nvshmemi_wait_until<uint64_t>(sig_addr, cmp, cmp_val);
 }
 
-/* ---- typed wait / test (14 types) ---- */
+/* ---- typed wait / test (14 types): scalar, all / any / some, and the _vector forms ---- */
 #define NVSHMEMI_STAMP_WAIT(NAME, TYPE)                                                           \
     NVSHMEMI_DEV void nvshmem_##NAME##_wait_until(TYPE *ivar, int cmp, TYPE cmp_value) {          \
         nvshmemi_wait_until<TYPE>(ivar, cmp, cmp_value);                                          \
@@ -209,15 +209,62 @@ NVSHMEMI_DEV uint64_t nvshmem_signal_wait_until(uint64_t *sig_addr, int cmp, uin
     NVSHMEMI_DEV void nvshmem_##NAME##_wait_until_all(TYPE *ivars, size_t nelems,                 \
                                                       const int *status, int cmp,                 \
                                                       TYPE cmp_value) {                           \
-        for (size_t i = 0; i < nelems; ++i)                                                       \
-            if (!status || !status[i]) nvshmemi_wait_until<TYPE>(ivars + i, cmp, cmp_value);      \
+        nvshmemi_wait_until_all<TYPE, false>(ivars, nelems, status, cmp, &cmp_value);             \
+    }                                                                                             \
+    NVSHMEMI_DEV size_t nvshmem_##NAME##_wait_until_any(TYPE *ivars, size_t nelems,               \
+                                                        const int *status, int cmp,               \
+                                                        TYPE cmp_value) {                         \
+        return nvshmemi_wait_until_any<TYPE, false>(ivars, nelems, status, cmp, &cmp_value);      \
+    }                                                                                             \
+    NVSHMEMI_DEV size_t nvshmem_##NAME##_wait_until_some(TYPE *ivars, size_t nelems,              \
+                                                         size_t *indices, const int *status,      \
+                                                         int cmp, TYPE cmp_value) {               \
+        return nvshmemi_wait_until_some<TYPE, false>(ivars, nelems, indices, status, cmp,         \
+                                                     &cmp_value);                                 \
+    }                                                                                             \
+    NVSHMEMI_DEV void nvshmem_##NAME##_wait_until_all_vector(TYPE *ivars, size_t nelems,          \
+                                                             const int *status, int cmp,          \
+                                                             TYPE *cmp_values) {                  \
+        nvshmemi_wait_until_all<TYPE, true>(ivars, nelems, status, cmp, cmp_values);              \
+    }                                                                                             \
+    NVSHMEMI_DEV size_t nvshmem_##NAME##_wait_until_any_vector(TYPE *ivars, size_t nelems,        \
+                                                               const int *status, int cmp,        \
+                                                               TYPE *cmp_values) {                \
+        return nvshmemi_wait_until_any<TYPE, true>(ivars, nelems, status, cmp, cmp_values);       \
+    }                                                                                             \
+    NVSHMEMI_DEV size_t nvshmem_##NAME##_wait_until_some_vector(TYPE *ivars, size_t nelems,       \
+                                                                size_t *indices,                  \
+                                                                const int *status, int cmp,       \
+                                                                TYPE *cmp_values) {               \
+        return nvshmemi_wait_until_some<TYPE, true>(ivars, nelems, indices, status, cmp,          \
+                                                    cmp_values);                                  \
     }                                                                                             \
     NVSHMEMI_DEV int nvshmem_##NAME##_test_all(TYPE *ivars, size_t nelems, const int *status,     \
                                                int cmp, TYPE cmp_value) {                         \
-        for (size_t i = 0; i < nelems; ++i)                                                       \
-            if ((!status || !status[i]) && !nvshmemi_test<TYPE>(ivars + i, cmp, cmp_value))       \
-                return 0;                                                                         \
-        return 1;                                                                                 \
+        return nvshmemi_test_all<TYPE, false>(ivars, nelems, status, cmp, &cmp_value);            \
+    }                                                                                             \
+    NVSHMEMI_DEV size_t nvshmem_##NAME##_test_any(TYPE *ivars, size_t nelems, const int *status,  \
+                                                  int cmp, TYPE cmp_value) {                      \
+        return nvshmemi_test_any<TYPE, false>(ivars, nelems, status, cmp, &cmp_value);            \
+    }                                                                                             \
+    NVSHMEMI_DEV size_t nvshmem_##NAME##_test_some(TYPE *ivars, size_t nelems, size_t *indices,   \
+                                                   const int *status, int cmp, TYPE cmp_value) {  \
+        return nvshmemi_test_some<TYPE, false>(ivars, nelems, indices, status, cmp, &cmp_value);  \
+    }                                                                                             \
+    NVSHMEMI_DEV int nvshmem_##NAME##_test_all_vector(TYPE *ivars, size_t nelems,                 \
+                                                      const int *status, int cmp,                 \
+                                                      TYPE *cmp_values) {                         \
+        return nvshmemi_test_all<TYPE, true>(ivars, nelems, status, cmp, cmp_values);             \
+    }                                                                                             \
+    NVSHMEMI_DEV size_t nvshmem_##NAME##_test_any_vector(TYPE *ivars, size_t nelems,              \
+                                                         const int *status, int cmp,              \
+                                                         TYPE *cmp_values) {                      \
+        return nvshmemi_test_any<TYPE, true>(ivars, nelems, status, cmp, cmp_values);             \
+    }                                                                                             \
+    NVSHMEMI_DEV size_t nvshmem_##NAME##_test_some_vector(TYPE *ivars, size_t nelems,             \
+                                                          size_t *indices, const int *status,     \
+                                                          int cmp, TYPE *cmp_values) {            \
+        return nvshmemi_test_some<TYPE, true>(ivars, nelems, indices, status, cmp, cmp_values);   \
     }
 NVSHMEMI_REPT_FOR_WAIT_TYPES(NVSHMEMI_STAMP_WAIT)
 #undef NVSHMEMI_STAMP_WAIT

@@ -435,6 +435,78 @@ NVSHMEMI_DEVICE_INLINE int nvshmemi_test(T *ivar, int cmp, T value) {
 }
 
 /* ------------------------------------------------------------------------------------------------
+ * Waits and tests over sets of variables (reference src/include/device/nvshmem_defines.h:446-735).
+ * status[i] != 0 takes ivars[i] out of the set; `values` is one comparison value (VECTOR false)
+ * or one per variable.  The "any" forms return an index that satisfies the comparison, or SIZE_MAX
+ * for an empty set; the "some" forms store the satisfied indices and return their number, at least
+ * one unless the set is empty.  The reference starts its "any" scans at a rotating index; here a
+ * scan starts at 0, which returns a member of the same set of valid answers.  A wait that exceeds
+ * the spin limit is recorded like in nvshmemi_wait_until and returns SIZE_MAX / 0.
+ * ---------------------------------------------------------------------------------------------- */
+template <typename T, bool VECTOR>
+NVSHMEMI_DEVICE_INLINE T nvshmemi_amd_cmp_value(const T *values, size_t i) {
+    return VECTOR ? values[i] : values[0];
+}
+template <typename T, bool VECTOR>
+NVSHMEMI_DEVICE_INLINE void nvshmemi_wait_until_all(T *ivars, size_t nelems, const int *status, int cmp,
+                                                    const T *values) {
+    for (size_t i = 0; i < nelems; ++i)
+        if (!status || !status[i]) nvshmemi_wait_until<T>(ivars + i, cmp, nvshmemi_amd_cmp_value<T, VECTOR>(values, i));
+}
+template <typename T, bool VECTOR>
+NVSHMEMI_DEVICE_INLINE int nvshmemi_test_all(T *ivars, size_t nelems, const int *status, int cmp,
+                                             const T *values) {
+    for (size_t i = 0; i < nelems; ++i)
+        if ((!status || !status[i]) && !nvshmemi_test<T>(ivars + i, cmp, nvshmemi_amd_cmp_value<T, VECTOR>(values, i)))
+            return 0;
+    return 1;
+}
+template <typename T, bool VECTOR>
+NVSHMEMI_DEVICE_INLINE size_t nvshmemi_test_any(T *ivars, size_t nelems, const int *status, int cmp,
+                                                const T *values) {
+    for (size_t i = 0; i < nelems; ++i)
+        if ((!status || !status[i]) && nvshmemi_test<T>(ivars + i, cmp, nvshmemi_amd_cmp_value<T, VECTOR>(values, i)))
+            return i;
+    return SIZE_MAX;
+}
+template <typename T, bool VECTOR>
+NVSHMEMI_DEVICE_INLINE size_t nvshmemi_test_some(T *ivars, size_t nelems, size_t *indices, const int *status,
+                                                 int cmp, const T *values) {
+    size_t found = 0;
+    for (size_t i = 0; i < nelems; ++i)
+        if ((!status || !status[i]) && nvshmemi_test<T>(ivars + i, cmp, nvshmemi_amd_cmp_value<T, VECTOR>(values, i)))
+            indices[found++] = i;
+    return found;
+}
+template <typename T, bool VECTOR>
+NVSHMEMI_DEVICE_INLINE size_t nvshmemi_wait_until_any(T *ivars, size_t nelems, const int *status, int cmp,
+                                                      const T *values) {
+    bool empty = true;
+    for (size_t i = 0; i < nelems && empty; ++i) empty = status && status[i];
+    if (empty) return SIZE_MAX;
+    const uint64_t limit = nvshmemi_device_state_d.spin_limit;
+    for (uint64_t sweeps = 0;; ++sweeps) {
+        const size_t hit = nvshmemi_test_any<T, VECTOR>(ivars, nelems, status, cmp, values);
+        if (hit != SIZE_MAX) return hit;
+        if (limit && sweeps >= limit) {
+            nvshmemi_amd_record_timeout(ivars, 0, (uint64_t)values[0]);
+            return SIZE_MAX;
+        }
+        __builtin_amdgcn_s_sleep(1);
+    }
+}
+template <typename T, bool VECTOR>
+NVSHMEMI_DEVICE_INLINE size_t nvshmemi_wait_until_some(T *ivars, size_t nelems, size_t *indices,
+                                                       const int *status, int cmp, const T *values) {
+    size_t found = nvshmemi_test_some<T, VECTOR>(ivars, nelems, indices, status, cmp, values);
+    if (found) return found;
+    const size_t hit = nvshmemi_wait_until_any<T, VECTOR>(ivars, nelems, status, cmp, values);
+    if (hit == SIZE_MAX) return 0;
+    indices[0] = hit;
+    return 1;
+}
+
+/* ------------------------------------------------------------------------------------------------
  * Atomic memory operations (reference src/include/device/nvshmem_defines.h:742-1236, whose
  * load/store branch applies atomic*_system to the translated address).  Here: relaxed agent-scope
  * atomics on the target PE's copy; every operation works at the full width of its type (the

@@ -69,6 +69,36 @@ __global__ void api_matrix_kernel(char *a, char *b, uint64_t *sig, int *ints, in
         my_out[8] = nvshmem_int_test(ints + 3, NVSHMEM_CMP_LT, 5);
         my_out[9] = nvshmem_int_test_all(ints, 4, skip, NVSHMEM_CMP_NE, 0);
         nvshmem_int_wait_until(ints + 1, NVSHMEM_CMP_EQ, 101);
+        // set forms: ints[0..4) now hold 100..103; the left neighbour also sets ints[5] = 77
+        nvshmem_int_p(ints + 5, 77, peer);
+        {
+            int *mine = (int *)nvshmem_ptr(ints, me);
+            size_t idx[8];
+            const int skip2[8] = {0, 0, 1, 0, 0, 0, 0, 0};
+            const int all_skipped[4] = {1, 1, 1, 1};
+            int exact[4] = {100, 101, 102, 103}, wrong[4] = {100, 101, 0, 103}, below[4] = {100, 101, 101, 103};
+            unsigned ok = 0;
+            ok |= (nvshmem_int_test_any(mine, 4, nullptr, NVSHMEM_CMP_EQ, 102) == 2) << 0;
+            ok |= (nvshmem_int_test_any(mine, 4, skip2, NVSHMEM_CMP_GE, 102) == 3) << 1;
+            ok |= (nvshmem_int_test_any(mine, 4, nullptr, NVSHMEM_CMP_GT, 1000) == SIZE_MAX) << 2;
+            ok |= (nvshmem_int_test_some(mine, 4, idx, nullptr, NVSHMEM_CMP_GE, 101) == 3 && idx[0] == 1 &&
+                   idx[1] == 2 && idx[2] == 3) << 3;
+            ok |= (nvshmem_int_test_some(mine, 4, idx, skip2, NVSHMEM_CMP_LT, 100) == 0) << 4;
+            ok |= (nvshmem_int_test_all_vector(mine, 4, nullptr, NVSHMEM_CMP_EQ, exact) == 1) << 5;
+            ok |= (nvshmem_int_test_all_vector(mine, 4, nullptr, NVSHMEM_CMP_EQ, wrong) == 0) << 6;
+            ok |= (nvshmem_int_test_all_vector(mine, 4, skip2, NVSHMEM_CMP_EQ, wrong) == 1) << 7;
+            ok |= (nvshmem_int_test_any_vector(mine, 4, nullptr, NVSHMEM_CMP_GT, below) == 2) << 8;
+            ok |= (nvshmem_int_test_some_vector(mine, 4, idx, nullptr, NVSHMEM_CMP_NE, wrong) == 1 && idx[0] == 2) << 9;
+            // waits on ints[4..8): only ints[5] ever changes
+            ok |= (nvshmem_int_wait_until_any(mine + 4, 4, nullptr, NVSHMEM_CMP_NE, 0) == 1) << 10;
+            ok |= (nvshmem_int_wait_until_some(mine + 4, 4, idx, nullptr, NVSHMEM_CMP_EQ, 77) == 1 && idx[0] == 1) << 11;
+            ok |= (nvshmem_int_wait_until_any(mine, 4, all_skipped, NVSHMEM_CMP_EQ, 5) == SIZE_MAX) << 12;
+            nvshmem_int_wait_until_all_vector(mine, 4, nullptr, NVSHMEM_CMP_EQ, exact);
+            ok |= (nvshmem_int_wait_until_any_vector(mine, 4, nullptr, NVSHMEM_CMP_GT, below) == 2) << 13;
+            ok |= (nvshmem_int_wait_until_some_vector(mine, 4, idx, nullptr, NVSHMEM_CMP_GE, exact) == 4 && idx[3] == 3) << 14;
+            ok |= (nvshmem_uint64_test_any(sig, 2, nullptr, NVSHMEM_CMP_EQ, 11) == 1) << 15;
+            my_out[13] = ok;
+        }
         nvshmem_quiet();
         nvshmem_fence();
         my_out[10] = me * 1000 + np;

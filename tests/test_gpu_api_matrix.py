@@ -72,5 +72,8 @@ def test_api_matrix():
             assert (o[7], o[8], o[9]) == (1, 0, 1)                       # test EQ 103 / LT 5 / all NE 0
             assert o[10] == me * 1000 + NPES and o[11] == me * 100 + NPES
             assert o[12] == 15
+            # the set forms of wait / test (any, some, _vector): one bit per check, all must hold
+            assert o[13] == 0xFFFF, "set wait/test checks failed: %s" % bin(int(o[13]))
+            assert INTS[me, 5] == 77
             assert SIG[me, 0] == 7 and SIG[me, 1] == 11
             assert list(INTS[me, :4]) == [100, 101, 102, 103]
