@@ -35,6 +35,18 @@ typedef void *nvshmemx_stream_t; /* hipStream_t */
 NVSHMEMI_HOST_ONLY void nvshmem_init(void);           /* nvshmem_api.h:52-58 */
 NVSHMEMI_HOST_ONLY void nvshmem_finalize(void);       /* nvshmem_api.h:66 */
 NVSHMEMI_HOST_ONLY int nvshmemx_init_status(void);    /* nvshmem_api.h:50 */
+/* nvshmem_init with a thread level (nvshmem_api.h:60-67); `provided` is NVSHMEM_THREAD_SERIALIZED
+ * whatever was requested, as in the reference (src/host/init/init.cu:1294,1309).  Returns 0. */
+NVSHMEMI_HOST_ONLY int nvshmem_init_thread(int requested, int *provided);
+NVSHMEMI_HOST_ONLY void nvshmem_query_thread(int *provided);   /* nvshmem_api.h:69 */
+/* Ends the program with `status` after finalizing (nvshmem_api.h:70). */
+NVSHMEMI_HOST_ONLY void nvshmem_global_exit(int status);
+/* Registration of local buffers used as put sources / get destinations
+ * (src/include/host/nvshmemx_api.h:47-49): every device allocation of the one GPU is reachable by
+ * load/store already, so these only validate their arguments and return 0. */
+NVSHMEMI_HOST_ONLY int nvshmemx_buffer_register(void *addr, size_t length);
+NVSHMEMI_HOST_ONLY int nvshmemx_buffer_unregister(void *addr);
+NVSHMEMI_HOST_ONLY void nvshmemx_buffer_unregister_all(void);
 NVSHMEMI_HOST_ONLY int nvshmem_my_pe(void);           /* nvshmem_api.h:60-64 */
 NVSHMEMI_HOST_ONLY int nvshmem_n_pes(void);
 /* ---- teams: src/include/host/nvshmem_api.h:465-482, src/host/team/team.cu:19-115 ----

@@ -42,6 +42,10 @@ def load():
         "nvshmemx_init_status": (i32, []),
         "nvshmem_my_pe": (i32, []),
         "nvshmem_n_pes": (i32, []),
+        "nvshmem_init_thread": (i32, [i32, C.POINTER(i32)]),
+        "nvshmem_query_thread": (None, [C.POINTER(i32)]),
+        "nvshmemx_buffer_register": (i32, [vp, sz]),
+        "nvshmemx_buffer_unregister": (i32, [vp]),
         "nvshmem_team_my_pe": (i32, [i32]),
         "nvshmem_team_n_pes": (i32, [i32]),
         "nvshmem_info_get_version": (None, [C.POINTER(i32), C.POINTER(i32)]),
@@ -68,6 +72,10 @@ def load():
         "nvshmem_fcollectmem": (i32, [i32, vp, vp, sz]),
         "nvshmemx_alltoallmem_on_stream": (i32, [i32, vp, vp, sz, vp]),
         "nvshmemx_fcollectmem_on_stream": (i32, [i32, vp, vp, sz, vp]),
+        "nvshmem_init_thread": (i32, [i32, C.POINTER(i32)]),
+        "nvshmem_query_thread": (None, [C.POINTER(i32)]),
+        "nvshmemx_buffer_register": (i32, [vp, sz]),
+        "nvshmemx_buffer_unregister": (i32, [vp]),
         "nvshmem_team_my_pe": (i32, [i32]),
         "nvshmem_team_n_pes": (i32, [i32]),
         "nvshmem_team_translate_pe": (i32, [i32, i32, i32]),

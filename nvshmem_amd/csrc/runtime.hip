@@ -240,6 +240,29 @@ int nvshmemx_init_status(void) {
                                       : NVSHMEM_STATUS_NOT_INITIALIZED;
 }
 
+int nvshmem_init_thread(int requested, int *provided) {
+    (void)requested;
+    nvshmem_init();
+    if (provided) *provided = NVSHMEM_THREAD_SERIALIZED;
+    return 0;
+}
+void nvshmem_query_thread(int *provided) {
+    if (provided) *provided = NVSHMEM_THREAD_SERIALIZED;
+}
+void nvshmem_global_exit(int status) {
+    nvshmem_finalize();
+    exit(status);
+}
+int nvshmemx_buffer_register(void *addr, size_t length) {
+    if (!addr || length == 0) {
+        set_error("nvshmemx_buffer_register: null buffer or zero length");
+        return NVSHMEMX_ERROR_INVALID_VALUE;
+    }
+    return 0;
+}
+int nvshmemx_buffer_unregister(void *addr) { return addr ? 0 : NVSHMEMX_ERROR_INVALID_VALUE; }
+void nvshmemx_buffer_unregister_all(void) {}
+
 int nvshmem_my_pe(void) { return 0; }
 int nvshmem_n_pes(void) { return Runtime::get().npes; }
 void nvshmem_info_get_version(int *major, int *minor) {

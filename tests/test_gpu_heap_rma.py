@@ -29,6 +29,17 @@ def test_identity_and_versions(rt):
     assert rt.lib.nvshmem_team_n_pes(N.TEAM_WORLD) == NPES
     assert rt.lib.nvshmemx_init_status() == 2      # NVSHMEM_STATUS_IS_INITIALIZED
     assert rt.lib.nvshmemx_amd_init(4, 1 << 20) != 0   # second init is refused
+    import ctypes as C
+    provided = C.c_int32(-1)
+    assert rt.lib.nvshmem_init_thread(3, C.byref(provided)) == 0 and provided.value == 2   # SERIALIZED
+    assert rt.lib.nvshmem_n_pes() == NPES              # init on a live runtime changes nothing
+    provided.value = -1
+    rt.lib.nvshmem_query_thread(C.byref(provided))
+    assert provided.value == 2
+    buf = rt.malloc(64)
+    assert rt.lib.nvshmemx_buffer_register(buf, 64) == 0 and rt.lib.nvshmemx_buffer_unregister(buf) == 0
+    assert rt.lib.nvshmemx_buffer_register(None, 64) != 0
+    rt.free(buf)
 
 
 def test_malloc_ptr_translation_matches_closed_form(rt):
