@@ -825,12 +825,13 @@ NVSHMEMI_DEVICE_INLINE uint64_t nvshmemi_amd_ll_recv_packet(const char *packet, 
     }
     return (uint64_t)v.x | ((uint64_t)v.z << 32);
 }
-/* Sends the npk chunks of src to the other members of the team, chunk j into slot slot0 + j of
- * their buffers; the (member, chunk) pairs are spread over the lanes. */
+/* Sends npk chunks to each other member of the team, chunk j into slot slot0 + j of its buffers:
+ * the chunks of src for everybody (dest_stride 0), or those of src + idx * dest_stride for member
+ * idx.  The (member, chunk) pairs are spread over the lanes. */
 template <int SCOPE>
 NVSHMEMI_DEVICE_INLINE void nvshmemi_amd_ll_send_to_all(nvshmem_team_t team, const nvshmemi_amd_team_view_t &tv,
                                                         const char *src, size_t nbytes, unsigned npk,
-                                                        unsigned slot0, uint32_t flag) {
+                                                        unsigned slot0, uint32_t flag, size_t dest_stride = 0) {
     const unsigned nthr = (unsigned)nvshmemi_threadgroup_size<SCOPE>();
     const unsigned total = (unsigned)(tv.size - 1) * npk;
     for (unsigned w = (unsigned)nvshmemi_thread_id_in_threadgroup<SCOPE>(); w < total; w += nthr) {
@@ -839,7 +840,8 @@ NVSHMEMI_DEVICE_INLINE void nvshmemi_amd_ll_send_to_all(nvshmem_team_t team, con
         if (idx >= tv.size) idx -= tv.size;
         nvshmemi_amd_ll_store_packet(
             nvshmemi_amd_ll_buffer(team, nvshmemi_amd_team_pe(tv, idx), flag) + (size_t)(slot0 + j) * 16,
-            nvshmemi_amd_ll_load_payload(src + 8 * (size_t)j, nbytes - 8 * (size_t)j), flag);
+            nvshmemi_amd_ll_load_payload(src + (size_t)idx * dest_stride + 8 * (size_t)j, nbytes - 8 * (size_t)j),
+            flag);
     }
 }
 /* Tells the other PEs that this PE has read everything of call `flag`. */
@@ -864,7 +866,7 @@ NVSHMEMI_DEVICE_INLINE bool nvshmemi_amd_ll_fits(size_t nbytes, int size) {
  * member p) fetches one packet (its own source for p == me), then the lanes of a chunk - adjacent,
  * in a group of G = npes rounded up to a power of two - pass their values to each other with
  * cross-lane reads and the first lane of the group stores the result. */
-template <typename T, int OP, int SCOPE>
+template <typename T, int OP, int SCOPE, bool SCATTER = false>
 NVSHMEMI_DEVICE_INLINE void nvshmemi_amd_ll_reduce(nvshmem_team_t team, const nvshmemi_amd_team_view_t &tv,
                                                    T *dest, const T *source, size_t nreduce, unsigned group) {
     constexpr size_t PER = 8 / sizeof(T);
@@ -873,9 +875,13 @@ NVSHMEMI_DEVICE_INLINE void nvshmemi_amd_ll_reduce(nvshmem_team_t team, const nv
     const size_t nbytes = nreduce * sizeof(T);
     const uint32_t flag = nvshmemi_amd_ll_next_flag<SCOPE>(team);
     const unsigned npk = nvshmemi_amd_ll_packets(nbytes);
-    const char *src = nvshmemi_amd_local(source);
+    /* reducescatter (SCATTER): member idx is sent block idx of the source and folds the blocks
+     * `me` it receives, with the operands in reducescatter's order */
+    const char *src_all = nvshmemi_amd_local(source);
+    const char *src = src_all + (SCATTER ? (size_t)me * nbytes : 0);
     char *dst = nvshmemi_amd_local(dest);
-    nvshmemi_amd_ll_send_to_all<SCOPE>(team, tv, src, nbytes, npk, (unsigned)me * npk, flag);
+    nvshmemi_amd_ll_send_to_all<SCOPE>(team, tv, src_all, nbytes, npk, (unsigned)me * npk, flag,
+                                       SCATTER ? nbytes : 0);
     /* dest may be source: everything is sent before any result is stored */
     nvshmemi_threadgroup_sync<SCOPE>();
     const char *mine = nvshmemi_amd_ll_buffer(team, nvshmemi_amd_my_pe(), flag);
@@ -888,7 +894,10 @@ NVSHMEMI_DEVICE_INLINE void nvshmemi_amd_ll_reduce(nvshmem_team_t team, const nv
                 T x[PER];
                 __builtin_memcpy(x, &v, 8);
 #pragma unroll
-                for (size_t k = 0; k < PER; ++k) acc[k] = p == 0 ? x[k] : nvshmemi_amd_fold_step<T, OP>(p, acc[k], x[k]);
+                for (size_t k = 0; k < PER; ++k)
+                    acc[k] = p == 0 ? x[k]
+                                    : SCATTER ? nvshmemi_amd_reduce_op<T, OP>(acc[k], x[k])
+                                              : nvshmemi_amd_fold_step<T, OP>(p, acc[k], x[k]);
             }
             uint64_t r;
             __builtin_memcpy(&r, acc, 8);
@@ -912,7 +921,10 @@ NVSHMEMI_DEVICE_INLINE void nvshmemi_amd_ll_reduce(nvshmem_team_t team, const nv
                 T x[PER];
                 __builtin_memcpy(x, &xv, 8);
 #pragma unroll
-                for (size_t k = 0; k < PER; ++k) acc[k] = q == 0 ? x[k] : nvshmemi_amd_fold_step<T, OP>(q, acc[k], x[k]);
+                for (size_t k = 0; k < PER; ++k)
+                    acc[k] = q == 0 ? x[k]
+                                    : SCATTER ? nvshmemi_amd_reduce_op<T, OP>(acc[k], x[k])
+                                              : nvshmemi_amd_fold_step<T, OP>(q, acc[k], x[k]);
             }
             if (p == 0 && j < npk) {
                 uint64_t r;
@@ -1052,6 +1064,29 @@ NVSHMEMI_DEVICE_INLINE int nvshmemi_alltoall_threadgroup(nvshmem_team_t team, T 
     if (tv.size <= 0) return 1;
     const int me = tv.my_pe;
     const int npes = tv.size;
+    const size_t nbytes = nelems * sizeof(T);
+    if (nvshmemi_amd_ll_fits<SCOPE>(nbytes, npes)) {
+        /* small blocks: like the fcollect packets, but member idx is sent block idx */
+        const unsigned tid = (unsigned)nvshmemi_thread_id_in_threadgroup<SCOPE>();
+        const unsigned nthr = (unsigned)nvshmemi_threadgroup_size<SCOPE>();
+        const uint32_t flag = nvshmemi_amd_ll_next_flag<SCOPE>(team);
+        const unsigned npk = nvshmemi_amd_ll_packets(nbytes);
+        const unsigned total = (unsigned)(npes - 1) * npk;
+        const char *src = nvshmemi_amd_local(source);
+        char *dst = nvshmemi_amd_local(dest);
+        nvshmemi_amd_ll_send_to_all<SCOPE>(team, tv, src, nbytes, npk, (unsigned)me * npk, flag, nbytes);
+        for (size_t b = tid; b < nbytes; b += nthr) dst[(size_t)me * nbytes + b] = src[(size_t)me * nbytes + b];
+        const char *mine = nvshmemi_amd_ll_buffer(team, nvshmemi_amd_my_pe(), flag);
+        for (unsigned w = tid; w < total; w += nthr) {
+            const unsigned off = w / npk, j = w - off * npk;
+            int idx = me + 1 + (int)off;
+            if (idx >= npes) idx -= npes;
+            const uint64_t v = nvshmemi_amd_ll_recv_packet(mine + ((size_t)idx * npk + j) * 16, flag);
+            nvshmemi_amd_ll_store_payload(dst + (size_t)idx * nbytes + 8 * (size_t)j, v, nbytes - 8 * (size_t)j);
+        }
+        nvshmemi_amd_ll_publish_done<SCOPE>(team, flag);
+        return 0;
+    }
     nvshmemi_threadgroup_sync<SCOPE>();
     for (int ii = 0; ii < npes; ++ii) {
         const int idx = (me + ii) % npes;
@@ -1133,6 +1168,10 @@ NVSHMEMI_DEVICE_INLINE int nvshmemi_reducescatter_threadgroup(nvshmem_team_t tea
     const int npes = tv.size;
     const size_t tid = (size_t)nvshmemi_thread_id_in_threadgroup<SCOPE>();
     const size_t nthr = (size_t)nvshmemi_threadgroup_size<SCOPE>();
+    if (const unsigned group = nvshmemi_amd_ll_reduce_group<SCOPE>(nreduce * sizeof(T), npes)) {
+        nvshmemi_amd_ll_reduce<T, OP, SCOPE, true>(team, tv, dest, source, nreduce, group);
+        return 0;
+    }
     /* every PE's source is complete and visible before anyone reads it */
     nvshmemi_barrier_threadgroup<SCOPE>(team);
     const T *src0 = reinterpret_cast<const T *>(nvshmemi_amd_remote(source, tv.start)) + (size_t)me * nreduce;

@@ -112,11 +112,13 @@ int nvshmem_perftest_amo_matrix(uint64_t *slots, const uint64_t *val, const uint
 int nvshmem_perftest_amo_contend(uint64_t *words, unsigned int *seen, unsigned long long *chain,
                                  int home, int blocks, int threads, void *stream);
 /* `rounds` rounds of {int32 sum reduce of n elements, broadcast of those n elements from PE
- * r % npes, fcollect of fc_bytes (a multiple of 4, at most 4n) per PE} back to back inside one
+ * r % npes, fcollect of fc_bytes (a multiple of 4, at most 4n) per PE, and when n >= npes an
+ * alltoall and an int32 sum reducescatter of n / npes words per member} back to back inside one
  * kernel, all on NVSHMEM_TEAM_WORLD into dst, with no barrier in between unless sync_between is
  * set.  Round r sends src[i] = (me*1000003 + r*7919 + i*31) & 0x7fffffff.  After every collective
  * each PE folds dst into its check[0]: h = h*1000003 + sum_i (uint32)dst[i] * (2i+1) (mod 2^64),
- * over the n (reduce, broadcast) or fc_bytes*npes/4 (fcollect) words the call produced. */
+ * over the n (reduce, broadcast), fc_bytes*npes/4 (fcollect), (n/npes)*npes (alltoall) or n/npes
+ * (reducescatter) words the call produced. */
 int nvshmem_perftest_coll_sequence(int32_t *src, int32_t *dst, uint64_t *check, int n, int fc_bytes,
                                    int rounds, int sync_between, int scope, int threads, void *stream);
 /* In-kernel collectives on a team handle (members only; the other PEs return at once).  what:

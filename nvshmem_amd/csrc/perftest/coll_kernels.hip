@@ -135,8 +135,9 @@ __global__ void team_barrier_kernel(uint64_t *counter, uint64_t *errors, int rou
 
 // Many collectives back to back without any barrier in between (sync_between = 0) or with one
 // after every check (1): round r fills src[i] = gen(me, r, i), then runs an int32 sum reduce of n
-// elements, a broadcast of the same n elements from member r % npes and an fcollect of fc_bytes per
-// PE, all into dst, and folds a position-weighted checksum of dst into check[0] after each.
+// elements, a broadcast of the same n elements from member r % npes, an fcollect of fc_bytes per
+// PE, and - when n >= npes - an alltoall and a reducescatter of n / npes words per member, all into
+// dst, and folds a position-weighted checksum of dst into check[0] after each.
 __device__ inline int32_t ll_gen(int me, int r, int i) {
     return (int32_t)(((uint32_t)me * 1000003u + (uint32_t)r * 7919u + (uint32_t)i * 31u) & 0x7fffffffu);
 }
@@ -170,6 +171,21 @@ __global__ void coll_sequence_kernel(int32_t *src, int32_t *dst, uint64_t *check
         if (threadIdx.x == 0) h = ll_checksum(h, my_dst, (size_t)fc_bytes * np / 4);
         __syncthreads();
         if (sync_between) SCOPED_CALL(SCOPE, barrier_all);
+        // alltoall of a2a_words per destination and reducescatter of the same count, both out of
+        // the first np * a2a_words words of src
+        const size_t a2a_words = (size_t)n / (size_t)np;
+        if (a2a_words) {
+            SCOPED_CALL(SCOPE, alltoallmem, NVSHMEM_TEAM_WORLD, dst, src, a2a_words * 4);
+            __syncthreads();
+            if (threadIdx.x == 0) h = ll_checksum(h, my_dst, a2a_words * np);
+            __syncthreads();
+            if (sync_between) SCOPED_CALL(SCOPE, barrier_all);
+            SCOPED_CALL(SCOPE, int32_sum_reducescatter, NVSHMEM_TEAM_WORLD, dst, src, a2a_words);
+            __syncthreads();
+            if (threadIdx.x == 0) h = ll_checksum(h, my_dst, a2a_words);
+            __syncthreads();
+            if (sync_between) SCOPED_CALL(SCOPE, barrier_all);
+        }
     }
     if (threadIdx.x == 0) *(uint64_t *)nvshmem_ptr(check, me) = h;
 }

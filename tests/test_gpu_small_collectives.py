@@ -39,10 +39,18 @@ def _expected_checks(npes, n, fc_bytes, rounds):
         red = O.reduce("i32", "sum", data)
         bc = data[r % npes]
         fc = O.fcollect(data.view(np.uint8)[:, :fc_bytes])
+        w = n // npes
+        if w:
+            block = np.ascontiguousarray(data[:, :w * npes])
+            a2a = O.alltoall(block.view(np.uint8)).view(np.int32)
+            rs = O.reducescatter("i32", "sum", block)
         for pe in range(npes):
             h[pe] = _checksum(h[pe], red)
             h[pe] = _checksum(h[pe], bc)
             h[pe] = _checksum(h[pe], fc[pe].view(np.int32))
+            if w:
+                h[pe] = _checksum(h[pe], a2a[pe])
+                h[pe] = _checksum(h[pe], rs[pe])
     return h
 
 
@@ -55,7 +63,7 @@ def _uses_packets(what, nbytes, npes, scope, threads):
     if what == "broadcast":
         return nbytes <= 16384 and npk * (npes - 1 if scope == N.SCOPE_THREAD else 1) <= lanes
     ok = nbytes <= 2048 and npk * 8 * npes <= 16384 and npk * (npes - 1) <= lanes
-    if what == "reduce" and scope != N.SCOPE_THREAD:
+    if what in ("reduce", "reducescatter") and scope != N.SCOPE_THREAD:
         group = 1
         while group < npes:
             group *= 2
@@ -76,7 +84,8 @@ def test_unsynchronised_sequences(rt8, scope, threads, n, fc_bytes, sync_between
     # a broadcast or fcollect that does not travel as packets writes into the other PEs' dst at
     # once, so - as in any NVSHMEM program - the PEs must have finished with dst before it starts
     if not (_uses_packets("broadcast", n * 4, 8, scope, threads) and
-            _uses_packets("fcollect", fc_bytes, 8, scope, threads)):
+            _uses_packets("fcollect", fc_bytes, 8, scope, threads) and
+            (n < 8 or _uses_packets("alltoall", (n // 8) * 4, 8, scope, threads))):
         sync_between = 1
     rounds = 6 if scope == N.SCOPE_THREAD and n > 1000 else 40
     src = rt8.malloc(5000 * 4); dst = rt8.malloc(8 * 2052 + 5000 * 4); check = rt8.calloc(1, 8)
@@ -124,6 +133,25 @@ def test_sizes_around_the_switch_over(rt8, scope, threads):
                                                        threads, None) == 0
             rt8.sync()
             assert bits_equal(rt8.download(src, 3, (n,), data.dtype), O.reduce(kind, op, data))
+    for kind, op, es in (("i32", "sum", 4), ("f32", "max", 4), ("bf16", "sum", 2), ("u64", "xor", 8)):
+        for nbytes in (es, 3 * es, 64, 256, 256 + es, 2048):
+            n = nbytes // es
+            if kind == "f32":
+                data = rng.standard_normal((8, 8 * n)).astype(np.float32)
+                data[rng.random(data.shape) < 0.1] = np.nan
+            elif kind == "bf16":
+                data = (rng.standard_normal((8, 8 * n)).astype(np.float32).view(np.uint32) >> 16).astype(np.uint16)
+            else:
+                info = np.iinfo(O.NP_STORAGE[kind])
+                data = rng.integers(info.min, info.max, (8, 8 * n), dtype=O.NP_STORAGE[kind], endpoint=True)
+            for off in (0, es):
+                rt8.upload_all(src, data, off)
+                note("device reducescatter %s %s n=%d off=%d scope=%d" % (kind, op, n, off, scope))
+                assert perf.nvshmem_perftest_device_reducescatter(N.DTYPES[kind], N.OPS[op], dst + off, src + off,
+                                                                  n, scope, threads, None) == 0
+                rt8.sync()
+                assert bits_equal(rt8.download_all(dst, (n,), data.dtype, off), O.reducescatter(kind, op, data)), \
+                    (kind, op, n, off)
     for nbytes in (1, 7, 8, 9, 63, 72, 73, 288, 289, 511, 512, 513, 2047, 2048, 2049, 16384, 16385):
         for soff, doff in ((0, 0), (3, 5)):
             data = rng.integers(0, 256, (8, nbytes), dtype=np.uint8)
@@ -135,6 +163,16 @@ def test_sizes_around_the_switch_over(rt8, scope, threads):
             got = rt8.download_all(dst, (8 * nbytes + 16,), np.uint8)
             assert np.array_equal(got[:, doff:doff + 8 * nbytes], O.fcollect(data))
             assert (got[:, :doff] == 0xCD).all() and (got[:, doff + 8 * nbytes:] == 0xCD).all()
+            if 8 * nbytes + soff <= (1 << 16):
+                data8 = rng.integers(0, 256, (8, 8 * nbytes), dtype=np.uint8)
+                rt8.fill(dst, 0xCD, 1 << 18)
+                rt8.upload_all(src, data8, soff)
+                assert perf.nvshmem_perftest_device_alltoall(dst + doff, src + soff, nbytes, scope, threads, None) == 0
+                rt8.sync()
+                got = rt8.download_all(dst, (8 * nbytes + 16,), np.uint8)
+                assert np.array_equal(got[:, doff:doff + 8 * nbytes], O.alltoall(data8))
+                assert (got[:, :doff] == 0xCD).all() and (got[:, doff + 8 * nbytes:] == 0xCD).all()
+                rt8.upload_all(src, data, soff)
             rt8.fill(dst, 0xCD, 1 << 18)
             assert perf.nvshmem_perftest_device_broadcast(dst + doff, src + soff, nbytes, 6, scope, threads, None) == 0
             rt8.sync()
