@@ -43,3 +43,35 @@ def test_graph_replays_match_eager_results():
             rt.reduce("float", "max", red, src, n)
             assert bits_equal(rt.download(red, 3, (n,), np.float32), O.reduce("f32", "max", f))
         g.destroy(); s.destroy()
+
+
+def test_graph_with_team_collectives_broadcast_and_reducescatter():
+    npes, n = 8, 4100
+    rng = np.random.default_rng(18)
+    with runtime(npes, 16 << 20) as rt:
+        src = rt.malloc(npes * n * 4); rs = rt.malloc(n * 4); bc = rt.malloc(n * 4); row = rt.malloc(n * 4)
+        x, y = rt.team_split_2d(0, 4)          # rows {0..3}, {4..7}; columns {p, p+4}
+        s = hip.Stream()
+        note("capturing reducescatter + broadcast + a reduce on every row of a 2-D split")
+        with hip.Graph(s) as g:
+            rt.reducescatter("float", "sum", rs, src, n, stream=s)
+            rt.broadcastmem(bc, src, n * 4, 5, stream=s)
+            rt.reduce("float", "sum", row, src, n, stream=s, team=x)
+        for replay in range(3):
+            f = rng.standard_normal((npes, npes * n)).astype(np.float32)
+            rt.upload_all(src, f)
+            for p in (rs, bc, row):
+                rt.fill(p, 0xFF, n * 4)
+            note("graph replay %d" % replay)
+            g.launch()
+            s.synchronize()
+            assert bits_equal(rt.download_all(rs, (n,), np.float32), O.reducescatter("f32", "sum", f))
+            got = rt.download_all(bc, (n,), np.float32)
+            assert all(bits_equal(got[pe], f[5, :n]) for pe in range(npes))
+            got = rt.download_all(row, (n,), np.float32)
+            for lo in (0, 4):
+                want = O.reduce("f32", "sum", f[lo:lo + 4, :n])
+                assert all(bits_equal(got[pe], want) for pe in range(lo, lo + 4))
+            rt.fcollectmem(src, bc, 64, team=y)     # eager work between replays
+        g.destroy(); s.destroy()
+        rt.team_destroy(x); rt.team_destroy(y)
