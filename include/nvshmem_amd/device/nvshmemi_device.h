@@ -749,6 +749,10 @@ NVSHMEMI_DEVICE_INLINE T nvshmemi_amd_fold_step(int i, T acc, T x) {
  * An agent-scope access costs about a memory round trip per instruction, whether one lane is active
  * or 64, so the packets of a call are spread over the lanes - one per lane - and the path is only
  * taken while that is possible; longer messages are faster through the copy engine and a barrier.
+ * The choice depends on the message size and on the size of the calling thread group, so all
+ * members of a team must make a collective call with the same scope and group size (they do when
+ * one launch carries all PEs).  The 32-bit flags and `done` counters are compared as plain
+ * integers: the protocol assumes fewer than 2^32 packet calls per team handle life.
  * ---------------------------------------------------------------------------------------------- */
 NVSHMEMI_DEVICE_INLINE char *nvshmemi_amd_ll_buffer(nvshmem_team_t team, int pe, uint32_t flag) {
     const size_t buf = 2 * (size_t)NVSHMEMI_AMD_LL_PAYLOAD_BYTES;
