@@ -100,3 +100,40 @@ def test_broadcast_and_reducescatter_on_other_team_sizes(npes):
         want = idata.view(np.uint8)[root, 3:3 + n * 4 - 7]
         assert all(np.array_equal(got[pe], want) for pe in range(npes))
         rt.free(src); rt.free(dst)
+
+
+@pytest.mark.parametrize("disable", ["1", "0"])
+def test_small_in_kernel_collectives_with_and_without_packets(disable, monkeypatch):
+    """NVSHMEM_AMD_DISABLE_LL=1 (read at init) sends every in-kernel collective through its copy and
+    barrier path; results are the same either way."""
+    monkeypatch.setenv("NVSHMEM_AMD_DISABLE_LL", disable)
+    rng = np.random.default_rng(int(disable))
+    with runtime(8, 1 << 22) as rt:
+        perf = rt.perftest()
+        n = 16
+        src = rt.malloc(8 * n * 4); dst = rt.malloc(8 * n * 4)
+        for rep in range(5):
+            data = rng.standard_normal((8, 8 * n)).astype(np.float32)
+            rt.upload_all(src, data)
+            note("packets disabled=%s rep=%d" % (disable, rep))
+            assert perf.nvshmem_perftest_device_reduce(N.DTYPES["f32"], N.OPS["sum"], dst, src, n,
+                                                       N.SCOPE_BLOCK, 256, None) == 0
+            rt.sync()
+            want = O.reduce("f32", "sum", data[:, :n])
+            assert all(bits_equal(rt.download(dst, pe, (n,), np.float32), want) for pe in range(8))
+            assert perf.nvshmem_perftest_device_reducescatter(N.DTYPES["f32"], N.OPS["sum"], dst, src, n,
+                                                              N.SCOPE_WARP, 64, None) == 0
+            rt.sync()
+            assert bits_equal(rt.download_all(dst, (n,), np.float32), O.reducescatter("f32", "sum", data))
+            raw = data.view(np.uint8)
+            assert perf.nvshmem_perftest_device_alltoall(dst, src, n * 4, N.SCOPE_BLOCK, 128, None) == 0
+            rt.sync()
+            assert np.array_equal(rt.download_all(dst, (8 * n * 4,), np.uint8), O.alltoall(raw))
+            assert perf.nvshmem_perftest_device_fcollect(dst, src, n * 4, N.SCOPE_BLOCK, 128, None) == 0
+            rt.sync()
+            assert np.array_equal(rt.download_all(dst, (8 * n * 4,), np.uint8), O.fcollect(raw[:, :n * 4]))
+            assert perf.nvshmem_perftest_device_broadcast(dst, src, n * 4, rep % 8, N.SCOPE_THREAD, 64, None) == 0
+            rt.sync()
+            assert all(np.array_equal(rt.download(dst, pe, (n * 4,), np.uint8), raw[rep % 8, :n * 4]) for pe in range(8))
+        assert rt.read_timeout(0)[0] == 0
+        rt.free(src); rt.free(dst)
