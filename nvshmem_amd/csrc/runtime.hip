@@ -193,6 +193,7 @@ int nvshmemx_amd_init(int npes, size_t symmetric_size) {
     rt.dev.sync_epoch = (uint64_t *)(uintptr_t)epoch;
     rt.dev.timeout_record = (uint64_t *)(uintptr_t)trec;
     rt.dev.spin_limit = env_size("NVSHMEM_AMD_SPIN_LIMIT", 1ull << 22);
+    rt.plain_collective_launch = env_size("NVSHMEM_AMD_PLAIN_COLLECTIVE_LAUNCH", 0) != 0;
     if (!teams_init(rt)) {
         teams_finalize(rt);
         (void)hipFree(rt.base);
@@ -603,12 +604,21 @@ int nvshmemx_amd_collective_launch(const void *func, unsigned grid_x, unsigned g
                   per_pe, rt.npes, cap, threads);
         return NVSHMEMX_ERROR_COLLECTIVE_LAUNCH_FAILED;
     }
-    hipError_t e = hipLaunchCooperativeKernel(func, dim3(grid_x, grid_y, (unsigned)rt.npes),
-                                              dim3(block_x, block_y, block_z), args,
-                                              (unsigned)shared_mem, (hipStream_t)stream);
+    // A cooperative launch guarantees that all blocks are resident together, whatever else runs on
+    // the GPU, and costs about 20 us more than a plain launch here.  The grid has just been checked
+    // against the occupancy limit, so a plain launch gives the same co-residency as long as no
+    // other kernel holds compute units while waiting for this one: NVSHMEM_AMD_PLAIN_COLLECTIVE_
+    // LAUNCH=1 opts into that for programs that launch their PE kernels one at a time.
+    const dim3 grid(grid_x, grid_y, (unsigned)rt.npes), block(block_x, block_y, block_z);
+    hipError_t e = rt.plain_collective_launch
+                       ? hipLaunchKernel(func, grid, block, args, shared_mem, (hipStream_t)stream)
+                       : hipLaunchCooperativeKernel(func, grid, block, args, (unsigned)shared_mem,
+                                                    (hipStream_t)stream);
     if (e != hipSuccess) {
         (void)hipGetLastError();
-        set_error("collective launch: hipLaunchCooperativeKernel failed: %s", hipGetErrorString(e));
+        set_error("collective launch: %s failed: %s",
+                  rt.plain_collective_launch ? "hipLaunchKernel" : "hipLaunchCooperativeKernel",
+                  hipGetErrorString(e));
         return NVSHMEMX_ERROR_COLLECTIVE_LAUNCH_FAILED;
     }
     return NVSHMEMX_SUCCESS;

@@ -58,6 +58,7 @@ struct Runtime {
     TeamTable teams{};
     std::set<nvshmemi_amd_state_updater_t> updaters;  // one per translation unit with a state block
     bool symbols_stale = false;
+    bool plain_collective_launch = false;  // NVSHMEM_AMD_PLAIN_COLLECTIVE_LAUNCH=1, read at init
 
     static Runtime &get();
 

@@ -102,11 +102,13 @@ def test_broadcast_and_reducescatter_on_other_team_sizes(npes):
         rt.free(src); rt.free(dst)
 
 
-@pytest.mark.parametrize("disable", ["1", "0"])
-def test_small_in_kernel_collectives_with_and_without_packets(disable, monkeypatch):
+@pytest.mark.parametrize("disable,plain", [("1", "0"), ("0", "0"), ("0", "1")])
+def test_small_in_kernel_collectives_with_and_without_packets(disable, plain, monkeypatch):
     """NVSHMEM_AMD_DISABLE_LL=1 (read at init) sends every in-kernel collective through its copy and
-    barrier path; results are the same either way."""
+    barrier path; NVSHMEM_AMD_PLAIN_COLLECTIVE_LAUNCH=1 starts the PE kernels with an ordinary launch
+    after the occupancy check.  Results are the same every way."""
     monkeypatch.setenv("NVSHMEM_AMD_DISABLE_LL", disable)
+    monkeypatch.setenv("NVSHMEM_AMD_PLAIN_COLLECTIVE_LAUNCH", plain)
     rng = np.random.default_rng(int(disable))
     with runtime(8, 1 << 22) as rt:
         perf = rt.perftest()
