@@ -952,7 +952,8 @@ NVSHMEMI_DEVICE_INLINE unsigned nvshmemi_amd_ll_reduce_group(size_t nbytes, int 
 /* ------------------------------------------------------------------------------------------------
  * Collectives called from inside a user kernel, one thread group per PE
  * (reference coll/reduce.cuh:1158-1196 get-based reduce, coll/fcollect.cuh:331-344,
- * coll/alltoall.cuh:122-143).  Each ends with barrier semantics.
+ * coll/alltoall.cuh:122-143).  Calls small enough for the packets above return when the caller's
+ * own dest is complete; the others end with a barrier of the team.
  * ---------------------------------------------------------------------------------------------- */
 /* Reduce: PE `me` owns the element range [me*chunk, (me+1)*chunk): it folds that range from every
  * PE's source and stores the result into every PE's dest.  Each element is read by exactly one lane
