@@ -68,6 +68,32 @@ def test_collectives_and_rma_for_team_size(npes):
         assert perf.nvshmem_perftest_device_alltoall(dst, src, seg, N.SCOPE_WARP, 64, None) == 0
         rt.sync()
         assert np.array_equal(rt.download_all(dst, (npes * seg,), np.uint8), O.alltoall(data))
+        # the packet paths of the in-kernel collectives (a few bytes per member), twice each
+        for rep in range(2):
+            small = rng.integers(-2**20, 2**20, (npes, max(npes * 4, 8)), dtype=np.int32)
+            raw = small.view(np.uint8)
+            rt.upload_all(src, small)
+            note("npes=%d small in-kernel collectives rep=%d" % (npes, rep))
+            assert perf.nvshmem_perftest_device_reduce(N.DTYPES["i32"], N.OPS["sum"], dst, src, 4,
+                                                       N.SCOPE_BLOCK, 256, None) == 0
+            rt.sync()
+            want = O.reduce("i32", "sum", small[:, :4])
+            assert all(np.array_equal(rt.download(dst, pe, (4,), np.int32), want) for pe in range(npes))
+            assert perf.nvshmem_perftest_device_reducescatter(N.DTYPES["i32"], N.OPS["sum"], dst, src, 2,
+                                                              N.SCOPE_BLOCK, 256, None) == 0
+            rt.sync()
+            assert np.array_equal(rt.download_all(dst, (2,), np.int32),
+                                  O.reducescatter("i32", "sum", np.ascontiguousarray(small[:, :npes * 2])))
+            assert perf.nvshmem_perftest_device_fcollect(dst, src, 8, N.SCOPE_WARP, 64, None) == 0
+            rt.sync()
+            assert np.array_equal(rt.download_all(dst, (npes * 8,), np.uint8), O.fcollect(raw[:, :8]))
+            assert perf.nvshmem_perftest_device_alltoall(dst, src, 8, N.SCOPE_BLOCK, 512, None) == 0
+            rt.sync()
+            assert np.array_equal(rt.download_all(dst, (npes * 8,), np.uint8),
+                                  O.alltoall(np.ascontiguousarray(raw[:, :npes * 8])))
+            assert perf.nvshmem_perftest_device_broadcast(dst, src, 21, npes - 1, N.SCOPE_THREAD, 64, None) == 0
+            rt.sync()
+            assert all(np.array_equal(rt.download(dst, pe, (21,), np.uint8), raw[npes - 1, :21]) for pe in range(npes))
         assert all(rt.read_timeout(pe)[0] == 0 for pe in range(npes))
 
 
