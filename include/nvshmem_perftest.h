@@ -177,6 +177,13 @@ int nvshmem_perftest_moe_combine_ex(void *out, const void *recv, size_t recv_cap
                                     const int32_t *dest_pe, const int64_t *dest_row, int tokens,
                                     int topk, size_t row_bytes, int blocks_per_pe, int threads,
                                     int scope, void *stream);
+/* The same with a work item of piece_bytes (1024, 2048 or 4096; wavefront scope) of a row instead of
+ * a whole row (0): with 2 KiB items and one wavefront per block every block moves one short piece
+ * and exits. */
+int nvshmem_perftest_moe_combine_pieces(void *out, const void *recv, size_t recv_cap_rows,
+                                        const int32_t *dest_pe, const int64_t *dest_row, int tokens,
+                                        int topk, size_t row_bytes, int piece_bytes,
+                                        int blocks_per_pe, int threads, int scope, void *stream);
 /* Per-expert counts exchange + prefix sum on the device (examples/moe_shuffle.cu:204-234):
  * counts holds num_experts int64 per PE (rows this PE sends to each expert); on return
  * seg_base[e*npes + src] (int64, num_experts*npes words per PE, every PE gets the full table) is the

@@ -153,6 +153,7 @@ def load_perftest():
         "nvshmem_perftest_moe_dispatch_ex": [vp, sz, vp, vp, vp, vp, vp, i32, i32, sz, i32, i32, i32, vp],
         "nvshmem_perftest_moe_combine": [vp, vp, sz, vp, vp, i32, i32, sz, i32, i32, vp],
         "nvshmem_perftest_moe_combine_ex": [vp, vp, sz, vp, vp, i32, i32, sz, i32, i32, i32, vp],
+        "nvshmem_perftest_moe_combine_pieces": [vp, vp, sz, vp, vp, i32, i32, sz, i32, i32, i32, i32, vp],
         "nvshmem_perftest_moe_exchange_offsets": [vp, vp, vp, i32, vp],
     }
     for name, args in sig.items():

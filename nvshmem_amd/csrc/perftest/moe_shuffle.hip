@@ -116,7 +116,9 @@ __global__ void moe_dispatch_rowsignal_kernel(char *recv, const char *send, cons
     }
 }
 
-template <bool WARP_SCOPED>
+// PIECE > 0 (wavefront scope): a work item is PIECE bytes of a row instead of a whole row, so that
+// with one wavefront per block every block moves one short aligned piece and exits.
+template <bool WARP_SCOPED, int PIECE = 0>
 __global__ void moe_combine_kernel(char *out, const char *recv, const int32_t *dest_pe,
                                    const int64_t *dest_row, int tokens, int topk,
                                    size_t row_bytes, size_t recv_cap_rows) {
@@ -129,6 +131,18 @@ __global__ void moe_combine_kernel(char *out, const char *recv, const int32_t *d
         const size_t waves_per_block = blockDim.x / NVSHMEMI_WARP_SIZE;
         const size_t wave = blockIdx.x * waves_per_block + threadIdx.x / NVSHMEMI_WARP_SIZE;
         const size_t nwaves = (size_t)gridDim.x * waves_per_block;
+        if (PIECE > 0) {
+            const size_t pieces = (row_bytes + PIECE - 1) / PIECE;
+            for (size_t item = wave; item < rows * pieces; item += nwaves) {
+                const size_t r = item / pieces, off = (item - r * pieces) * PIECE;
+                const size_t len = row_bytes - off < (size_t)PIECE ? row_bytes - off : (size_t)PIECE;
+                if (row_ok(my_dest_pe[r], my_dest_row[r], np, recv_cap_rows))
+                    nvshmemx_getmem_nbi_warp(out + r * row_bytes + off,
+                                             recv + (size_t)my_dest_row[r] * row_bytes + off, len,
+                                             my_dest_pe[r]);
+            }
+            return;
+        }
         for (size_t r = wave; r < rows; r += nwaves)
             if (row_ok(my_dest_pe[r], my_dest_row[r], np, recv_cap_rows))
             nvshmemx_getmem_nbi_warp(out + r * row_bytes, recv + (size_t)my_dest_row[r] * row_bytes,
@@ -219,26 +233,42 @@ int nvshmem_perftest_moe_dispatch(void *recv, size_t recv_cap_rows, const void *
                                             NVSHMEM_PERFTEST_SCOPE_WARP, stream);
 }
 
-int nvshmem_perftest_moe_combine_ex(void *out, const void *recv, size_t recv_cap_rows, const int32_t *dest_pe,
-                                    const int64_t *dest_row, int tokens, int topk,
-                                    size_t row_bytes, int blocks_per_pe, int threads, int scope,
-                                    void *stream) {
+// piece_bytes: 0 = a work item is a whole row; 1024 / 2048 / 4096 (wavefront scope only) = a work
+// item is that many bytes of a row.  With one wavefront per block and 2 KiB items every block moves
+// one short piece and exits, which the memory system serves faster (measured 6.06 TB/s against
+// 5.3 TB/s for whole 14 KiB rows).
+int nvshmem_perftest_moe_combine_pieces(void *out, const void *recv, size_t recv_cap_rows,
+                                        const int32_t *dest_pe, const int64_t *dest_row, int tokens,
+                                        int topk, size_t row_bytes, int piece_bytes, int blocks_per_pe,
+                                        int threads, int scope, void *stream) {
     const bool warp = scope == NVSHMEM_PERFTEST_SCOPE_WARP;
     if (!warp && scope != NVSHMEM_PERFTEST_SCOPE_BLOCK) return NVSHMEMX_ERROR_INVALID_VALUE;
+    if (piece_bytes != 0 && (!warp || (piece_bytes != 1024 && piece_bytes != 2048 && piece_bytes != 4096)))
+        return NVSHMEMX_ERROR_INVALID_VALUE;
     if (!moe_args_ok(dest_pe, dest_row, tokens, topk, row_bytes, blocks_per_pe, threads, warp) ||
         !perftest::check_range(out, (size_t)tokens * (size_t)topk * row_bytes) ||
         !perftest::check_range(recv, recv_cap_rows * row_bytes))
         return NVSHMEMX_ERROR_INVALID_VALUE;
     const dim3 grid((unsigned)blocks_per_pe, 1, (unsigned)nvshmem_n_pes());
-    if (warp)
-        hipLaunchKernelGGL(moe_combine_kernel<true>, grid, dim3(threads), 0, (hipStream_t)stream,
-                           (char *)out, (const char *)recv, dest_pe, dest_row, tokens, topk, row_bytes,
-                           recv_cap_rows);
-    else
-        hipLaunchKernelGGL(moe_combine_kernel<false>, grid, dim3(threads), 0, (hipStream_t)stream,
-                           (char *)out, (const char *)recv, dest_pe, dest_row, tokens, topk, row_bytes,
-                           recv_cap_rows);
+#define LAUNCH_COMBINE(...)                                                                        \
+    hipLaunchKernelGGL((moe_combine_kernel<__VA_ARGS__>), grid, dim3(threads), 0, (hipStream_t)stream, \
+                       (char *)out, (const char *)recv, dest_pe, dest_row, tokens, topk, row_bytes,    \
+                       recv_cap_rows)
+    if (piece_bytes == 1024) LAUNCH_COMBINE(true, 1024);
+    else if (piece_bytes == 2048) LAUNCH_COMBINE(true, 2048);
+    else if (piece_bytes == 4096) LAUNCH_COMBINE(true, 4096);
+    else if (warp) LAUNCH_COMBINE(true, 0);
+    else LAUNCH_COMBINE(false, 0);
+#undef LAUNCH_COMBINE
     return perftest::launch_status("moe_combine");
+}
+
+int nvshmem_perftest_moe_combine_ex(void *out, const void *recv, size_t recv_cap_rows, const int32_t *dest_pe,
+                                    const int64_t *dest_row, int tokens, int topk,
+                                    size_t row_bytes, int blocks_per_pe, int threads, int scope,
+                                    void *stream) {
+    return nvshmem_perftest_moe_combine_pieces(out, recv, recv_cap_rows, dest_pe, dest_row, tokens, topk,
+                                               row_bytes, 0, blocks_per_pe, threads, scope, stream);
 }
 
 int nvshmem_perftest_moe_combine(void *out, const void *recv, size_t recv_cap_rows, const int32_t *dest_pe,

@@ -126,6 +126,9 @@ def sweep_moe(N, hip, iters):
                                                           None), iters, 2, hip)
     print("combine  (getmem_nbi per copy):        %.3f ms; %.1f GB/s (%.3f GiB read + written)"
           % (ms, 2 * moved / ms / 1e6, 2 * moved / 2**30))
+    ms = timeit(lambda: perf.nvshmem_perftest_moe_combine_pieces(out, recv, cap, d_pe, d_row, T, K, row, 2048,
+                                                                 262144, 64, N.SCOPE_WARP, None), iters, 2, hip)
+    print("combine  (getmem_nbi per 2 KiB piece):  %.3f ms; %.1f GB/s" % (ms, 2 * moved / ms / 1e6))
     assert all(rt.read_timeout(pe)[0] == 0 for pe in range(npes))
     rt.finalize()
 

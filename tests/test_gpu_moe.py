@@ -67,6 +67,17 @@ def _shuffle(rt, npes, T, K, E, row_bytes, blocks, threads, scope, seed_route=8,
         got = rt.download(out, pe, (rows, row_bytes), np.uint8)
         assert np.array_equal(got, want_out[pe]), pe
         assert np.array_equal(got, np.repeat(payload[pe], K, axis=0))   # round trip identity
+    # the same with a work item of part of a row per wavefront (ragged last piece included)
+    for piece in (1024, 2048, 4096):
+        rt.fill(out, 0xEE, rows * row_bytes)
+        note("moe_combine pieces of %d" % piece)
+        assert perf.nvshmem_perftest_moe_combine_pieces(out, recv, cap, d_pe, d_row, T, K, row_bytes, piece,
+                                                        4 * blocks, 64, N.SCOPE_WARP, None) == 0
+        rt.sync()
+        for pe in (0, npes - 1):
+            assert np.array_equal(rt.download(out, pe, (rows, row_bytes), np.uint8), want_out[pe]), (piece, pe)
+    assert perf.nvshmem_perftest_moe_combine_pieces(out, recv, cap, d_pe, d_row, T, K, row_bytes, 512,
+                                                    blocks, 64, N.SCOPE_WARP, None) != 0
     for p in (send, recv, out, d_pe, d_row, expected, sig, d_counts, d_seg, d_recv_rows):
         rt.free(p)
 
