@@ -151,6 +151,7 @@ def load_perftest():
         "nvshmem_perftest_device_barrier": [vp, vp, i32, i32, i32, vp],
         "nvshmem_perftest_moe_dispatch": [vp, sz, vp, vp, vp, vp, vp, i32, i32, sz, i32, i32, vp],
         "nvshmem_perftest_moe_dispatch_ex": [vp, sz, vp, vp, vp, vp, vp, i32, i32, sz, i32, i32, i32, vp],
+        "nvshmem_perftest_moe_dispatch_pieces": [vp, sz, vp, vp, vp, vp, vp, i32, i32, sz, i32, i32, vp],
         "nvshmem_perftest_moe_combine": [vp, vp, sz, vp, vp, i32, i32, sz, i32, i32, vp],
         "nvshmem_perftest_moe_combine_ex": [vp, vp, sz, vp, vp, i32, i32, sz, i32, i32, i32, vp],
         "nvshmem_perftest_moe_combine_pieces": [vp, vp, sz, vp, vp, i32, i32, sz, i32, i32, i32, i32, vp],

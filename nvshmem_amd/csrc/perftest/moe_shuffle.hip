@@ -8,6 +8,7 @@
 // A row of 14336 bytes is 896 16-byte vectors: a wavefront moves it with 14 vectors per lane, so
 // the default scope is one row per wavefront with no block-wide synchronisation in the loop.
 #include <hip/hip_runtime.h>
+#include <cstdlib>
 
 // A row is 14 vectors per lane: rounds of 8 + 4 + 2 keep more loads in flight than the default
 // 4 + 4 + 4 + 2 (measured 5 % faster for dispatch and combine).
@@ -25,6 +26,11 @@ constexpr int kMaxPes = NVSHMEMI_AMD_MAX_PES;
 __device__ __forceinline__ bool row_ok(int pe, int64_t row, int np, size_t cap_rows) {
     return (unsigned)pe < (unsigned)np && (uint64_t)row < (uint64_t)cap_rows;
 }
+
+// The wavefront's index is deliberately left a per-lane value: the routing entries indexed with it are
+// then fetched by vector loads of one address.  Making it a scalar (readfirstlane) turns them into
+// scalar loads, which measured 5 % slower here: the tables stream through the small scalar cache.
+__device__ __forceinline__ unsigned wave_in_block() { return threadIdx.x / NVSHMEMI_WARP_SIZE; }
 
 // Dispatch.  Rows are dealt round-robin to the thread groups of the PE's blocks.  Each group tallies
 // what it sent to every destination; once all its puts are complete it adds the tallies to the
@@ -44,7 +50,7 @@ __global__ void moe_dispatch_kernel(char *recv, const char *send, const int32_t 
 
     if (WARP_SCOPED) {
         const size_t waves_per_block = blockDim.x / NVSHMEMI_WARP_SIZE;
-        const size_t wave = blockIdx.x * waves_per_block + threadIdx.x / NVSHMEMI_WARP_SIZE;
+        const size_t wave = blockIdx.x * waves_per_block + wave_in_block();
         const size_t nwaves = (size_t)gridDim.x * waves_per_block;
         const bool lane0 = (threadIdx.x % NVSHMEMI_WARP_SIZE) == 0;
         // A wavefront takes a token and pushes its topk copies back to back: the first put streams
@@ -95,7 +101,7 @@ __global__ void moe_dispatch_rowsignal_kernel(char *recv, const char *send, cons
     const size_t rows = (size_t)tokens * (size_t)topk;
     if (WARP_SCOPED) {
         const size_t waves_per_block = blockDim.x / NVSHMEMI_WARP_SIZE;
-        const size_t wave = blockIdx.x * waves_per_block + threadIdx.x / NVSHMEMI_WARP_SIZE;
+        const size_t wave = blockIdx.x * waves_per_block + wave_in_block();
         const size_t nwaves = (size_t)gridDim.x * waves_per_block;
         for (size_t r = wave; r < rows; r += nwaves)
             if (row_ok(my_dest_pe[r], my_dest_row[r], np, recv_cap_rows))
@@ -116,6 +122,96 @@ __global__ void moe_dispatch_rowsignal_kernel(char *recv, const char *send, cons
     }
 }
 
+// Dispatch cut into short work items: an item is one piece of one token's row, pushed to all of the
+// token's topk destinations by one wavefront.  Grid: blockIdx.x = piece of the row, blockIdx.y (times
+// the wavefronts of a block) = token, so neither needs a division and consecutive blocks work on the
+// same row.  No tallies and no signalling here: the counts are published by
+// moe_dispatch_signal_kernel, launched behind this kernel on the same stream, so the end of this
+// kernel is what orders every row before its signal.
+//
+// PIECE bytes per item, moved with nvshmemx_putmem_nbi_warp (any alignment, any row size): the first
+// put streams the piece from HBM, the others find it in the cache.
+template <int PIECE>
+__global__ void moe_dispatch_pieces_kernel(char *recv, const char *send, const int32_t *dest_pe,
+                                           const int64_t *dest_row, int tokens, int topk,
+                                           size_t row_bytes, size_t recv_cap_rows) {
+    const int me = nvshmem_my_pe(), np = nvshmem_n_pes();
+    const int32_t *my_dest_pe = (const int32_t *)nvshmem_ptr(dest_pe, me);
+    const int64_t *my_dest_row = (const int64_t *)nvshmem_ptr(dest_row, me);
+    const unsigned waves_per_block = blockDim.x / NVSHMEMI_WARP_SIZE;
+    const size_t off = (size_t)blockIdx.x * PIECE;
+    if (off >= row_bytes) return;
+    const size_t len = row_bytes - off < (size_t)PIECE ? row_bytes - off : (size_t)PIECE;
+    for (size_t t = (size_t)blockIdx.y * waves_per_block + wave_in_block(); t < (size_t)tokens;
+         t += (size_t)gridDim.y * waves_per_block) {
+        const char *src = send + t * row_bytes + off;
+        for (int k = 0; k < topk; ++k) {
+            const size_t r = t * (size_t)topk + (size_t)k;
+            const int pe = my_dest_pe[r];
+            const int64_t row = my_dest_row[r];
+            if (!row_ok(pe, row, np, recv_cap_rows)) continue;
+            nvshmemx_putmem_nbi_warp(recv + (size_t)row * row_bytes + off, src, len, pe);
+        }
+    }
+}
+
+// The same work items moved with nvshmem_ptr and plain vector accesses: the piece is loaded ONCE into
+// registers (V 16-byte vectors per lane) and stored to the topk destinations from there, so a source
+// byte crosses the memory system once instead of topk times.  Needs 16-byte aligned buffers and
+// rows; the host picks moe_dispatch_pieces_kernel otherwise.
+template <int V>
+__global__ void moe_dispatch_direct_kernel(char *recv, const char *send, const int32_t *dest_pe,
+                                           const int64_t *dest_row, int tokens, int topk,
+                                           size_t row_bytes, size_t recv_cap_rows) {
+    const int me = nvshmem_my_pe(), np = nvshmem_n_pes();
+    const int32_t *my_dest_pe = (const int32_t *)nvshmem_ptr(dest_pe, me);
+    const int64_t *my_dest_row = (const int64_t *)nvshmem_ptr(dest_row, me);
+    const nvshmemi_v4u *my_send = (const nvshmemi_v4u *)nvshmem_ptr(send, me);
+    const unsigned waves_per_block = blockDim.x / NVSHMEMI_WARP_SIZE;
+    const unsigned row_vecs = (unsigned)(row_bytes / 16);
+    const unsigned v0 = blockIdx.x * (64 * V) + threadIdx.x % NVSHMEMI_WARP_SIZE;
+    for (size_t t = (size_t)blockIdx.y * waves_per_block + wave_in_block(); t < (size_t)tokens;
+         t += (size_t)gridDim.y * waves_per_block) {
+        const nvshmemi_v4u *src = my_send + t * row_vecs;
+        nvshmemi_v4u x[V];
+#pragma unroll
+        for (int u = 0; u < V; ++u)
+            if (v0 + 64 * u < row_vecs) x[u] = __builtin_nontemporal_load(src + v0 + 64 * u);
+        for (int k = 0; k < topk; ++k) {
+            const size_t r = t * (size_t)topk + (size_t)k;
+            const int pe = my_dest_pe[r];
+            const int64_t row = my_dest_row[r];
+            if (!row_ok(pe, row, np, recv_cap_rows)) continue;
+            nvshmemi_v4u *d = (nvshmemi_v4u *)nvshmem_ptr(recv, pe) + (size_t)row * row_vecs;
+#pragma unroll
+            for (int u = 0; u < V; ++u)
+                if (v0 + 64 * u < row_vecs) __builtin_nontemporal_store(x[u], d + v0 + 64 * u);
+        }
+    }
+}
+
+// One block per PE: counts the rows this PE sent to every destination, adds the counts to the
+// destinations' signal words and waits until every source has announced what this PE expects.
+__global__ void moe_dispatch_signal_kernel(const int32_t *dest_pe, const int64_t *dest_row,
+                                           const uint64_t *expected, uint64_t *sig, int tokens,
+                                           int topk, size_t recv_cap_rows) {
+    __shared__ unsigned tally[kMaxPes];
+    const int me = nvshmem_my_pe(), np = nvshmem_n_pes();
+    const int32_t *my_dest_pe = (const int32_t *)nvshmem_ptr(dest_pe, me);
+    const int64_t *my_dest_row = (const int64_t *)nvshmem_ptr(dest_row, me);
+    const size_t rows = (size_t)tokens * (size_t)topk;
+    for (int i = threadIdx.x; i < np; i += blockDim.x) tally[i] = 0;
+    __syncthreads();
+    for (size_t r = threadIdx.x; r < rows; r += blockDim.x)
+        if (row_ok(my_dest_pe[r], my_dest_row[r], np, recv_cap_rows)) atomicAdd(&tally[my_dest_pe[r]], 1u);
+    __syncthreads();
+    for (int pe = threadIdx.x; pe < np; pe += blockDim.x)
+        if (tally[pe]) nvshmemx_signal_op(sig + me, (uint64_t)tally[pe], NVSHMEM_SIGNAL_ADD, pe);
+    const uint64_t *my_expected = (const uint64_t *)nvshmem_ptr(expected, me);
+    for (int src = threadIdx.x; src < np; src += blockDim.x)
+        nvshmem_signal_wait_until(sig + src, NVSHMEM_CMP_GE, my_expected[src]);
+}
+
 // PIECE > 0 (wavefront scope): a work item is PIECE bytes of a row instead of a whole row, so that
 // with one wavefront per block every block moves one short aligned piece and exits.
 template <bool WARP_SCOPED, int PIECE = 0>
@@ -129,7 +225,7 @@ __global__ void moe_combine_kernel(char *out, const char *recv, const int32_t *d
     const size_t rows = (size_t)tokens * (size_t)topk;
     if (WARP_SCOPED) {
         const size_t waves_per_block = blockDim.x / NVSHMEMI_WARP_SIZE;
-        const size_t wave = blockIdx.x * waves_per_block + threadIdx.x / NVSHMEMI_WARP_SIZE;
+        const size_t wave = blockIdx.x * waves_per_block + wave_in_block();
         const size_t nwaves = (size_t)gridDim.x * waves_per_block;
         if (PIECE > 0) {
             const size_t pieces = (row_bytes + PIECE - 1) / PIECE;
@@ -231,6 +327,54 @@ int nvshmem_perftest_moe_dispatch(void *recv, size_t recv_cap_rows, const void *
     return nvshmem_perftest_moe_dispatch_ex(recv, recv_cap_rows, send, dest_pe, dest_row, expected, sig, tokens,
                                             topk, row_bytes, blocks_per_pe, threads,
                                             NVSHMEM_PERFTEST_SCOPE_WARP, stream);
+}
+
+// Dispatch as two launches on `stream`: a grid with one wavefront per work item - piece_bytes (1024 /
+// 2048 / 4096) of a token's row, pushed to its topk destinations - then one block per PE that
+// publishes the row counts through the signal words and waits for the expected ones.  `threads` (a
+// multiple of 64) sets how many tokens a block takes.
+int nvshmem_perftest_moe_dispatch_pieces(void *recv, size_t recv_cap_rows, const void *send,
+                                         const int32_t *dest_pe, const int64_t *dest_row,
+                                         const uint64_t *expected, uint64_t *sig, int tokens, int topk,
+                                         size_t row_bytes, int piece_bytes, int threads, void *stream) {
+    if (piece_bytes != 1024 && piece_bytes != 2048 && piece_bytes != 4096) return NVSHMEMX_ERROR_INVALID_VALUE;
+    if (!moe_args_ok(dest_pe, dest_row, tokens, topk, row_bytes, 1, threads, true))
+        return NVSHMEMX_ERROR_INVALID_VALUE;
+    const size_t words = sizeof(uint64_t) * (size_t)nvshmem_n_pes();
+    const size_t pieces = (row_bytes + (size_t)piece_bytes - 1) / (size_t)piece_bytes;
+    if (pieces > 0x7fffffffull || !perftest::check_range(expected, words) ||
+        !perftest::check_range(sig, words) || !perftest::check_range(send, (size_t)tokens * row_bytes) ||
+        !perftest::check_range(recv, recv_cap_rows * row_bytes))
+        return NVSHMEMX_ERROR_INVALID_VALUE;
+    const unsigned waves = (unsigned)threads / NVSHMEMI_WARP_SIZE;
+    unsigned token_blocks = ((unsigned)tokens + waves - 1) / waves;
+    if (token_blocks > 65535u) token_blocks = 65535u;  // the kernels stride over the rest
+    const dim3 grid((unsigned)pieces, token_blocks, (unsigned)nvshmem_n_pes());
+    const bool aligned = row_bytes % 16 == 0 && ((uintptr_t)recv | (uintptr_t)send) % 16 == 0;
+    const bool direct = aligned && getenv("NVSHMEM_PERFTEST_MOE_PUTS") == nullptr;
+#define LAUNCH_DIRECT(V)                                                                           \
+    hipLaunchKernelGGL((moe_dispatch_direct_kernel<V>), grid, dim3(threads), 0, (hipStream_t)stream, \
+                       (char *)recv, (const char *)send, dest_pe, dest_row, tokens, topk, row_bytes, \
+                       recv_cap_rows)
+#define LAUNCH_DISPATCH(P)                                                                         \
+    hipLaunchKernelGGL((moe_dispatch_pieces_kernel<P>), grid, dim3(threads), 0, (hipStream_t)stream, \
+                       (char *)recv, (const char *)send, dest_pe, dest_row, tokens, topk, row_bytes, \
+                       recv_cap_rows)
+    if (direct) {
+        if (piece_bytes == 1024) LAUNCH_DIRECT(1);
+        else if (piece_bytes == 2048) LAUNCH_DIRECT(2);
+        else LAUNCH_DIRECT(4);
+    } else if (piece_bytes == 1024) LAUNCH_DISPATCH(1024);
+    else if (piece_bytes == 2048) LAUNCH_DISPATCH(2048);
+    else LAUNCH_DISPATCH(4096);
+#undef LAUNCH_DISPATCH
+#undef LAUNCH_DIRECT
+    int rc = perftest::launch_status("moe_dispatch_pieces");
+    if (rc != 0) return rc;
+    // 8..64 blocks in all: co-resident on any GPU, an ordinary launch is enough for the waits
+    hipLaunchKernelGGL(moe_dispatch_signal_kernel, dim3(1, 1, (unsigned)nvshmem_n_pes()), dim3(1024), 0,
+                       (hipStream_t)stream, dest_pe, dest_row, expected, sig, tokens, topk, recv_cap_rows);
+    return perftest::launch_status("moe_dispatch_signal");
 }
 
 // piece_bytes: 0 = a work item is a whole row; 1024 / 2048 / 4096 (wavefront scope only) = a work

@@ -50,7 +50,7 @@ def counter_avg(directory, counter):
 WORKLOADS = {
     "ring_rma_kernel<2, false>": (
         "ring_rma_kernel_put_block_8pe_256MiB.txt",
-        "put_block: nvshmemx_putmem_block ring, 8 logical PEs x 256 MiB, 65536 blocks x 128 threads per PE.\n"
+        "put_block: nvshmemx_putmem_block ring, 8 logical PEs x 256 MiB, 262144 blocks x 64 threads per PE (1 KiB per block).\n"
         "Algorithmic bytes per launch: 8 x 256 MiB read + 8 x 256 MiB written = 4 GiB.", 4 << 30),
     "reduce_vector_kernel<float, 5, 8, true, false,": (
         "reduce_vector_kernel_float_sum_8pe_64Mi.txt",

@@ -58,6 +58,25 @@ def _shuffle(rt, npes, T, K, E, row_bytes, blocks, threads, scope, seed_route=8,
     sigs = rt.download_all(sig, (npes,), np.uint64)
     assert np.array_equal(sigs, exp_tab)                 # ADD signals count the rows exactly
 
+    # dispatch cut into short work items (two launches: data, then signals): same result, same signals.
+    # Aligned buffers and rows take the load-once path, anything else the put path.
+    for piece, threads in ((1024, 64), (2048, 128), (4096, 256)):
+        rt.fill(recv, 0, cap * row_bytes)
+        rt.fill(sig, 0, npes * 8)
+        note("moe_dispatch_pieces piece=%d threads=%d row=%d" % (piece, threads, row_bytes))
+        assert perf.nvshmem_perftest_moe_dispatch_pieces(recv, cap, send, d_pe, d_row, expected, sig, T, K,
+                                                         row_bytes, piece, threads, None) == 0
+        rt.sync()
+        assert all(rt.read_timeout(pe)[0] == 0 for pe in range(npes)), "a receiver gave up waiting"
+        for pe in range(npes):
+            got = rt.download(recv, pe, (int(recv_rows[pe]), row_bytes), np.uint8)
+            assert np.array_equal(got, want_recv[pe]), (piece, pe)
+        assert np.array_equal(rt.download_all(sig, (npes,), np.uint64), exp_tab)
+    assert perf.nvshmem_perftest_moe_dispatch_pieces(recv, cap, send, d_pe, d_row, expected, sig, T, K,
+                                                     row_bytes, 512, 64, None) != 0
+    assert perf.nvshmem_perftest_moe_dispatch_pieces(recv, cap, send, d_pe, d_row, expected, sig, T, K,
+                                                     row_bytes, 1024, 96, None) != 0
+
     note("moe_combine")
     assert perf.nvshmem_perftest_moe_combine_ex(out, recv, cap, d_pe, d_row, T, K, row_bytes, blocks,
                                                 threads, scope & 255, None) == 0
@@ -104,6 +123,12 @@ def test_moe_routing_table_outside_the_buffer_is_skipped_not_written():
                                                   row, 2, 128, None) == 0
         rt.sync()
         assert (rt.download_all(sig, (4,), np.uint64) == 0).all()
+        note("moe_dispatch_pieces with invalid routing entries")
+        assert perf.nvshmem_perftest_moe_dispatch_pieces(recv, 8, send, d_pe, d_row, expected, sig, T, K,
+                                                         row, 1024, 128, None) == 0
+        rt.sync()
+        assert (rt.download_all(sig, (4,), np.uint64) == 0).all()
+        assert (rt.download_all(recv, (8 * row,), np.uint8) == 0).all()
 
 
 def test_config5_full_size_moe_shuffle():
