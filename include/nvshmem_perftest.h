@@ -64,6 +64,28 @@ int nvshmem_perftest_signal_wait(uint64_t *sig, int cmp, uint64_t cmp_value, uin
 int nvshmem_perftest_put_signal_pingpong(void *data, uint64_t *sig, size_t bytes, int iters,
                                          int threads, void *stream);
 
+/* Latency loops of the reference's perftest/device/pt-to-pt programs, one block per PE, `iters`
+ * repetitions inside one launch.  Kinds 0-4: PE 0 acts on PE 1 - PUT: nvshmemx_putmem_block of `bytes`
+ * of data + quiet (afterwards PE 1's data equals PE 0's); GET: nvshmemx_getmem_block (PE 0's data
+ * equals PE 1's); P: nvshmem_uint64_p(sig, i) + quiet (PE 1's sig[0] == iters); G: nvshmem_uint64_g
+ * of PE 1's sig[0], the sum of the values read goes to PE 0's sig[1]; ATOMIC: a dependent chain of
+ * nvshmem_uint64_atomic_fetch_add(sig, 1) (PE 1's sig[0] grows by iters, the last value fetched
+ * goes to PE 0's sig[1]).  Kinds 5-7: PE 0 and PE 1 bounce a word with signal_op SET / uint64_p /
+ * atomic_inc and nvshmem_uint64_wait_until(EQ): sig[0] must be 0 before, is iters on both after.
+ * sig holds two words per PE; npes must be >= 2. */
+enum {
+    NVSHMEM_PERFTEST_LAT_PUT = 0,
+    NVSHMEM_PERFTEST_LAT_GET = 1,
+    NVSHMEM_PERFTEST_LAT_P = 2,
+    NVSHMEM_PERFTEST_LAT_G = 3,
+    NVSHMEM_PERFTEST_LAT_ATOMIC = 4,
+    NVSHMEM_PERFTEST_LAT_SIGNAL_PINGPONG = 5,
+    NVSHMEM_PERFTEST_LAT_P_PINGPONG = 6,
+    NVSHMEM_PERFTEST_LAT_ATOMIC_PINGPONG = 7
+};
+int nvshmem_perftest_pt2pt_latency(int what, void *data, uint64_t *sig, size_t bytes, int iters,
+                                   int threads, void *stream);
+
 /* Ring allreduce of int32 built from put_signal_nbi + signal_wait_until, the algorithm of
  * examples/ring-reduce.cu:88-144: reduce phase around the ring, then broadcast phase.  nreduce must
  * be a multiple of blocks*chunk_elems.  signal holds `blocks` words (zero before the call; the

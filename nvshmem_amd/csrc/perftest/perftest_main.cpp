@@ -14,6 +14,9 @@
 //        coll_latency                       the same five calls made inside a kernel, the call
 //                                           repeated --iters times in one launch
 //        barrier_latency                    nvshmem_barrier_all inside a kernel
+//        pt2pt_latency                      put / get (+ put_signal ping-pong) latency per size and
+//                                           p, g, fetching atomic, signal / p / atomic ping-pong
+//                                           latency between PE 0 and PE 1, inside one kernel
 #include <hip/hip_runtime.h>
 
 #include <cstdio>
@@ -38,7 +41,7 @@ struct Options {
 
 [[noreturn]] void usage(const char *why) {
     fprintf(stderr, "nvshmem_perftest: %s\nusage: nvshmem_perftest <put_bw|get_bw|reduce|reducescatter|fcollect|"
-                    "alltoall|broadcast|coll_latency|barrier_latency> [--npes N] [--min B] [--max B] [--iters K] "
+                    "alltoall|broadcast|coll_latency|barrier_latency|pt2pt_latency> [--npes N] [--min B] [--max B] [--iters K] "
                     "[--warmup W] [--blocks B] [--threads T] [--scope thread|warp|block]\n", why);
     exit(2);
 }
@@ -236,13 +239,60 @@ int run_device_latency(const Options &o, bool barrier_only) {
     return 0;
 }
 
+// (launch with K + 1 repetitions - launch with 1) / K, like run_device_latency; sig is cleared before
+// every launch because the ping-pong kinds count from zero.
+int run_pt2pt_latency(const Options &o) {
+    void *data = nvshmem_malloc(o.max_bytes);
+    uint64_t *sig = (uint64_t *)nvshmem_calloc(2, sizeof(uint64_t));
+    if (!data || !sig) return 1;
+    const int threads = o.threads ? o.threads : 256;
+    auto clear = [&] {
+        for (int pe = 0; pe < 2; ++pe) CHECK_HIP(hipMemsetAsync(nvshmem_ptr(sig, pe), 0, 16, nullptr));
+    };
+    auto latency_us = [&](auto launch) {
+        auto one = [&] { clear(); return launch(1); };
+        auto many = [&] { clear(); return launch(o.iters + 1); };
+        const double t1 = time_ms(one, 5, 2), tk = time_ms(many, 5, 2);
+        return (tk - t1) * 1e3 / o.iters;
+    };
+    std::vector<size_t> sizes = sweep(o, 1);
+    static const struct { int what; const char *job; } sized[] = {
+        {NVSHMEM_PERFTEST_LAT_PUT, "shmem_put_latency"}, {NVSHMEM_PERFTEST_LAT_GET, "shmem_get_latency"}};
+    for (const auto &c : sized) {
+        std::vector<double> us;
+        for (size_t bytes : sizes)
+            us.push_back(latency_us([&](int k) { return nvshmem_perftest_pt2pt_latency(c.what, data, sig, bytes, k, threads, nullptr); }));
+        print_table(c.job, "block", "latency", "us", sizes, us);
+    }
+    {
+        std::vector<double> us;  // a full round trip, as the reference reports it
+        for (size_t bytes : sizes)
+            us.push_back(latency_us([&](int k) { return nvshmem_perftest_put_signal_pingpong(data, sig, bytes, k, threads, nullptr); }));
+        print_table("shmem_put_signal_ping_pong_latency", "block", "round trip", "us", sizes, us);
+    }
+    static const struct { int what; const char *job; } scalar[] = {
+        {NVSHMEM_PERFTEST_LAT_P, "shmem_p_latency (p + quiet)"},
+        {NVSHMEM_PERFTEST_LAT_G, "shmem_g_latency"},
+        {NVSHMEM_PERFTEST_LAT_ATOMIC, "shmem_atomic_latency (fetch_add)"},
+        {NVSHMEM_PERFTEST_LAT_SIGNAL_PINGPONG, "shmem_signal_ping_pong_latency (round trip)"},
+        {NVSHMEM_PERFTEST_LAT_P_PINGPONG, "shmem_p_ping_pong_latency (round trip)"},
+        {NVSHMEM_PERFTEST_LAT_ATOMIC_PINGPONG, "shmem_atomic_ping_pong_latency (round trip)"}};
+    printf("#scalar operations, PE 0 <-> PE 1\n%-48s  %-16s\n", "test", "latency (us)");
+    for (const auto &c : scalar)
+        printf("%-48s  %-16.6f\n", c.job,
+               latency_us([&](int k) { return nvshmem_perftest_pt2pt_latency(c.what, data, sig, 8, k, threads, nullptr); }));
+    nvshmem_free(data);
+    nvshmem_free(sig);
+    return 0;
+}
+
 }  // namespace
 
 int main(int argc, char **argv) {
     const Options o = parse(argc, argv);
-    const bool device_lat = o.test == "coll_latency" || o.test == "barrier_latency";
+    const bool device_lat = o.test == "coll_latency" || o.test == "barrier_latency" || o.test == "pt2pt_latency";
     // heap: source and dest of the largest size, times npes for the collectives
-    const bool rma = o.test == "put_bw" || o.test == "get_bw";
+    const bool rma = o.test == "put_bw" || o.test == "get_bw" || o.test == "pt2pt_latency";
     Options eff = o;
     if (device_lat && o.max_bytes > ((size_t)1 << 20)) eff.max_bytes = (size_t)1 << 20;
     const size_t per_pe = (rma ? 2 * eff.max_bytes : 2 * eff.max_bytes * (size_t)eff.npes) + ((size_t)16 << 20);
@@ -260,6 +310,7 @@ int main(int argc, char **argv) {
     else if (o.test == "broadcast") rc = run_host_collective(eff, kBroadcast);
     else if (o.test == "coll_latency") rc = run_device_latency(eff, false);
     else if (o.test == "barrier_latency") rc = run_device_latency(eff, true);
+    else if (o.test == "pt2pt_latency") rc = run_pt2pt_latency(eff);
     else usage("unknown test");
     if (rc != 0) fprintf(stderr, "nvshmem_perftest: %s\n", nvshmemx_amd_last_error());
     nvshmem_finalize();

@@ -96,6 +96,63 @@ __global__ void pingpong_kernel(char *data, uint64_t *sig, size_t bytes, int ite
     }
 }
 
+// Point-to-point latency loops in the shape of the reference's perftest/device/pt-to-pt programs:
+// PE 0 acts on PE 1 `iters` times (kinds 0-4: shmem_put_latency.cu, shmem_get_latency.cu,
+// shmem_p_latency.cu, shmem_g_latency.cu, shmem_atomic_latency.cu), or PE 0 and PE 1 bounce a word
+// (kinds 5-7: shmem_signal_ping_pong_latency.cu, shmem_p_ping_pong_latency.cu,
+// shmem_atomic_ping_pong_latency.cu).  sig holds two words per PE.
+__global__ void pt2pt_latency_kernel(int what, char *data, uint64_t *sig, size_t bytes, int iters) {
+    const int me = nvshmem_my_pe();
+    if (me > 1) return;
+    const int peer = 1 - me;
+    if (what <= NVSHMEM_PERFTEST_LAT_ATOMIC) {
+        if (me != 0) return;
+        uint64_t acc = 0;
+        for (int i = 1; i <= iters; ++i) {
+            switch (what) {
+                case NVSHMEM_PERFTEST_LAT_PUT:
+                    nvshmemx_putmem_block(data, data, bytes, peer);
+                    nvshmem_quiet();
+                    break;
+                case NVSHMEM_PERFTEST_LAT_GET:
+                    nvshmemx_getmem_block(data, data, bytes, peer);
+                    break;
+                case NVSHMEM_PERFTEST_LAT_P:
+                    if (threadIdx.x == 0) {
+                        nvshmem_uint64_p(sig, (uint64_t)i, peer);
+                        nvshmem_quiet();
+                    }
+                    break;
+                case NVSHMEM_PERFTEST_LAT_G:
+                    if (threadIdx.x == 0) acc += nvshmem_uint64_g(sig, peer);
+                    break;
+                default:
+                    // every fetch depends on the one before: a chain of round trips
+                    if (threadIdx.x == 0) acc = nvshmem_uint64_atomic_fetch_add(sig, 1 + (acc >> 63), peer);
+                    break;
+            }
+        }
+        if (threadIdx.x == 0 && what >= NVSHMEM_PERFTEST_LAT_G) ((uint64_t *)nvshmem_ptr(sig, me))[1] = acc;
+        return;
+    }
+    if (threadIdx.x != 0) return;
+    for (int i = 1; i <= iters; ++i) {
+        if (me == 1) nvshmem_uint64_wait_until(sig, NVSHMEM_CMP_EQ, (uint64_t)i);
+        switch (what) {
+            case NVSHMEM_PERFTEST_LAT_SIGNAL_PINGPONG:
+                nvshmemx_signal_op(sig, (uint64_t)i, NVSHMEM_SIGNAL_SET, peer);
+                break;
+            case NVSHMEM_PERFTEST_LAT_P_PINGPONG:
+                nvshmem_uint64_p(sig, (uint64_t)i, peer);
+                break;
+            default:
+                nvshmem_uint64_atomic_inc(sig, peer);
+                break;
+        }
+        if (me == 0) nvshmem_uint64_wait_until(sig, NVSHMEM_CMP_EQ, (uint64_t)i);
+    }
+}
+
 // Ring allreduce: the partial sum travels PE 0 -> 1 -> ... -> n-1 chunk by chunk (reduce phase),
 // then the finished chunks travel n-1 -> 0 -> ... -> n-2 (broadcast phase).  A signal word per
 // block counts the chunks that have arrived.
@@ -244,6 +301,18 @@ int nvshmem_perftest_put_signal_pingpong(void *data, uint64_t *sig, size_t bytes
     char *d = (char *)data;
     void *args[] = {&d, &sig, &bytes, &iters};
     return nvshmemx_collective_launch((const void *)pingpong_kernel, dim3(1), dim3(threads), args,
+                                      0, (hipStream_t)stream);
+}
+
+int nvshmem_perftest_pt2pt_latency(int what, void *data, uint64_t *sig, size_t bytes, int iters,
+                                   int threads, void *stream) {
+    if (!perftest::ready() || nvshmem_n_pes() < 2 || what < 0 || what > NVSHMEM_PERFTEST_LAT_ATOMIC_PINGPONG ||
+        iters < 1 || !perftest::check_launch(1, threads) || !perftest::check_range(data, bytes) ||
+        !perftest::check_range(sig, 2 * sizeof(uint64_t)))
+        return NVSHMEMX_ERROR_INVALID_VALUE;
+    char *d = (char *)data;
+    void *args[] = {&what, &d, &sig, &bytes, &iters};
+    return nvshmemx_collective_launch((const void *)pt2pt_latency_kernel, dim3(1), dim3(threads), args,
                                       0, (hipStream_t)stream);
 }
 

@@ -63,3 +63,15 @@ def test_device_latency_tables():
 def test_bad_arguments_are_refused():
     proc = subprocess.run([DRIVER, "nonsense"], stdout=subprocess.PIPE, stderr=subprocess.PIPE, timeout=100)
     assert proc.returncode == 2 and b"usage" in proc.stderr
+
+
+def test_point_to_point_latency_tables():
+    out = _run("pt2pt_latency", "--min", "8", "--max", "4k", "--iters", "50")
+    for job in ("shmem_put_latency", "shmem_get_latency", "shmem_put_signal_ping_pong_latency"):
+        rows = _rows(out, job)
+        assert [r[0] for r in rows] == [8 << i for i in range(10)]
+        assert all(0.0 < v < 1000.0 for _, _, v in rows), (job, rows)
+    for name in ("shmem_p_latency", "shmem_g_latency", "shmem_atomic_latency", "shmem_signal_ping_pong_latency",
+                 "shmem_p_ping_pong_latency", "shmem_atomic_ping_pong_latency"):
+        line = next(l for l in out.splitlines() if l.startswith(name))
+        assert 0.0 < float(line.split()[-1]) < 1000.0, line

@@ -156,6 +156,42 @@ def test_put_signal_pingpong(rt):
         rt.free(data); rt.free(sig)
 
 
+def test_point_to_point_latency_loops_leave_the_documented_state(rt):
+    # kinds of nvshmem_perftest_pt2pt_latency (include/nvshmem_perftest.h): what PE 0 and PE 1 hold
+    # afterwards is fixed by the loop, so the timing kernels double as functional checks
+    perf = rt.perftest()
+    nbytes, iters = 4099, 37
+    data = rt.malloc(nbytes); sig = rt.calloc(2, 8)
+    payload = O.fill_all("bytes", NPES, nbytes, 31)
+
+    def run(what, start=0):
+        rt.upload_all(data, payload)
+        rt.upload_all(sig, np.tile(np.array([start, 0], np.uint64), (NPES, 1)))
+        note("pt2pt_latency kind=%d" % what)
+        assert perf.nvshmem_perftest_pt2pt_latency(what, data, sig, nbytes, iters, 128, None) == 0
+        rt.sync()
+        assert all(rt.read_timeout(pe)[0] == 0 for pe in range(NPES))
+        return rt.download_all(data, (nbytes,), np.uint8), _words(rt, sig, 2)
+
+    got, w = run(0)                                            # put: PE 1 receives PE 0's bytes
+    assert np.array_equal(got[1], payload[0]) and np.array_equal(got[0], payload[0])
+    assert np.array_equal(got[2:], payload[2:]) and (w == 0).all()
+    got, w = run(1)                                            # get: PE 0 fetches PE 1's bytes
+    assert np.array_equal(got[0], payload[1]) and np.array_equal(got[1], payload[1])
+    got, w = run(2)                                            # p: the last value written is iters
+    assert w[1, 0] == iters and w[0, 0] == 0 and np.array_equal(got, payload)
+    got, w = run(3, start=5)                                   # g: iters reads of the value 5
+    assert w[0, 1] == 5 * iters and w[1, 0] == 5
+    got, w = run(4, start=100)                                 # fetch_add chain on PE 1's word
+    assert w[1, 0] == 100 + iters and w[0, 1] == 100 + iters - 1 and w[0, 0] == 100
+    for what in (5, 6, 7):                                     # ping-pong: both words count the rounds
+        got, w = run(what)
+        assert w[0, 0] == iters and w[1, 0] == iters and (w[2:] == 0).all()
+    assert perf.nvshmem_perftest_pt2pt_latency(8, data, sig, nbytes, iters, 128, None) != 0
+    assert perf.nvshmem_perftest_pt2pt_latency(0, data, sig, nbytes, 0, 128, None) != 0
+    rt.free(data); rt.free(sig)
+
+
 def test_ring_allreduce_from_put_signal_known_answer_and_oracle(rt):
     perf = rt.perftest()
     blocks, chunk, chunks = 4, 1024, 3
