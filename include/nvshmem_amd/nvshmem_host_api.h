@@ -245,10 +245,44 @@ NVSHMEMI_REPT_FOR_SIZES(NVSHMEMI_DECL_SIZED_RMA_HOST)
                                                                    nvshmemx_stream_t stream);     \
     NVSHMEMI_HOST_ONLY void nvshmemx_##NAME##_wait_until_all_on_stream(                           \
         TYPE *ivars, size_t nelems, const int *status, int cmp, TYPE cmp_value,                   \
+        nvshmemx_stream_t stream);                                                                \
+    NVSHMEMI_HOST_ONLY void nvshmemx_##NAME##_wait_until_all_vector_on_stream(                    \
+        TYPE *ivars, size_t nelems, const int *status, int cmp, TYPE *cmp_values,                 \
         nvshmemx_stream_t stream);
 NVSHMEMI_REPT_FOR_WAIT_TYPES(NVSHMEMI_DECL_WAIT_ON_STREAM)
 #undef NVSHMEMI_DECL_WAIT_ON_STREAM
 NVSHMEMI_HOST_ONLY uint64_t nvshmem_signal_fetch(uint64_t *sig_addr);
+
+/* ---- atomic memory operations from the host (nvshmem_api.h:113-197) ----
+ * Blocking: the operation is applied to `target` on PE `pe` by a one-thread kernel on the default
+ * stream and the call returns once it is done (with the value fetched, for the fetching forms).
+ * The reference declares the same names and defines them as stubs that print "not implemented"
+ * (src/host/comm/amo.cpp); here they perform the operation. */
+#define NVSHMEMI_DECL_AMO_FETCH_SET_SWAP_HOST(NAME, TYPE)                                         \
+    NVSHMEMI_HOST_ONLY TYPE nvshmem_##NAME##_atomic_fetch(const TYPE *target, int pe);            \
+    NVSHMEMI_HOST_ONLY void nvshmem_##NAME##_atomic_set(TYPE *target, TYPE value, int pe);        \
+    NVSHMEMI_HOST_ONLY TYPE nvshmem_##NAME##_atomic_swap(TYPE *target, TYPE value, int pe);
+NVSHMEMI_REPT_FOR_STANDARD_AMO_TYPES(NVSHMEMI_DECL_AMO_FETCH_SET_SWAP_HOST)
+NVSHMEMI_REPT_FOR_EXTENDED_AMO_TYPES(NVSHMEMI_DECL_AMO_FETCH_SET_SWAP_HOST)
+#undef NVSHMEMI_DECL_AMO_FETCH_SET_SWAP_HOST
+#define NVSHMEMI_DECL_AMO_ARITH_HOST(NAME, TYPE)                                                  \
+    NVSHMEMI_HOST_ONLY TYPE nvshmem_##NAME##_atomic_compare_swap(TYPE *target, TYPE cond,         \
+                                                                 TYPE value, int pe);             \
+    NVSHMEMI_HOST_ONLY TYPE nvshmem_##NAME##_atomic_fetch_add(TYPE *target, TYPE value, int pe);  \
+    NVSHMEMI_HOST_ONLY void nvshmem_##NAME##_atomic_add(TYPE *target, TYPE value, int pe);        \
+    NVSHMEMI_HOST_ONLY TYPE nvshmem_##NAME##_atomic_fetch_inc(TYPE *target, int pe);              \
+    NVSHMEMI_HOST_ONLY void nvshmem_##NAME##_atomic_inc(TYPE *target, int pe);
+NVSHMEMI_REPT_FOR_STANDARD_AMO_TYPES(NVSHMEMI_DECL_AMO_ARITH_HOST)
+#undef NVSHMEMI_DECL_AMO_ARITH_HOST
+#define NVSHMEMI_DECL_AMO_BITWISE_HOST(NAME, TYPE)                                                \
+    NVSHMEMI_HOST_ONLY TYPE nvshmem_##NAME##_atomic_fetch_and(TYPE *target, TYPE value, int pe);  \
+    NVSHMEMI_HOST_ONLY TYPE nvshmem_##NAME##_atomic_fetch_or(TYPE *target, TYPE value, int pe);   \
+    NVSHMEMI_HOST_ONLY TYPE nvshmem_##NAME##_atomic_fetch_xor(TYPE *target, TYPE value, int pe);  \
+    NVSHMEMI_HOST_ONLY void nvshmem_##NAME##_atomic_and(TYPE *target, TYPE value, int pe);        \
+    NVSHMEMI_HOST_ONLY void nvshmem_##NAME##_atomic_or(TYPE *target, TYPE value, int pe);         \
+    NVSHMEMI_HOST_ONLY void nvshmem_##NAME##_atomic_xor(TYPE *target, TYPE value, int pe);
+NVSHMEMI_REPT_FOR_BITWISE_AMO_TYPES(NVSHMEMI_DECL_AMO_BITWISE_HOST)
+#undef NVSHMEMI_DECL_AMO_BITWISE_HOST
 
 /* ---- collectives: src/include/host/nvshmem_coll_api.h:27-80, nvshmemx_coll_api.h:27-80 ----
  * One call serves every PE of the team.  dest and src are canonical symmetric addresses.

@@ -189,7 +189,18 @@ def declared_symbols(header_paths=None):
             names.add("nvshmemx_" + form % bits + "_on_stream")
         names.update({"nvshmemx_put%d_signal_on_stream" % bits, "nvshmemx_put%d_signal_nbi_on_stream" % bits})
     for t in WAIT_TYPES:
-        names.update({"nvshmemx_%s_wait_until_on_stream" % t, "nvshmemx_%s_wait_until_all_on_stream" % t})
+        names.update({"nvshmemx_%s_wait_until_on_stream" % t, "nvshmemx_%s_wait_until_all_on_stream" % t,
+                      "nvshmemx_%s_wait_until_all_vector_on_stream" % t})
+    bitwise = ["uint", "ulong", "ulonglong", "int32", "int64", "uint32", "uint64"]
+    standard = bitwise + ["int", "long", "longlong", "size", "ptrdiff"]
+    for t in standard + ["float", "double"]:
+        names.update("nvshmem_%s_atomic_%s" % (t, op) for op in ("fetch", "set", "swap"))
+    for t in standard:
+        names.update("nvshmem_%s_atomic_%s" % (t, op)
+                     for op in ("compare_swap", "fetch_add", "add", "fetch_inc", "inc"))
+    for t in bitwise:
+        names.update("nvshmem_%s_atomic_%s" % (t, op)
+                     for op in ("fetch_and", "fetch_or", "fetch_xor", "and", "or", "xor"))
     for op in ("and", "or", "xor"):
         for t in REDUCE_TYPES_BITWISE:
             names.update({"nvshmem_%s_%s_reduce" % (t, op), "nvshmemx_%s_%s_reduce_on_stream" % (t, op),

@@ -5,6 +5,8 @@
 // for the waits).  Declarations: reference src/include/host/nvshmem_api.h:199-353 and
 // src/include/host/nvshmemx_api.h:94-275.
 #include <cstring>
+#include <mutex>
+#include <type_traits>
 
 #include "nvshmem.h"
 #include "runtime.hpp"
@@ -136,7 +138,92 @@ void wait_until_all_on_stream(T *ivars, size_t nelems, const int *status, int cm
     NVSHMEM_AMD_HIP_CHECK(hipGetLastError());
 }
 
+template <typename T>
+__global__ void wait_until_all_vector_kernel(T *ivars, size_t nelems, const int *status, int cmp,
+                                             const T *values) {
+    for (size_t i = threadIdx.x; i < nelems; i += blockDim.x)
+        if (!status || !status[i]) nvshmemi_wait_until<T>(ivars + i, cmp, values[i]);
+}
+
+// `status` and `cmp_values` are read by the kernel: device-accessible memory, as in the reference
+// (src/include/internal/non_abi/nvshmemi_h_to_d_sync_defs.cuh:52-70)
+template <typename T>
+void wait_until_all_vector_on_stream(T *ivars, size_t nelems, const int *status, int cmp, const T *values,
+                                     hipStream_t stream) {
+    Runtime &rt = Runtime::get();
+    uint64_t off = 0;
+    if (nelems == 0 || !rt.initialized ||
+        !check_symmetric_range(rt, "wait_until_all_vector_on_stream", ivars, nelems * sizeof(T), &off))
+        return;
+    if (cmp < NVSHMEM_CMP_EQ || cmp > NVSHMEM_CMP_GE) {
+        set_error("wait_until_all_vector_on_stream: unknown comparison %d", cmp);
+        return;
+    }
+    if (!values) {
+        set_error("wait_until_all_vector_on_stream: cmp_values is NULL");
+        return;
+    }
+    hipLaunchKernelGGL(wait_until_all_vector_kernel<T>, dim3(1), dim3(64), 0, stream, ivars, nelems, status,
+                       cmp, values);
+    NVSHMEM_AMD_HIP_CHECK(hipGetLastError());
+}
+
 void sync0() { NVSHMEM_AMD_HIP_CHECK(hipStreamSynchronize(nullptr)); }
+
+// Host-initiated atomics: one thread applies the device-side operation and leaves what it fetched in
+// a pinned word that the host reads after the stream has drained.
+template <typename T>
+__global__ void host_amo_kernel(int op, T *target, T value, T cond, int pe, T *fetched) {
+    T r = T(0);
+    switch (op) {
+        case NVSHMEMI_AMO_FETCH: r = nvshmemi_atomic_fetch<T>(target, pe); break;
+        case NVSHMEMI_AMO_SET: nvshmemi_atomic_set<T>(target, value, pe); break;
+        case NVSHMEMI_AMO_SWAP: r = nvshmemi_atomic_swap<T>(target, value, pe); break;
+        default:
+            if constexpr (!std::is_floating_point<T>::value) {
+                switch (op) {
+                    case NVSHMEMI_AMO_COMPARE_SWAP: r = nvshmemi_atomic_compare_swap<T>(target, cond, value, pe); break;
+                    case NVSHMEMI_AMO_FETCH_ADD: r = nvshmemi_atomic_fetch_add<T>(target, value, pe); break;
+                    case NVSHMEMI_AMO_FETCH_AND: r = nvshmemi_atomic_fetch_and<T>(target, value, pe); break;
+                    case NVSHMEMI_AMO_FETCH_OR: r = nvshmemi_atomic_fetch_or<T>(target, value, pe); break;
+                    case NVSHMEMI_AMO_FETCH_XOR: r = nvshmemi_atomic_fetch_xor<T>(target, value, pe); break;
+                    default: break;
+                }
+            }
+            break;
+    }
+    *fetched = r;
+}
+
+template <typename T>
+T host_amo(const char *what, int op, const T *target, T value, T cond, int pe) {
+    Runtime &rt = Runtime::get();
+    std::lock_guard<std::recursive_mutex> lock(rt.mu);
+    uint64_t off = 0;
+    if (!rt.initialized) {
+        set_error("%s called before nvshmem_init", what);
+        return T(0);
+    }
+    if (pe < 0 || pe >= rt.npes) {
+        set_error("%s: pe %d outside [0, %d)", what, pe, rt.npes);
+        return T(0);
+    }
+    if (!check_symmetric_range(rt, what, target, sizeof(T), &off)) return T(0);
+    if (off % sizeof(T)) {
+        set_error("%s: target is not aligned to its type", what);
+        return T(0);
+    }
+    static uint64_t *slot = nullptr;  // pinned, lives until the process ends
+    if (!slot) NVSHMEM_AMD_HIP_CHECK(hipHostMalloc((void **)&slot, sizeof(uint64_t), hipHostMallocDefault));
+    *slot = 0;
+    hipLaunchKernelGGL(host_amo_kernel<T>, dim3(1), dim3(1), 0, nullptr, op, const_cast<T *>(target), value, cond,
+                       pe, reinterpret_cast<T *>(slot));
+    NVSHMEM_AMD_HIP_CHECK(hipGetLastError());
+    sync0();
+    T out;
+    memcpy(&out, slot, sizeof(T));
+    return out;
+}
 
 }  // namespace
 }  // namespace nvshmem_amd
@@ -297,5 +384,69 @@ NVSHMEMI_REPT_FOR_SIZES(NVSHMEMI_DEFINE_SIZED_HOST_RMA)
     }
 NVSHMEMI_REPT_FOR_WAIT_TYPES(NVSHMEMI_DEFINE_WAIT_ON_STREAM)
 #undef NVSHMEMI_DEFINE_WAIT_ON_STREAM
+
+#define NVSHMEMI_DEFINE_WAIT_VECTOR_ON_STREAM(NAME, TYPE)                                         \
+    void nvshmemx_##NAME##_wait_until_all_vector_on_stream(TYPE *ivars, size_t nelems,            \
+                                                           const int *status, int cmp,            \
+                                                           TYPE *cmp_values, nvshmemx_stream_t s) { \
+        wait_until_all_vector_on_stream<TYPE>(ivars, nelems, status, cmp, cmp_values, (hipStream_t)s); \
+    }
+NVSHMEMI_REPT_FOR_WAIT_TYPES(NVSHMEMI_DEFINE_WAIT_VECTOR_ON_STREAM)
+#undef NVSHMEMI_DEFINE_WAIT_VECTOR_ON_STREAM
+
+#define NVSHMEMI_DEFINE_AMO_FETCH_SET_SWAP_HOST(NAME, TYPE)                                       \
+    TYPE nvshmem_##NAME##_atomic_fetch(const TYPE *target, int pe) {                              \
+        return host_amo<TYPE>("nvshmem_" #NAME "_atomic_fetch", NVSHMEMI_AMO_FETCH, target, (TYPE)0, (TYPE)0, pe); \
+    }                                                                                             \
+    void nvshmem_##NAME##_atomic_set(TYPE *target, TYPE value, int pe) {                          \
+        (void)host_amo<TYPE>("nvshmem_" #NAME "_atomic_set", NVSHMEMI_AMO_SET, target, value, (TYPE)0, pe); \
+    }                                                                                             \
+    TYPE nvshmem_##NAME##_atomic_swap(TYPE *target, TYPE value, int pe) {                         \
+        return host_amo<TYPE>("nvshmem_" #NAME "_atomic_swap", NVSHMEMI_AMO_SWAP, target, value, (TYPE)0, pe); \
+    }
+NVSHMEMI_REPT_FOR_STANDARD_AMO_TYPES(NVSHMEMI_DEFINE_AMO_FETCH_SET_SWAP_HOST)
+NVSHMEMI_REPT_FOR_EXTENDED_AMO_TYPES(NVSHMEMI_DEFINE_AMO_FETCH_SET_SWAP_HOST)
+#undef NVSHMEMI_DEFINE_AMO_FETCH_SET_SWAP_HOST
+
+#define NVSHMEMI_DEFINE_AMO_ARITH_HOST(NAME, TYPE)                                                \
+    TYPE nvshmem_##NAME##_atomic_compare_swap(TYPE *target, TYPE cond, TYPE value, int pe) {      \
+        return host_amo<TYPE>("nvshmem_" #NAME "_atomic_compare_swap", NVSHMEMI_AMO_COMPARE_SWAP, target, value, cond, pe); \
+    }                                                                                             \
+    TYPE nvshmem_##NAME##_atomic_fetch_add(TYPE *target, TYPE value, int pe) {                    \
+        return host_amo<TYPE>("nvshmem_" #NAME "_atomic_fetch_add", NVSHMEMI_AMO_FETCH_ADD, target, value, (TYPE)0, pe); \
+    }                                                                                             \
+    void nvshmem_##NAME##_atomic_add(TYPE *target, TYPE value, int pe) {                          \
+        (void)host_amo<TYPE>("nvshmem_" #NAME "_atomic_add", NVSHMEMI_AMO_FETCH_ADD, target, value, (TYPE)0, pe); \
+    }                                                                                             \
+    TYPE nvshmem_##NAME##_atomic_fetch_inc(TYPE *target, int pe) {                                \
+        return host_amo<TYPE>("nvshmem_" #NAME "_atomic_fetch_inc", NVSHMEMI_AMO_FETCH_ADD, target, (TYPE)1, (TYPE)0, pe); \
+    }                                                                                             \
+    void nvshmem_##NAME##_atomic_inc(TYPE *target, int pe) {                                      \
+        (void)host_amo<TYPE>("nvshmem_" #NAME "_atomic_inc", NVSHMEMI_AMO_FETCH_ADD, target, (TYPE)1, (TYPE)0, pe); \
+    }
+NVSHMEMI_REPT_FOR_STANDARD_AMO_TYPES(NVSHMEMI_DEFINE_AMO_ARITH_HOST)
+#undef NVSHMEMI_DEFINE_AMO_ARITH_HOST
+
+#define NVSHMEMI_DEFINE_AMO_BITWISE_HOST(NAME, TYPE)                                              \
+    TYPE nvshmem_##NAME##_atomic_fetch_and(TYPE *target, TYPE value, int pe) {                    \
+        return host_amo<TYPE>("nvshmem_" #NAME "_atomic_fetch_and", NVSHMEMI_AMO_FETCH_AND, target, value, (TYPE)0, pe); \
+    }                                                                                             \
+    TYPE nvshmem_##NAME##_atomic_fetch_or(TYPE *target, TYPE value, int pe) {                     \
+        return host_amo<TYPE>("nvshmem_" #NAME "_atomic_fetch_or", NVSHMEMI_AMO_FETCH_OR, target, value, (TYPE)0, pe); \
+    }                                                                                             \
+    TYPE nvshmem_##NAME##_atomic_fetch_xor(TYPE *target, TYPE value, int pe) {                    \
+        return host_amo<TYPE>("nvshmem_" #NAME "_atomic_fetch_xor", NVSHMEMI_AMO_FETCH_XOR, target, value, (TYPE)0, pe); \
+    }                                                                                             \
+    void nvshmem_##NAME##_atomic_and(TYPE *target, TYPE value, int pe) {                          \
+        (void)host_amo<TYPE>("nvshmem_" #NAME "_atomic_and", NVSHMEMI_AMO_FETCH_AND, target, value, (TYPE)0, pe); \
+    }                                                                                             \
+    void nvshmem_##NAME##_atomic_or(TYPE *target, TYPE value, int pe) {                           \
+        (void)host_amo<TYPE>("nvshmem_" #NAME "_atomic_or", NVSHMEMI_AMO_FETCH_OR, target, value, (TYPE)0, pe); \
+    }                                                                                             \
+    void nvshmem_##NAME##_atomic_xor(TYPE *target, TYPE value, int pe) {                          \
+        (void)host_amo<TYPE>("nvshmem_" #NAME "_atomic_xor", NVSHMEMI_AMO_FETCH_XOR, target, value, (TYPE)0, pe); \
+    }
+NVSHMEMI_REPT_FOR_BITWISE_AMO_TYPES(NVSHMEMI_DEFINE_AMO_BITWISE_HOST)
+#undef NVSHMEMI_DEFINE_AMO_BITWISE_HOST
 
 }  // extern "C"

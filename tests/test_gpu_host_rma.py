@@ -104,3 +104,106 @@ def test_host_typed_sized_strided_rma_and_waits():
         flag, rec = rt.read_timeout(0)
         assert flag == 1 and rec[2] == 0xFFFFFFFB and rec[3] == 5      # found (uint)-5, expected 5
         s.destroy()
+
+
+def test_wait_until_all_vector_on_stream():
+    with runtime(NPES, 1 << 20) as rt:
+        lib = rt.lib
+        s = hip.Stream()
+        flags = rt.calloc(4, 8); values = rt.malloc(32); status = rt.malloc(16)
+        rt.upload(flags, 0, np.array([3, 10, -2, 99], np.int64))
+        rt.upload(values, 0, np.array([3, 11, -2, 5], np.int64))       # element 1 does not match ...
+        rt.upload(status, 0, np.array([0, 1, 0, 0], np.int32))         # ... and is excluded
+        wait = _fn(lib, "nvshmemx_int64_wait_until_all_vector_on_stream", None, [vp, sz, vp, i32, vp, vp])
+        note("int64 wait_until_all_vector_on_stream GE")
+        wait(flags, 4, status, N.CMP["GE"], values, s.ptr)
+        s.synchronize()
+        assert rt.read_timeout(0)[0] == 0
+        # without the exclusion the wait on element 1 runs into the spin limit and is recorded
+        rt.lib.nvshmemx_amd_set_spin_limit(100)
+        wait(flags, 4, None, N.CMP["GE"], values, s.ptr)
+        s.synchronize()
+        rt.lib.nvshmemx_amd_set_spin_limit(1 << 22)
+        flag, rec = rt.read_timeout(0)
+        assert flag == 1 and rec[2] == 10 and rec[3] == 11
+        wait(flags, 4, None, 17, values, s.ptr)
+        assert b"unknown comparison" in lib.nvshmemx_amd_last_error()
+        wait(flags, 4, None, N.CMP["GE"], None, s.ptr)
+        assert b"cmp_values is NULL" in lib.nvshmemx_amd_last_error()
+        s.destroy()
+
+
+AMO_BITWISE = [("uint", 32), ("ulong", 64), ("ulonglong", 64), ("int32", 32), ("int64", 64),
+               ("uint32", 32), ("uint64", 64)]
+AMO_STANDARD = AMO_BITWISE + [("int", 32), ("long", 64), ("longlong", 64), ("size", 64), ("ptrdiff", 64)]
+SIGNED = {"int32", "int64", "int", "long", "longlong", "ptrdiff"}
+
+
+def _ctype(name, bits):
+    if name in ("float", "double"):
+        return C.c_float if bits == 32 else C.c_double
+    if name in SIGNED:
+        return C.c_int32 if bits == 32 else C.c_int64
+    return C.c_uint32 if bits == 32 else C.c_uint64
+
+
+def test_host_atomics_every_name_against_the_oracle():
+    """The blocking host forms apply the same operations as the device forms: compare the word left
+    behind and the value returned with the oracle's integer model, on a remote PE."""
+    rng = np.random.default_rng(77)
+    with runtime(NPES, 1 << 20) as rt:
+        lib = rt.lib
+        word = rt.calloc(1, 8)
+        count = 0
+
+        def check(name, bits, op, cond_kind=None):
+            nonlocal count
+            ct = _ctype(name, bits)
+            mask = 2**bits - 1
+            pe = 1 + count % (NPES - 1)
+            init = int(rng.integers(0, 2**64, dtype=np.uint64))
+            value = int(rng.integers(0, 2**64, dtype=np.uint64))
+            cond = (init & mask) if cond_kind == "hit" else ((init ^ 1) & mask)
+            rt.upload(word, pe, np.array([init], np.uint64))
+            fname = "nvshmem_" + name + "_atomic_" + op
+            fetching = op in ("fetch", "swap", "compare_swap", "fetch_add", "fetch_inc", "fetch_and",
+                              "fetch_or", "fetch_xor")
+            args = {"fetch": [], "inc": [], "fetch_inc": [], "compare_swap": [ct, ct]}.get(op, [ct])
+            f = _fn(lib, fname, ct if fetching else None, [vp] + args + [i32])
+
+            def as_c(v):   # the low `bits` bits as a value of the C type
+                v &= mask
+                if ct in (C.c_int32, C.c_int64) and v >> (bits - 1):
+                    v -= 1 << bits
+                return v
+            call = [word] + ([as_c(cond), as_c(value)] if op == "compare_swap" else [as_c(value)] * len(args)) + [pe]
+            got = f(*call)
+            new, fetched = O.amo(op, bits, init, value, cond)
+            left = int(rt.download(word, pe, (1,), np.uint64)[0])
+            assert left == (init & ~mask) | new, (fname, cond_kind, hex(init), hex(value))
+            if fetching:
+                assert (int(got) & mask) == fetched, (fname, cond_kind)
+            count += 1
+
+        for name, bits in AMO_STANDARD:
+            for op in ("fetch", "set", "swap", "fetch_add", "add", "fetch_inc", "inc"):
+                check(name, bits, op)
+            check(name, bits, "compare_swap", "hit")
+            check(name, bits, "compare_swap", "miss")
+        for name, bits in AMO_BITWISE:
+            for op in ("fetch_and", "and", "fetch_or", "or", "fetch_xor", "xor"):
+                check(name, bits, op)
+        assert count == 12 * 9 + 7 * 6
+        # float / double: fetch, set, swap move the bits unchanged
+        for name, ct, npt in (("float", C.c_float, np.float32), ("double", C.c_double, np.float64)):
+            fword = rt.calloc(1, 8)
+            amo_name = lambda op: "nvshmem_" + name + "_atomic_" + op
+            _fn(lib, amo_name("set"), None, [vp, ct, i32])(fword, 1.5, 2)
+            assert _fn(lib, amo_name("fetch"), ct, [vp, i32])(fword, 2) == 1.5
+            assert _fn(lib, amo_name("swap"), ct, [vp, ct, i32])(fword, -0.25, 2) == 1.5
+            assert rt.download(fword, 2, (1,), npt)[0] == npt(-0.25)
+            assert rt.download(fword, 1, (1,), npt)[0] == 0
+        # errors are reported, not executed
+        f = _fn(lib, "nvshmem_int_atomic_fetch_add", C.c_int32, [vp, C.c_int32, i32])
+        assert f(word, 1, NPES) == 0 and b"outside" in lib.nvshmemx_amd_last_error()
+        assert f(word + 2, 1, 1) == 0 and b"aligned" in lib.nvshmemx_amd_last_error()
