@@ -408,5 +408,30 @@ NVSHMEMI_STAMP_MEM_COLL(nvshmemx, _block, NVSHMEMI_THREADGROUP_BLOCK)
 NVSHMEMI_REPT_FOR_ALL_REDUCE_TYPES_AND_OPS(NVSHMEMI_STAMP_REDUCE)
 #undef NVSHMEMI_STAMP_REDUCE
 
+/* (value, location) maximum, block scope only (reference nvshmemx_coll_defines.cuh:210-214) */
+NVSHMEMI_DEV int nvshmemx_double2_maxloc_reduce_block(nvshmem_team_t team, double2 *dest,
+                                                      const double2 *source, size_t nreduce) {
+    return nvshmemi_double2_maxloc_reduce_block(team, dest, source, nreduce);
+}
+
+/* ---- library identification from device code (reference nvshmem_defines.h:63-77) ---- */
+NVSHMEMI_DEV void nvshmem_info_get_version(int *major, int *minor) {
+    if (major) *major = NVSHMEM_MAJOR_VERSION;
+    if (minor) *minor = NVSHMEM_MINOR_VERSION;
+}
+/* name receives at most NVSHMEM_MAX_NAME_LEN bytes including the terminator */
+NVSHMEMI_DEV void nvshmem_info_get_name(char *name) {
+    static constexpr char vendor[] = NVSHMEM_VENDOR_STRING;
+    constexpr size_t len = sizeof(vendor) < NVSHMEM_MAX_NAME_LEN ? sizeof(vendor) : NVSHMEM_MAX_NAME_LEN;
+    if (!name) return;
+    for (size_t k = 0; k + 1 < len; ++k) name[k] = vendor[k];
+    name[len - 1] = 0;
+}
+NVSHMEMI_DEV void nvshmemx_vendor_get_version_info(int *major, int *minor, int *patch) {
+    if (major) *major = NVSHMEM_VENDOR_MAJOR_VERSION;
+    if (minor) *minor = NVSHMEM_VENDOR_MINOR_VERSION;
+    if (patch) *patch = NVSHMEM_VENDOR_PATCH_VERSION;
+}
+
 #undef NVSHMEMI_DEV
 #endif

@@ -1211,4 +1211,74 @@ NVSHMEMI_DEVICE_INLINE int nvshmemi_reducescatter_threadgroup(nvshmem_team_t tea
     return 0;
 }
 
+/* maxloc on (value, location) pairs (reference reduce.cuh:107-111 and :1718-1751): every member's
+ * dest[i] = fold over the members 0..n-1 of source[i], acc = (acc.x > x.x) ? acc : x - the order of the
+ * reference's rooted flat reduce, whose result all members then share: on equal values the later
+ * member wins, and a NaN met as x replaces acc.  The reference takes one element per call; any
+ * nreduce is served here.  Every member folds all elements itself and writes only its own dest. */
+NVSHMEMI_DEVICE_INLINE int nvshmemi_double2_maxloc_reduce_block(nvshmem_team_t team, double2 *dest,
+                                                               const double2 *source, size_t nreduce) {
+    constexpr int SCOPE = NVSHMEMI_THREADGROUP_BLOCK;
+    const nvshmemi_amd_team_view_t tv = nvshmemi_amd_team_view(team);
+    if (tv.size <= 0) return 1; /* the calling PE is not a member */
+    const size_t tid = (size_t)nvshmemi_thread_id_in_threadgroup<SCOPE>();
+    const size_t nthr = (size_t)nvshmemi_threadgroup_size<SCOPE>();
+    double2 *dst = reinterpret_cast<double2 *>(nvshmemi_amd_remote(dest, nvshmemi_amd_my_pe()));
+    /* One pair per PE, the reference's case: every member sends its pair to all others as two
+     * packets and folds what it receives.  Lane (j, p) of the first wavefront holds word j (0: value,
+     * 1: location) of member p, so the fold reads its operands across lanes instead of polling
+     * packet after packet. */
+    unsigned group = 1;
+    while ((int)group < tv.size) group <<= 1;
+    if (nreduce == 1 && 2 * group <= 64 && nthr >= 64 && nvshmemi_amd_ll_fits<SCOPE>(sizeof(double2), tv.size)) {
+        const int me = tv.my_pe;
+        const uint32_t flag = nvshmemi_amd_ll_next_flag<SCOPE>(team);
+        const char *src = nvshmemi_amd_local(source);
+        nvshmemi_amd_ll_send_to_all<SCOPE>(team, tv, src, sizeof(double2), 2, (unsigned)me * 2, flag);
+        nvshmemi_threadgroup_sync<SCOPE>(); /* dest may be source: sent before the result is stored */
+        if (tid < 64) {
+            const char *mine = nvshmemi_amd_ll_buffer(team, nvshmemi_amd_my_pe(), flag);
+            const unsigned gshift = 31u - (unsigned)__builtin_clz(group);
+            const unsigned j = (unsigned)tid >> gshift, p = (unsigned)tid & (group - 1);
+            uint64_t v = 0;
+            if (j < 2 && (int)p < tv.size)
+                v = (int)p == me ? nvshmemi_amd_ll_load_payload(src + 8 * (size_t)j, 8)
+                                 : nvshmemi_amd_ll_recv_packet(mine + ((size_t)p * 2 + j) * 16, flag);
+            uint64_t best_v = 0, best_l = 0;
+            for (int q = 0; q < tv.size; ++q) {
+                const uint64_t xv = (uint64_t)__shfl((unsigned long long)v, q, 64);
+                const uint64_t xl = (uint64_t)__shfl((unsigned long long)v, (int)group + q, 64);
+                double a, b;
+                __builtin_memcpy(&a, &best_v, 8);
+                __builtin_memcpy(&b, &xv, 8);
+                if (q == 0 || !(a > b)) {
+                    best_v = xv;
+                    best_l = xl;
+                }
+            }
+            if (tid == 0) {
+                nvshmemi_amd_ll_store_payload(reinterpret_cast<char *>(dst), best_v, 8);
+                nvshmemi_amd_ll_store_payload(reinterpret_cast<char *>(dst) + 8, best_l, 8);
+            }
+        }
+        nvshmemi_amd_ll_publish_done<SCOPE>(team, flag);
+        return 0;
+    }
+    /* every PE's source is complete and visible before anyone reads it */
+    nvshmemi_barrier_threadgroup<SCOPE>(team);
+    const double2 *src0 = reinterpret_cast<const double2 *>(nvshmemi_amd_remote(source, tv.start));
+    const size_t pe_stride = (size_t)(nvshmemi_device_state_d.heap_size / sizeof(double2)) * (size_t)tv.stride;
+    for (size_t i = tid; i < nreduce; i += nthr) {
+        double2 acc = src0[i];
+        for (int pe = 1; pe < tv.size; ++pe) {
+            const double2 x = src0[(size_t)pe * pe_stride + i];
+            acc = (acc.x > x.x) ? acc : x;
+        }
+        dst[i] = acc;
+    }
+    /* nobody may overwrite its source before every member has read it */
+    nvshmemi_barrier_threadgroup<SCOPE>(team);
+    return 0;
+}
+
 #endif

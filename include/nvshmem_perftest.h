@@ -153,6 +153,14 @@ int nvshmem_perftest_device_team_coll(int what, int team, void *dest, const void
 int nvshmem_perftest_device_team_coll_loop(int what, int team, void *dest, const void *src,
                                            size_t n, int root, int iters, int scope, int threads,
                                            void *stream);
+/* One block of `threads` per PE calls nvshmemx_double2_maxloc_reduce_block(team, dest, src, nreduce)
+ * `iters` times (perftest/device/coll/redmaxloc_latency.cu); dest and src hold nreduce (value,
+ * location) pairs of doubles.  With info != NULL (4 ints, symmetric) thread 0 of every PE also
+ * records what the device-side nvshmem_info_get_version, nvshmemx_vendor_get_version_info
+ * (major * 10000 + minor * 100 + patch) and nvshmem_info_get_name (length of the name) report. */
+int nvshmem_perftest_device_maxloc(int team, void *dest, const void *src, size_t nreduce, int iters,
+                                   int threads, int *info, void *stream);
+
 /* Every PE writes into its copy of `out` (4 + 64 ints): team_my_pe(a), team_n_pes(a),
  * team_my_pe(b), team_n_pes(b), then team_translate_pe(a, i, b) for i = 0..63, all evaluated in
  * device code. */

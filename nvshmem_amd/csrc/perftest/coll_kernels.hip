@@ -101,6 +101,27 @@ __global__ void team_coll_kernel(int what, nvshmem_team_t team, void *dest, cons
     }
 }
 
+// (value, location) maximum among the members of `team`, `iters` times; thread 0 of every PE also
+// stores what the device-side identification calls report into info[0..3] (major, minor of the
+// specification, then vendor major * 10000 + minor * 100 + patch, then the length of the name).
+__global__ void maxloc_kernel(nvshmem_team_t team, double2 *dest, const double2 *src, size_t n, int iters,
+                              int *info) {
+    if (threadIdx.x == 0 && info) {
+        int *mine = (int *)nvshmem_ptr(info, nvshmem_my_pe());
+        int major = 0, minor = 0, patch = 0;
+        nvshmem_info_get_version(&mine[0], &mine[1]);
+        nvshmemx_vendor_get_version_info(&major, &minor, &patch);
+        mine[2] = major * 10000 + minor * 100 + patch;
+        char name[NVSHMEM_MAX_NAME_LEN];
+        nvshmem_info_get_name(name);
+        int len = 0;
+        while (len < NVSHMEM_MAX_NAME_LEN && name[len]) ++len;
+        mine[3] = len;
+    }
+    if (nvshmem_team_my_pe(team) < 0) return;
+    for (int it = 0; it < iters; ++it) nvshmemx_double2_maxloc_reduce_block(team, dest, src, n);
+}
+
 // out (symmetric, 4 + NVSHMEMI_AMD_MAX_PES ints per PE): my_pe(a), n_pes(a), my_pe(b), n_pes(b),
 // then translate_pe(a, i, b) for i = 0 .. NVSHMEMI_AMD_MAX_PES-1
 __global__ void team_query_kernel(int *out, nvshmem_team_t a, nvshmem_team_t b) {
@@ -323,6 +344,21 @@ int nvshmem_perftest_device_team_coll(int what, int team, void *dest, const void
     if (what == kTeamBarrier) return NVSHMEMX_ERROR_INVALID_VALUE;
     return nvshmem_perftest_device_team_coll_loop(what, team, dest, src, n, root, 1, scope, threads,
                                                   stream);
+}
+
+int nvshmem_perftest_device_maxloc(int team, void *dest, const void *src, size_t nreduce, int iters,
+                                   int threads, int *info, void *stream) {
+    if (!perftest::ready() || iters < 1 || !perftest::check_launch(1, threads) ||
+        !perftest::check_range(dest, nreduce * sizeof(double2)) ||
+        !perftest::check_range(src, nreduce * sizeof(double2)) ||
+        (info && !perftest::check_range(info, 4 * sizeof(int))))
+        return NVSHMEMX_ERROR_INVALID_VALUE;
+    nvshmem_team_t t = team;
+    double2 *d = (double2 *)dest;
+    const double2 *s = (const double2 *)src;
+    void *args[] = {(void *)&t, (void *)&d, (void *)&s, (void *)&nreduce, (void *)&iters, (void *)&info};
+    return nvshmemx_collective_launch((const void *)maxloc_kernel, dim3(1), dim3(threads), args, 0,
+                                      (hipStream_t)stream);
 }
 
 int nvshmem_perftest_team_query(int *out, int team_a, int team_b, void *stream) {

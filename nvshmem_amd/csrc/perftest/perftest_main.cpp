@@ -233,6 +233,11 @@ int run_device_latency(const Options &o, bool barrier_only) {
             for (size_t bytes : sizes) us.push_back(latency_us(c.what, c.what <= 1 ? bytes / 4 : bytes));
             print_table(c.job, scope_name(o.scope), "latency", "us", sizes, us);
         }
+        // (value, location) maximum of one pair per PE, block scope (redmaxloc_latency.cu)
+        auto maxloc = [&](int k) { return nvshmem_perftest_device_maxloc(NVSHMEM_TEAM_WORLD, dst, src, 1, k, threads, nullptr, nullptr); };
+        const double t1 = time_ms([&] { return maxloc(1); }, 5, 2), tk = time_ms([&] { return maxloc(o.iters + 1); }, 5, 2);
+        printf("#redmaxloc_latency\n%-10s  %-8s  %-16s\n%-10d  %-8s  %-16.6f\n", "size(B)", "scope", "latency (us)", 16,
+               "block", (tk - t1) * 1e3 / o.iters);
     }
     nvshmem_free(src);
     nvshmem_free(dst);

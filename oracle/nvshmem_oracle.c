@@ -339,6 +339,27 @@ int oracle_reducescatter(int dtype, int op, int npes, size_t nelems, const void 
     return 0;
 }
 
+/* maxloc over (value, location) pairs: operator reference src/include/non_abi/device/coll/reduce.cuh:107-111
+ * `(op1.x > op2.x) ? op1 : op2`, folded as in the rooted flat reduce (:1738-1747): acc = source of
+ * member 0, then acc = op(acc, source of member i) for i = 1..n-1; all members receive the result.
+ * src is [npes][nelems][2] doubles, dst likewise. */
+void oracle_maxloc_reduce(int npes, size_t nelems, const double *src, double *dst) {
+    for (size_t k = 0; k < nelems; ++k) {
+        double v = src[2 * k], loc = src[2 * k + 1];
+        for (int p = 1; p < npes; ++p) {
+            const double *x = src + ((size_t)p * nelems + k) * 2;
+            if (!(v > x[0])) {
+                v = x[0];
+                loc = x[1];
+            }
+        }
+        for (int q = 0; q < npes; ++q) {
+            dst[((size_t)q * nelems + k) * 2] = v;
+            dst[((size_t)q * nelems + k) * 2 + 1] = loc;
+        }
+    }
+}
+
 /* broadcast: reference src/include/non_abi/device/coll/broadcast.cuh:276-337 (every PE's dest gets
  * the root's source; the root copies too when dest != source, :97) */
 void oracle_broadcast(int npes, size_t bytes, int root, const uint8_t *src, uint8_t *dst) {

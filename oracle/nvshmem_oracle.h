@@ -91,6 +91,10 @@ void oracle_alltoall(int npes, size_t seg_bytes, const uint8_t *src, uint8_t *ds
  * p >= 2 (operands the other way round than in oracle_reduce); src is [npes][npes*nelems], dst is
  * [npes][nelems].  Returns 0, or -1 when op is not defined for dtype. */
 int oracle_reducescatter(int dtype, int op, int npes, size_t nelems, const void *src, void *dst);
+/* (value, location) maximum: dst[q][k] = fold over p = 0..npes-1 of src[p][k] with
+ * acc = (acc.value > x.value) ? acc : x (equal values: the later PE wins; a NaN x replaces acc);
+ * src and dst are [npes][nelems][2] doubles */
+void oracle_maxloc_reduce(int npes, size_t nelems, const double *src, double *dst);
 /* dst[q][k] = src[root][k] for every q including the root; src, dst are [npes][bytes] */
 void oracle_broadcast(int npes, size_t bytes, int root, const uint8_t *src, uint8_t *dst);
 

@@ -51,6 +51,7 @@ def lib():
         "oracle_ptr": (u64, [u64, u64, i32, u64, i32]),
         "oracle_reduce": (i32, [i32, i32, i32, sz, vp, vp]),
         "oracle_reducescatter": (i32, [i32, i32, i32, sz, vp, vp]),
+        "oracle_maxloc_reduce": (None, [i32, sz, vp, vp]),
         "oracle_broadcast": (None, [i32, sz, i32, vp, vp]),
         "oracle_amo": (C.c_uint64, [i32, i32, C.c_uint64, C.c_uint64, C.c_uint64, vp]),
         "oracle_team_split_strided": (i32, [vp, i32, i32, i32, i32, vp]),
@@ -127,6 +128,14 @@ def reducescatter(dtype, op, src):
     rc = lib().oracle_reducescatter(DT[dtype], OP[op], npes, n, _p(src), _p(out))
     if rc != 0:
         raise ValueError("oracle_reducescatter: %s/%s undefined" % (dtype, op))
+    return out
+
+
+def maxloc_reduce(src):
+    """src: [npes, n, 2] float64 (value, location) -> [npes, n, 2]."""
+    src = np.ascontiguousarray(src, dtype=np.float64)
+    out = np.empty_like(src)
+    lib().oracle_maxloc_reduce(src.shape[0], src.shape[1], _p(src), _p(out))
     return out
 
 

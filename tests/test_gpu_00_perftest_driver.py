@@ -56,6 +56,7 @@ def test_device_latency_tables():
         rows = _rows(out, job)
         assert [r[0] for r in rows] == [8, 16, 32, 64, 128, 256, 512] and all(r[1] == "warp" for r in rows)
         assert all(0.0 < v < 1000.0 for _, _, v in rows), (job, rows)
+    assert 0.0 < _rows(out, "redmaxloc_latency")[0][2] < 1000.0
     out = _run("barrier_latency", "--iters", "100")
     assert "barrier_latency" in out
 

@@ -104,7 +104,7 @@ def test_init_rejects_bad_team_sizes():
     assert lib.nvshmemx_init_status() == 0
 
 
-@pytest.mark.parametrize("npes", [1, 2, 3, 16, 24])
+@pytest.mark.parametrize("npes", [1, 2, 3, 16, 24, 32, 33, 64])
 def test_broadcast_and_reducescatter_on_other_team_sizes(npes):
     rng = np.random.default_rng(npes)
     n = 2052
@@ -125,6 +125,14 @@ def test_broadcast_and_reducescatter_on_other_team_sizes(npes):
         got = rt.download_all(dst, (n * 4 - 7,), np.uint8, 1)
         want = idata.view(np.uint8)[root, 3:3 + n * 4 - 7]
         assert all(np.array_equal(got[pe], want) for pe in range(npes))
+        # (value, location) maximum of one pair per PE: packets up to 32 PEs, barriers beyond
+        pairs = np.stack([rng.integers(0, 3, (npes, 1)).astype(np.float64),
+                          np.arange(npes, dtype=np.float64)[:, None]], axis=2)
+        rt.upload_all(src, pairs)
+        note("npes=%d maxloc" % npes)
+        assert rt.perftest().nvshmem_perftest_device_maxloc(N.TEAM_WORLD, dst, src, 1, 3, 128, None, None) == 0
+        rt.sync()
+        assert bits_equal(rt.download_all(dst, (1, 2), np.float64), O.maxloc_reduce(pairs))
         rt.free(src); rt.free(dst)
 
 
@@ -163,5 +171,10 @@ def test_small_in_kernel_collectives_with_and_without_packets(disable, plain, mo
             assert perf.nvshmem_perftest_device_broadcast(dst, src, n * 4, rep % 8, N.SCOPE_THREAD, 64, None) == 0
             rt.sync()
             assert all(np.array_equal(rt.download(dst, pe, (n * 4,), np.uint8), raw[rep % 8, :n * 4]) for pe in range(8))
+            pairs = data[:, :2].astype(np.float64).reshape(8, 1, 2)
+            rt.upload_all(src, pairs)
+            assert perf.nvshmem_perftest_device_maxloc(N.TEAM_WORLD, dst, src, 1, 2, 64, None, None) == 0
+            rt.sync()
+            assert bits_equal(rt.download_all(dst, (1, 2), np.float64), O.maxloc_reduce(pairs))
         assert rt.read_timeout(0)[0] == 0
         rt.free(src); rt.free(dst)

@@ -348,6 +348,47 @@ def test_device_scope_collectives_on_teams(rt, scope, threads, n):
         rt.team_destroy(t)
 
 
+def test_maxloc_reduce_and_device_identification(rt):
+    """nvshmemx_double2_maxloc_reduce_block on the world team, a strided team and the rows of a 2-D
+    split, with ties and NaNs in the values; plus what the device-side identification calls report."""
+    perf = rt.perftest()
+    rng = np.random.default_rng(61)
+    x, y = rt.team_split_2d(N.TEAM_WORLD, 4)
+    odd = rt.team_split_strided(N.TEAM_WORLD, 1, 2, 8)
+    want2d = [O.team_split_2d(WORLD, 4, pe) for pe in range(NPES)]
+    cases = [(N.TEAM_WORLD, [WORLD] * NPES), (x, [w[0] for w in want2d]),
+             (odd, [(1, 2, 8) if pe % 2 else None for pe in range(NPES)])]
+    nmax = 70
+    src = rt.malloc(nmax * 16); dst = rt.malloc(nmax * 16); info = rt.calloc(4, 4)
+    for team, members_of in cases:
+        for n, threads in ((1, 64), (nmax, 256)):
+            pairs = np.empty((NPES, n, 2))
+            pairs[:, :, 0] = rng.integers(-3, 4, (NPES, n))          # few distinct values: many ties
+            pairs[:, :, 1] = np.arange(NPES)[:, None] * 1000 + np.arange(n)[None, :]
+            pairs[rng.random((NPES, n)) < 0.1, 0] = np.nan
+            rt.upload_all(src, pairs)
+            rt.fill(dst, 0xCD, nmax * 16)
+            note("maxloc team=%d n=%d threads=%d" % (team, n, threads))
+            assert perf.nvshmem_perftest_device_maxloc(team, dst, src, n, 2, threads, info, None) == 0
+            rt.sync()
+            for g in _groups(members_of):
+                members = O.team_members(g)
+                want = O.maxloc_reduce(pairs[members])
+                for i, pe in enumerate(members):
+                    assert bits_equal(rt.download(dst, pe, (n, 2), np.float64), want[i]), (team, g, pe, n)
+            for pe in range(NPES):
+                if members_of[pe] is None:
+                    assert (rt.download(dst, pe, (n * 4,), np.uint32) == 0xCDCDCDCD).all()
+    got = rt.download_all(info, (4,), np.int32)
+    name = C.create_string_buffer(256)
+    rt.lib.nvshmem_info_get_name(name)
+    assert (got == np.array([1, 3, 30501, len(name.value)], np.int32)).all(), got
+    assert perf.nvshmem_perftest_device_maxloc(N.TEAM_WORLD, dst, src, 1 << 40, 1, 64, None, None) != 0
+    rt.team_destroy(x); rt.team_destroy(y); rt.team_destroy(odd)
+    for p in (src, dst, info):
+        rt.free(p)
+
+
 def test_a_reused_handle_starts_clean(rt):
     """Packet flags and barrier epochs restart when a handle is reused by other members."""
     perf = rt.perftest()

@@ -468,3 +468,31 @@ def test_amo_semantics_against_python_integers():
     assert O.amo("fetch_add", 32, 0xFFFFFFFF, 2) == (1, 0xFFFFFFFF)
     assert O.amo("inc", 64, 2**64 - 1) == (0, 2**64 - 1)
     assert O.amo("compare_swap", 64, 5, 9, 4) == (5, 5) and O.amo("compare_swap", 64, 5, 9, 5) == (9, 5)
+
+
+def test_maxloc_reduce_is_argmax_with_later_pe_winning_ties():
+    # operator (a.x > b.x) ? a : b folded from PE 0 upwards (reduce.cuh:107-111, :1738-1747)
+    rng = np.random.default_rng(21)
+    npes, n = 7, 300
+    vals = rng.standard_normal((npes, n))
+    locs = rng.integers(0, 1 << 20, (npes, n)).astype(np.float64)
+    got = O.maxloc_reduce(np.stack([vals, locs], axis=2))
+    win = vals.argmax(axis=0)                                   # distinct values: plain argmax
+    for q in range(npes):
+        assert np.array_equal(got[q, :, 0], vals.max(axis=0))
+        assert np.array_equal(got[q, :, 1], locs[win, np.arange(n)])
+    # equal values: the pair of the LAST PE holding the maximum comes out
+    tie = np.array([[[5.0, 10.0]], [[7.0, 11.0]], [[7.0, 12.0]], [[3.0, 13.0]]])
+    assert np.array_equal(O.maxloc_reduce(tie)[0, 0], [7.0, 12.0])
+    # signed zeros compare equal: the later one wins, with its sign
+    z = np.array([[[0.0, 1.0]], [[-0.0, 2.0]]])
+    out = O.maxloc_reduce(z)[1, 0]
+    assert out[1] == 2.0 and np.signbit(out[0])
+    # NaN: a NaN met as the new operand replaces the accumulator, and is dropped by the next one
+    nan = float("nan")
+    def fold(values):
+        return O.maxloc_reduce(np.array([[[v, float(i)]] for i, v in enumerate(values)]))[0, 0]
+    assert np.isnan(fold([1.0, 2.0, nan])[0]) and fold([1.0, 2.0, nan])[1] == 2.0
+    assert np.array_equal(fold([nan, 1.0, 2.0]), [2.0, 2.0])
+    assert np.array_equal(fold([1.0, nan, 0.0]), [0.0, 2.0])
+    assert np.array_equal(fold([4.0]), [4.0, 0.0])              # a single PE: its own pair
