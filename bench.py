@@ -32,7 +32,7 @@ MEASURED_TRAFFIC_BYTES = {
     "sum_reduce": (2048 + 2048) << 20,   # profiles/reduce_vector_kernel_float_sum_8pe_64Mi.txt
     "alltoall": (256 + 256) << 20,       # profiles/segment_copy_kernel_alltoall_16pe_4Mi_fp32.txt
     "alltoall_1GiB": None,              # not profiled
-    "reducescatter": (2048 + 256) << 20,  # profiles/reduce_vector_kernel_float_sum_reducescatter_8pe_8Mi.txt
+    "reducescatter": (2048 + 256) << 20,  # profiles/reducescatter_gather_kernel_float_sum_8pe_8Mi.txt
     "broadcast": (256 + 2048) << 20,      # profiles/segment_copy_kernel_broadcast_8pe_256MiB.txt
 }
 
@@ -230,7 +230,7 @@ def bench_reducescatter(N, O, hip, np, steps, warmup, cpu_budget):
         "config": {"workload": "reducescatter: nvshmemx_float_sum_reducescatter_on_stream, 8 logical PEs, "
                                "source 8 x 2^23 fp32 (256 MiB) per PE, result 2^23 fp32 per PE",
                    "npes": npes, "nreduce": n},
-        "kernel": "reduce_vector_kernel<float, sum, 8, scatter>",
+        "kernel": "reducescatter_gather_kernel<float, sum, 8>",
         "cpu_baseline": cpu,
     }
 

@@ -67,8 +67,8 @@ WORKLOADS = {
         "segment_copy_kernel_fcollect_16pe_4Mi_fp32.txt",
         "fcollect: nvshmemx_float_fcollect_on_stream, 16 logical PEs x 2^22 fp32.\n"
         "Algorithmic bytes per launch: 256 MiB read + 16 x 256 MiB written = 4.25 GiB.", (17 * 256) << 20),
-    "reduce_vector_kernel<float, 5, 8, true, true,": (
-        "reduce_vector_kernel_float_sum_reducescatter_8pe_8Mi.txt",
+    "reducescatter_gather_kernel<float, 5, 8, true>": (
+        "reducescatter_gather_kernel_float_sum_8pe_8Mi.txt",
         "reducescatter: nvshmemx_float_sum_reducescatter_on_stream, 8 logical PEs, source 8 x 2^23 fp32\n"
         "(256 MiB) per PE, result 2^23 fp32 (32 MiB) per PE.\n"
         "Algorithmic bytes per launch: 8 sources of 256 MiB read once + 8 results of 32 MiB written = 2.25 GiB.",
