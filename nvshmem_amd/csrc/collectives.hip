@@ -46,13 +46,11 @@ namespace {
 #ifndef NVSHMEM_AMD_COLL_NT /* bit 0: non-temporal loads allowed, bit 1: non-temporal stores */
 #define NVSHMEM_AMD_COLL_NT 3
 #endif
-/* Sources up to this many bytes (all PEs together) are loaded with the default, cacheable policy:
- * they fit the 256 MiB Infinity Cache, so a source that is sent again (or was just produced) is
- * served from it (measured +30 % on the 1M-element reduce, +20..45 % on 256 MiB collectives).
- * Larger sources are streamed with non-temporal loads (+5 % at 2 GiB).  Stores always stream. */
-#ifndef NVSHMEM_AMD_CACHEABLE_SOURCE_BYTES
-#define NVSHMEM_AMD_CACHEABLE_SOURCE_BYTES ((uint64_t)256 << 20)
-#endif
+/* Sources of up to Runtime::cacheable_source_bytes (all PEs together, 256 MiB unless the environment
+ * says otherwise) are loaded with the default, cacheable policy: they fit the 256 MiB Infinity
+ * Cache, so a source that is sent again (or was just produced) is served from it (measured +30 % on
+ * the 1M-element reduce, +20..45 % on 256 MiB collectives).  Larger sources are streamed with
+ * non-temporal loads (+5 % at 2 GiB).  Stores always stream. */
 
 constexpr int kThreads = NVSHMEM_AMD_COLL_THREADS;
 constexpr int kCopyThreads = NVSHMEM_AMD_COPY_THREADS;
@@ -85,7 +83,8 @@ enum { kModeFcollect = 0, kModeAlltoall = 1, kModeBroadcast = 2 };
 // the segment wrap to huge unsigned values and are skipped the same way as those behind it.
 template <bool SRC_ALIGNED, bool REPLICATE, int kCopyUnroll, bool NTL>
 __device__ __forceinline__ void copy_tile(char *__restrict__ dst, const char *__restrict__ src,
-                                          uint64_t v0, uint64_t nvec, uint64_t rep_stride, int nrep) {
+                                          uint64_t v0, uint64_t nvec, uint64_t rep_stride, int r0,
+                                          int r1) {
     nvshmemi_v4u v[kCopyUnroll];
 #pragma unroll
     for (int u = 0; u < kCopyUnroll; ++u) {
@@ -93,7 +92,7 @@ __device__ __forceinline__ void copy_tile(char *__restrict__ dst, const char *__
         if (i < nvec) v[u] = SRC_ALIGNED ? stream_load<NTL>(src + 16 * i) : nvshmemi_amd_load16<false>(src + 16 * i);
     }
     if (REPLICATE) {
-        for (int r = 0; r < nrep; ++r) {
+        for (int r = r0; r < r1; ++r) {
             char *d = dst + (uint64_t)r * rep_stride;
 #pragma unroll
             for (int u = 0; u < kCopyUnroll; ++u) {
@@ -115,7 +114,7 @@ __global__ __launch_bounds__(kCopyThreads) void segment_copy_kernel(char *base, 
                                                                 const nvshmemi_amd_team_view_t *groups,
                                                                 int max_size, uint64_t dst_off,
                                                                 uint64_t src_off, uint64_t seg_bytes,
-                                                                int root) {
+                                                                int root, uint32_t part_shift) {
     // this block's team: members are the PEs start + i*stride, i < size
     const nvshmemi_amd_team_view_t g = groups[blockIdx.z];
     const unsigned npes = (unsigned)g.size;
@@ -163,17 +162,21 @@ __global__ __launch_bounds__(kCopyThreads) void segment_copy_kernel(char *base, 
     // lie in front of the segment
     const uint64_t lead = ((uint64_t)(uintptr_t)(dst + head) >> 4) & 63;
     constexpr uint64_t kTileVectors = (uint64_t)kCopyThreads * kCopyUnroll;
-    const uint64_t v0 = (uint64_t)blockIdx.x * kTileVectors - lead;
+    // fcollect / broadcast: 2^part_shift consecutive blocks share a tile and split its destinations
+    const uint64_t v0 = (uint64_t)(blockIdx.x >> part_shift) * kTileVectors - lead;
     if ((int64_t)v0 >= (int64_t)nvec_total) return;
     const char *s = src + head;
     char *d = dst + head;
     const bool aligned = (((uintptr_t)s) & 15) == 0;
     if (MODE != kModeAlltoall) {
-        if (aligned) copy_tile<true, true, kCopyUnroll, NTL>(d, s, v0, nvec_total, rep_stride, nrep);
-        else copy_tile<false, true, kCopyUnroll, NTL>(d, s, v0, nvec_total, rep_stride, nrep);
+        const int per = (nrep + (1 << part_shift) - 1) >> part_shift;
+        const int r0 = (int)(blockIdx.x & ((1u << part_shift) - 1)) * per;
+        const int r1 = r0 + per < nrep ? r0 + per : nrep;
+        if (aligned) copy_tile<true, true, kCopyUnroll, NTL>(d, s, v0, nvec_total, rep_stride, r0, r1);
+        else copy_tile<false, true, kCopyUnroll, NTL>(d, s, v0, nvec_total, rep_stride, r0, r1);
     } else {
-        if (aligned) copy_tile<true, false, kCopyUnroll, NTL>(d, s, v0, nvec_total, rep_stride, 1);
-        else copy_tile<false, false, kCopyUnroll, NTL>(d, s, v0, nvec_total, rep_stride, 1);
+        if (aligned) copy_tile<true, false, kCopyUnroll, NTL>(d, s, v0, nvec_total, rep_stride, 0, 1);
+        else copy_tile<false, false, kCopyUnroll, NTL>(d, s, v0, nvec_total, rep_stride, 0, 1);
     }
 }
 
@@ -342,6 +345,21 @@ __global__ __launch_bounds__(kThreads) void reduce_scalar_kernel(char *base, uin
     }
 }
 
+// fcollect / broadcast of sources too large to stay in the Infinity Cache: a wavefront stores its
+// piece to at most four destinations; the blocks that share a piece are neighbours in the grid, so
+// all but the first find it in the L2.  Measured with random data: broadcast of 512 MiB to 8 PEs
+// 5.05 -> 6.03 TB/s, fcollect of 16 x 32 MiB 5.25 -> 6.10, of 8 x 64 MiB 5.55 -> 6.2; two or eight
+// destinations per wavefront are slower.  Cache-resident sources keep one wavefront per piece: the
+// split costs them up to 9 %.
+#ifndef NVSHMEM_AMD_REPLICAS_PER_WAVE
+#define NVSHMEM_AMD_REPLICAS_PER_WAVE 4
+#endif
+static uint32_t replica_part_shift(int max_size) {
+    uint32_t shift = 0;
+    while (((max_size + (1 << shift) - 1) >> shift) > NVSHMEM_AMD_REPLICAS_PER_WAVE) ++shift;
+    return shift;
+}
+
 // members of all teams of the handle together
 static uint64_t total_members(const TeamLaunch &tl) {
     // sizes lie between min and max; the exact sum only matters for the cache policy threshold
@@ -366,7 +384,7 @@ void launch_reduce(Runtime &rt, const TeamLaunch &tl, uint64_t dst_off, uint64_t
         const size_t lds = ((size_t)tl.max_size + 1) * 16 * tile_vecs;
         const dim3 grid((unsigned)blocks, 1, ngroups);
         const bool stream_source =
-            total_members(tl) * nelems * sizeof(T) > NVSHMEM_AMD_CACHEABLE_SOURCE_BYTES;
+            total_members(tl) * nelems * sizeof(T) > rt.cacheable_source_bytes;
 #define NVSHMEM_AMD_LAUNCH_REDUCE(N)                                                              \
     do {                                                                                          \
         if (stream_source)                                                                        \
@@ -410,7 +428,7 @@ void launch_reducescatter(Runtime &rt, const TeamLaunch &tl, uint64_t dst_off, u
         }
         const dim3 grid((unsigned)blocks, (unsigned)tl.max_size, ngroups);
         const bool stream_source =
-            total_members(tl) * tl.max_size * nelems * sizeof(T) > NVSHMEM_AMD_CACHEABLE_SOURCE_BYTES;
+            total_members(tl) * tl.max_size * nelems * sizeof(T) > rt.cacheable_source_bytes;
         const bool eight = tl.min_size == 8 && tl.max_size == 8;
 #define NVSHMEM_AMD_LAUNCH_GATHER(N, NTL)                                                         \
     hipLaunchKernelGGL((reducescatter_gather_kernel<T, OP, N, NTL>), grid, dim3(64), 0, stream,   \
@@ -434,7 +452,7 @@ void launch_reducescatter(Runtime &rt, const TeamLaunch &tl, uint64_t dst_off, u
         const size_t lds = ((size_t)tl.max_size + 1) * 16 * tile_vecs;
         const dim3 grid((unsigned)blocks, (unsigned)tl.max_size, ngroups);
         const bool stream_source =
-            total_members(tl) * tl.max_size * nelems * sizeof(T) > NVSHMEM_AMD_CACHEABLE_SOURCE_BYTES;
+            total_members(tl) * tl.max_size * nelems * sizeof(T) > rt.cacheable_source_bytes;
 #define NVSHMEM_AMD_LAUNCH_SCATTER(N, NTL)                                                        \
     hipLaunchKernelGGL((reduce_vector_kernel<T, OP, N, NTL, true, 1>), grid, dim3(threads), lds,  \
                        stream, rt.base, rt.heap_shift, tl.groups, lane_shift, dst_off, src_off,   \
@@ -601,20 +619,24 @@ int broadcast_on_stream(nvshmem_team_t team, void *dest, const void *src, size_t
         set_error("broadcast: dest and source overlap without being identical");
         return NVSHMEMX_ERROR_INVALID_VALUE;
     }
-    const uint64_t tiles = (bytes / 16 + 64 + kCopyThreads - 1) / kCopyThreads + 1;
+    // a source that cannot stay in the Infinity Cache: split the destinations (see replica_part_shift)
+    const bool big_source = bytes * (uint64_t)tl.ngroups > rt.cacheable_source_bytes;
+    const uint32_t part_shift = big_source ? replica_part_shift(tl.max_size) : 0;
+    const uint64_t tiles = ((bytes / 16 + 64 + kCopyThreads - 1) / kCopyThreads + 1) << part_shift;
     if (tiles > 0x7fffffffull) {
         set_error("broadcast: message too large");
         return NVSHMEMX_ERROR_INVALID_VALUE;
     }
     const dim3 grid((unsigned)tiles, 1, (unsigned)tl.ngroups), block(kCopyThreads);
-    if (bytes * (uint64_t)tl.ngroups > NVSHMEM_AMD_CACHEABLE_SOURCE_BYTES)
+    // blocks that share a piece re-read it from the cache, so the loads stay cacheable then
+    if (part_shift == 0 && big_source)
         hipLaunchKernelGGL((segment_copy_kernel<kModeBroadcast, 1, true>), grid, block, 0, stream,
                            rt.base, rt.heap_shift, tl.groups, tl.max_size, doff, soff,
-                           (uint64_t)bytes, root);
+                           (uint64_t)bytes, root, part_shift);
     else
         hipLaunchKernelGGL((segment_copy_kernel<kModeBroadcast, 1, false>), grid, block, 0, stream,
                            rt.base, rt.heap_shift, tl.groups, tl.max_size, doff, soff,
-                           (uint64_t)bytes, root);
+                           (uint64_t)bytes, root, part_shift);
     hipError_t e = hipGetLastError();
     if (e != hipSuccess) {
         set_error("broadcast: kernel launch failed: %s", hipGetErrorString(e));
@@ -646,17 +668,21 @@ static int segment_collective(int mode, const char *what, nvshmem_team_t team, v
     }
     const uint64_t tile_vectors = (uint64_t)kCopyThreads * (mode == kModeFcollect ? NVSHMEM_AMD_FCOLLECT_UNROLL
                                                                               : NVSHMEM_AMD_ALLTOALL_UNROLL);
-    const uint64_t tiles = (seg_bytes / 16 + 64 + tile_vectors - 1) / tile_vectors + 1;
+    const bool big_source = src_bytes * total_members(tl) > rt.cacheable_source_bytes;
+    const uint32_t part_shift = mode == kModeFcollect && big_source ? replica_part_shift(tl.max_size) : 0;
+    const uint64_t tiles = ((seg_bytes / 16 + 64 + tile_vectors - 1) / tile_vectors + 1) << part_shift;
     const unsigned segs = mode == kModeFcollect ? (unsigned)n : (unsigned)(n * n);
     if (tiles > 0x7fffffffull) {
         set_error("%s: message too large", what);
         return NVSHMEMX_ERROR_INVALID_VALUE;
     }
-    const bool stream_source = src_bytes * total_members(tl) > NVSHMEM_AMD_CACHEABLE_SOURCE_BYTES;
+    // blocks that share a piece re-read it from the cache, so the loads stay cacheable then
+    const bool stream_source = part_shift == 0 && big_source;
     const dim3 grid((unsigned)tiles, segs, (unsigned)tl.ngroups), block(kCopyThreads);
 #define NVSHMEM_AMD_LAUNCH_SEGCOPY(MODE, U, NTL)                                                   \
     hipLaunchKernelGGL((segment_copy_kernel<MODE, U, NTL>), grid, block, 0, stream, rt.base,       \
-                       rt.heap_shift, tl.groups, tl.max_size, doff, soff, (uint64_t)seg_bytes, 0)
+                       rt.heap_shift, tl.groups, tl.max_size, doff, soff, (uint64_t)seg_bytes, 0,  \
+                       part_shift)
     if (mode == kModeFcollect) {
         if (stream_source) NVSHMEM_AMD_LAUNCH_SEGCOPY(kModeFcollect, NVSHMEM_AMD_FCOLLECT_UNROLL, true);
         else NVSHMEM_AMD_LAUNCH_SEGCOPY(kModeFcollect, NVSHMEM_AMD_FCOLLECT_UNROLL, false);

@@ -194,6 +194,7 @@ int nvshmemx_amd_init(int npes, size_t symmetric_size) {
     rt.dev.timeout_record = (uint64_t *)(uintptr_t)trec;
     rt.dev.spin_limit = env_size("NVSHMEM_AMD_SPIN_LIMIT", 1ull << 22);
     rt.plain_collective_launch = env_size("NVSHMEM_AMD_PLAIN_COLLECTIVE_LAUNCH", 0) != 0;
+    rt.cacheable_source_bytes = env_size("NVSHMEM_AMD_CACHEABLE_SOURCE_BYTES", (size_t)256 << 20);
     if (!teams_init(rt)) {
         teams_finalize(rt);
         (void)hipFree(rt.base);

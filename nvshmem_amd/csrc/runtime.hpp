@@ -59,6 +59,9 @@ struct Runtime {
     std::set<nvshmemi_amd_state_updater_t> updaters;  // one per translation unit with a state block
     bool symbols_stale = false;
     bool plain_collective_launch = false;  // NVSHMEM_AMD_PLAIN_COLLECTIVE_LAUNCH=1, read at init
+    // Host-launched collectives treat sources of more bytes than this (all PEs together) as too
+    // large to stay in the Infinity Cache: NVSHMEM_AMD_CACHEABLE_SOURCE_BYTES, read at init
+    uint64_t cacheable_source_bytes = (uint64_t)256 << 20;
 
     static Runtime &get();
 

@@ -178,3 +178,47 @@ def test_small_in_kernel_collectives_with_and_without_packets(disable, plain, mo
             assert bits_equal(rt.download_all(dst, (1, 2), np.float64), O.maxloc_reduce(pairs))
         assert rt.read_timeout(0)[0] == 0
         rt.free(src); rt.free(dst)
+
+
+@pytest.mark.parametrize("npes", [3, 8, 13, 16])
+def test_large_source_policy_of_fcollect_and_broadcast(npes, monkeypatch):
+    """Sources beyond NVSHMEM_AMD_CACHEABLE_SOURCE_BYTES (read at init) are streamed, and fcollect /
+    broadcast then split the destinations of a piece over neighbouring blocks (at most four per
+    wavefront).  With the threshold at zero every size takes that path: ragged, misaligned messages
+    must come out the same, bytes outside the destination untouched."""
+    monkeypatch.setenv("NVSHMEM_AMD_CACHEABLE_SOURCE_BYTES", "0")
+    rng = np.random.default_rng(100 + npes)
+    with runtime(npes, 1 << 24) as rt:
+        cap = 1 << 16
+        src = rt.malloc(cap + 64); dst = rt.malloc(npes * cap + 64)
+        for nbytes, soff, doff in ((1, 0, 0), (15, 1, 2), (16, 0, 0), (1023, 3, 0), (1024, 0, 16), (4100, 5, 9),
+                                   (65536, 0, 0), (40001, 16, 3)):
+            data = rng.integers(0, 256, (npes, nbytes), dtype=np.uint8)
+            rt.upload_all(src, data, soff)
+            rt.fill(dst, 0xCD, npes * cap + 64)
+            note("large-source path npes=%d fcollect bytes=%d soff=%d doff=%d" % (npes, nbytes, soff, doff))
+            rt.fcollectmem(dst + doff, src + soff, nbytes)
+            got = rt.download_all(dst, (npes * nbytes + doff + 16,), np.uint8)
+            assert np.array_equal(got[:, doff:doff + npes * nbytes], O.fcollect(data)), (nbytes, soff, doff)
+            assert (got[:, :doff] == 0xCD).all() and (got[:, doff + npes * nbytes:] == 0xCD).all()
+            root = (nbytes + soff) % npes
+            rt.fill(dst, 0xCD, npes * cap + 64)
+            note("large-source path npes=%d broadcast bytes=%d root=%d" % (npes, nbytes, root))
+            rt.broadcastmem(dst + doff, src + soff, nbytes, root)
+            got = rt.download_all(dst, (nbytes + doff + 16,), np.uint8)
+            assert np.array_equal(got[:, doff:doff + nbytes], O.broadcast(data, root)), (nbytes, soff, doff)
+            assert (got[:, :doff] == 0xCD).all() and (got[:, doff + nbytes:] == 0xCD).all()
+        # reductions and alltoall with streamed sources
+        n = 3000
+        fsrc = rt.malloc(npes * n * 4); fdst = rt.malloc(npes * n * 4)
+        fdata = rng.standard_normal((npes, npes * n)).astype(np.float32)
+        rt.upload_all(fsrc, fdata)
+        rt.reducescatter("float", "sum", fdst, fsrc, n)
+        assert bits_equal(rt.download_all(fdst, (n,), np.float32), O.reducescatter("f32", "sum", fdata))
+        rt.reduce("float", "sum", fdst, fsrc, n)
+        want = O.reduce("f32", "sum", fdata[:, :n])
+        assert all(bits_equal(rt.download(fdst, pe, (n,), np.float32), want) for pe in range(npes))
+        rt.alltoall("float", fdst, fsrc, n)
+        assert np.array_equal(rt.download_all(fdst, (npes * n * 4,), np.uint8), O.alltoall(fdata.view(np.uint8)))
+        for p in (src, dst, fsrc, fdst):
+            rt.free(p)
