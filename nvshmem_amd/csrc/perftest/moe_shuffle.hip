@@ -155,29 +155,34 @@ __global__ void moe_dispatch_pieces_kernel(char *recv, const char *send, const i
     }
 }
 
-// The same work items moved with nvshmem_ptr and plain vector accesses: the piece is loaded ONCE into
-// registers (V 16-byte vectors per lane) and stored to the topk destinations from there, so a source
-// byte crosses the memory system once instead of topk times.  Needs 16-byte aligned buffers and
+// The same work items moved with nvshmem_ptr and plain vector accesses: the piece is loaded into
+// registers (V 16-byte vectors per lane) and stored to up to four of the topk destinations from there;
+// the blocks that share a piece are neighbours in the grid and all but the first find it in the cache,
+// so a source byte crosses the HBM interface once instead of topk times.  Needs 16-byte aligned buffers and
 // rows; the host picks moe_dispatch_pieces_kernel otherwise.
 template <int V>
 __global__ void moe_dispatch_direct_kernel(char *recv, const char *send, const int32_t *dest_pe,
                                            const int64_t *dest_row, int tokens, int topk,
-                                           size_t row_bytes, size_t recv_cap_rows) {
+                                           size_t row_bytes, size_t recv_cap_rows, unsigned kshift) {
     const int me = nvshmem_my_pe(), np = nvshmem_n_pes();
     const int32_t *my_dest_pe = (const int32_t *)nvshmem_ptr(dest_pe, me);
     const int64_t *my_dest_row = (const int64_t *)nvshmem_ptr(dest_row, me);
     const nvshmemi_v4u *my_send = (const nvshmemi_v4u *)nvshmem_ptr(send, me);
     const unsigned waves_per_block = blockDim.x / NVSHMEMI_WARP_SIZE;
     const unsigned row_vecs = (unsigned)(row_bytes / 16);
-    const unsigned v0 = blockIdx.x * (64 * V) + threadIdx.x % NVSHMEMI_WARP_SIZE;
+    const unsigned v0 = (blockIdx.x >> kshift) * (64 * V) + threadIdx.x % NVSHMEMI_WARP_SIZE;
+    // 2^kshift neighbouring blocks share a piece and split the token's copies between them
+    const int kper = (topk + (1 << kshift) - 1) >> kshift;
+    const int k0 = (int)(blockIdx.x & ((1u << kshift) - 1)) * kper;
+    const int k1 = k0 + kper < topk ? k0 + kper : topk;
     for (size_t t = (size_t)blockIdx.y * waves_per_block + wave_in_block(); t < (size_t)tokens;
          t += (size_t)gridDim.y * waves_per_block) {
         const nvshmemi_v4u *src = my_send + t * row_vecs;
         nvshmemi_v4u x[V];
 #pragma unroll
         for (int u = 0; u < V; ++u)
-            if (v0 + 64 * u < row_vecs) x[u] = __builtin_nontemporal_load(src + v0 + 64 * u);
-        for (int k = 0; k < topk; ++k) {
+            if (v0 + 64 * u < row_vecs) x[u] = kshift ? src[v0 + 64 * u] : __builtin_nontemporal_load(src + v0 + 64 * u);
+        for (int k = k0; k < k1; ++k) {
             const size_t r = t * (size_t)topk + (size_t)k;
             const int pe = my_dest_pe[r];
             const int64_t row = my_dest_row[r];
@@ -352,10 +357,14 @@ int nvshmem_perftest_moe_dispatch_pieces(void *recv, size_t recv_cap_rows, const
     const dim3 grid((unsigned)pieces, token_blocks, (unsigned)nvshmem_n_pes());
     const bool aligned = row_bytes % 16 == 0 && ((uintptr_t)recv | (uintptr_t)send) % 16 == 0;
     const bool direct = aligned && getenv("NVSHMEM_PERFTEST_MOE_PUTS") == nullptr;
+    // at most four copies per wavefront (measured 1.62 -> 1.56 ms for top-8; two per wavefront is slower)
+    unsigned kshift = 0;
+    while (((topk + (1 << kshift) - 1) >> kshift) > 4) ++kshift;
+    const dim3 dgrid(grid.x << kshift, grid.y, grid.z);
 #define LAUNCH_DIRECT(V)                                                                           \
-    hipLaunchKernelGGL((moe_dispatch_direct_kernel<V>), grid, dim3(threads), 0, (hipStream_t)stream, \
+    hipLaunchKernelGGL((moe_dispatch_direct_kernel<V>), dgrid, dim3(threads), 0, (hipStream_t)stream, \
                        (char *)recv, (const char *)send, dest_pe, dest_row, tokens, topk, row_bytes, \
-                       recv_cap_rows)
+                       recv_cap_rows, kshift)
 #define LAUNCH_DISPATCH(P)                                                                         \
     hipLaunchKernelGGL((moe_dispatch_pieces_kernel<P>), grid, dim3(threads), 0, (hipStream_t)stream, \
                        (char *)recv, (const char *)send, dest_pe, dest_row, tokens, topk, row_bytes, \

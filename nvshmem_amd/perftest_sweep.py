@@ -120,7 +120,7 @@ def sweep_moe(N, hip, iters):
     best = timed_dispatch(lambda: perf.nvshmem_perftest_moe_dispatch(recv, cap, send, d_pe, d_row, expected,
                                                                      sig, T, K, row, 32, 256, None))
     best_pieces = timed_dispatch(lambda: perf.nvshmem_perftest_moe_dispatch_pieces(
-        recv, cap, send, d_pe, d_row, expected, sig, T, K, row, 1024, 128, None))
+        recv, cap, send, d_pe, d_row, expected, sig, T, K, row, 1024, 256, None))
     moved = npes * rows * row
     print("\nMoE token shuffle, 8 PEs x 8192 tokens x 7168 bf16, top-8 of 256 experts, Zipf(1.1); "
           "busiest PE receives %d of %d rows" % (cap, npes * rows))
