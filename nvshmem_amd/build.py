@@ -57,6 +57,17 @@ def _link(objs, out, extra=()):
 
 BINDIR = os.path.join(ROOT, "nvshmem_amd", "bin")
 DRIVER_SOURCE = "perftest/perftest_main.cpp"   # command-line driver over both libraries
+EXAMPLES = os.path.join(ROOT, "nvshmem_amd", "examples")   # user programs: public headers + the library only
+
+
+def _build_example(name):
+    """One command, as a user of the library would write it."""
+    out = os.path.join(BINDIR, "examples", name)
+    _run([HIPCC, "--offload-arch=gfx950", "-O3", "-std=c++17", "-Wall", "-Wno-unused-function",
+          "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops", "-I" + INCLUDE,
+          os.path.join(EXAMPLES, name + ".hip"), "-o", out, "-L" + LIBDIR, "-lnvshmem_amd",
+          "-Wl,-rpath,$ORIGIN/../../lib"])
+    return out
 
 
 def build_native(jobs=8):
@@ -77,6 +88,11 @@ def build_native(jobs=8):
         _run([HIPCC, "--offload-arch=gfx950", "-o", os.path.join(BINDIR, "nvshmem_perftest"),
               objs[DRIVER_SOURCE], "-L" + LIBDIR, "-lnvshmem_amd_perftest", "-lnvshmem_amd",
               "-Wl,-rpath,$ORIGIN/../lib"])
+    if os.path.isdir(EXAMPLES):
+        os.makedirs(os.path.join(BINDIR, "examples"), exist_ok=True)
+        names = sorted(f[:-4] for f in os.listdir(EXAMPLES) if f.endswith(".hip"))
+        with ThreadPoolExecutor(max_workers=jobs) as pool:
+            list(pool.map(_build_example, names))
     return runtime
 
 

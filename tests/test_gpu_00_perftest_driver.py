@@ -15,9 +15,10 @@ ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
 DRIVER = os.path.join(ROOT, "nvshmem_amd", "bin", "nvshmem_perftest")
 
 
-def _run(*args):
-    assert os.path.exists(DRIVER), "run `python -m nvshmem_amd.build` first"
-    proc = subprocess.run([DRIVER] + list(args), stdout=subprocess.PIPE, stderr=subprocess.PIPE, timeout=100)
+def _run(*args, exe=DRIVER, env=None):
+    assert os.path.exists(exe), "run `python -m nvshmem_amd.build` first"
+    proc = subprocess.run([exe] + list(args), stdout=subprocess.PIPE, stderr=subprocess.PIPE, timeout=100,
+                          env=dict(os.environ, **(env or {})))
     err = proc.stderr.decode()
     if proc.returncode != 0 and "cannot be performed in the present state" in err:
         pytest.skip("cooperative launches are held by another process on this GPU")
@@ -76,3 +77,14 @@ def test_point_to_point_latency_tables():
                  "shmem_p_ping_pong_latency", "shmem_atomic_ping_pong_latency"):
         line = next(l for l in out.splitlines() if l.startswith(name))
         assert 0.0 < float(line.split()[-1]) < 1000.0, line
+
+
+@pytest.mark.parametrize("name,npes", [("put_block", 8), ("ring_bcast", 8), ("ring_bcast", 3), ("allreduce", 8),
+                                       ("allreduce", 5), ("on_stream", 8), ("on_stream", 16)])
+def test_example_programs_reach_their_known_answers(name, npes):
+    """nvshmem_amd/examples/*.hip are user programs built with one hipcc command against include/ and
+    libnvshmem_amd.so; each checks the closed-form answer of the reference example it models on every
+    PE and prints PASSED."""
+    exe = os.path.join(ROOT, "nvshmem_amd", "bin", "examples", name)
+    out = _run(exe=exe, env={"NVSHMEM_AMD_NPES": str(npes), "NVSHMEM_SYMMETRIC_SIZE": str(64 << 20)})
+    assert out.strip().endswith(name + ": PASSED"), out
