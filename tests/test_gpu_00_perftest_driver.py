@@ -80,11 +80,11 @@ def test_point_to_point_latency_tables():
 
 
 @pytest.mark.parametrize("name,npes", [("put_block", 8), ("ring_bcast", 8), ("ring_bcast", 3), ("allreduce", 8),
-                                       ("allreduce", 5), ("on_stream", 8), ("on_stream", 16)])
+                                       ("allreduce", 5), ("on_stream", 8), ("on_stream", 16), ("moe_shuffle", 8), ("moe_shuffle", 3)])
 def test_example_programs_reach_their_known_answers(name, npes):
     """nvshmem_amd/examples/*.hip are user programs built with one hipcc command against include/ and
     libnvshmem_amd.so; each checks the closed-form answer of the reference example it models on every
     PE and prints PASSED."""
     exe = os.path.join(ROOT, "nvshmem_amd", "bin", "examples", name)
-    out = _run(exe=exe, env={"NVSHMEM_AMD_NPES": str(npes), "NVSHMEM_SYMMETRIC_SIZE": str(64 << 20)})
+    out = _run(exe=exe, env={"NVSHMEM_AMD_NPES": str(npes), "NVSHMEM_SYMMETRIC_SIZE": str(128 << 20)})
     assert out.strip().endswith(name + ": PASSED"), out
