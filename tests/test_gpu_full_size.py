@@ -79,3 +79,37 @@ def test_config4_fcollect_alltoall_16_pes_4M_elements(tname, es):
         for pe in range(16):
             assert np.array_equal(rt.download(fdst, pe, (16 * n * es,), np.uint8), want), pe
         rt.free(src); rt.free(fdst); rt.free(adst)
+
+
+def test_host_put_and_get_beyond_the_cache_size():
+    """Host-initiated transfers of more than 128 MiB between device buffers run on the library's own
+    copy kernel instead of hipMemcpyAsync: every mutual alignment class once, host memory on the
+    other side still works, bytes around the destination untouched."""
+    import ctypes as C
+    from nvshmem_amd import hip
+    size = (128 << 20) + 4099
+    rng = np.random.default_rng(9)
+    with runtime(4, 2 * size + (64 << 20)) as rt:
+        a = rt.malloc(size + 64); b = rt.malloc(size + 64)
+        data = rng.integers(0, 256, size + 32, dtype=np.uint8)
+        rt.upload(a, 0, data)
+        s = hip.Stream()
+        for soff, doff in ((0, 0), (3, 1), (16, 5)):
+            rt.fill(b, 0xCD, size + 64)
+            note("host put of %d bytes soff=%d doff=%d" % (size, soff, doff))
+            rt.lib.nvshmemx_putmem_on_stream(b + doff, a + soff, size, 2, s.ptr)    # PE 0's a -> PE 2's b
+            s.synchronize()
+            got = rt.download(b, 2, (size + 48,), np.uint8)
+            assert np.array_equal(got[doff:doff + size], data[soff:soff + size]), (soff, doff)
+            assert (got[:doff] == 0xCD).all() and (got[doff + size:] == 0xCD).all()
+            assert (rt.download(b, 0, (4096,), np.uint8) == 0xCD).all()
+        note("host get of %d bytes" % size)
+        rt.lib.nvshmemx_getmem_on_stream(rt.ptr(a, 1) + 7, b + 5, size, 2, s.ptr)   # PE 2's b -> PE 1's a
+        s.synchronize()
+        assert np.array_equal(rt.download(a, 1, (size,), np.uint8, 7), data[16:16 + size])
+        host = np.zeros(size, np.uint8)                                             # pageable host memory
+        rt.lib.nvshmemx_getmem_on_stream(host.ctypes.data_as(C.c_void_p), b + 5, size, 2, s.ptr)
+        s.synchronize()
+        assert np.array_equal(host, data[16:16 + size])
+        s.destroy()
+        rt.free(a); rt.free(b)
