@@ -14,6 +14,8 @@
 //        coll_latency                       the same five calls made inside a kernel, the call
 //                                           repeated --iters times in one launch
 //        barrier_latency                    nvshmem_barrier_all inside a kernel
+//        host_put_bw host_get_bw            nvshmemx_putmem_on_stream / getmem_on_stream from PE 0 to
+//                                           PE 1 (perftest/host/pt-to-pt/bw.cpp)
 //        pt2pt_latency                      put / get (+ put_signal ping-pong) latency per size and
 //                                           p, g, fetching atomic, signal / p / atomic ping-pong
 //                                           latency between PE 0 and PE 1, inside one kernel
@@ -41,7 +43,7 @@ struct Options {
 
 [[noreturn]] void usage(const char *why) {
     fprintf(stderr, "nvshmem_perftest: %s\nusage: nvshmem_perftest <put_bw|get_bw|reduce|reducescatter|fcollect|"
-                    "alltoall|broadcast|coll_latency|barrier_latency|pt2pt_latency> [--npes N] [--min B] [--max B] [--iters K] "
+                    "alltoall|broadcast|coll_latency|barrier_latency|pt2pt_latency|host_put_bw|host_get_bw> [--npes N] [--min B] [--max B] [--iters K] "
                     "[--warmup W] [--blocks B] [--threads T] [--scope thread|warp|block]\n", why);
     exit(2);
 }
@@ -244,6 +246,28 @@ int run_device_latency(const Options &o, bool barrier_only) {
     return 0;
 }
 
+// host-initiated transfers on the default stream between PE 0 and PE 1
+int run_host_rma(const Options &o, bool is_get) {
+    void *src = nvshmem_malloc(o.max_bytes), *dst = nvshmem_malloc(o.max_bytes);
+    if (!src || !dst) return 1;
+    std::vector<size_t> sizes = sweep(o, 1);
+    std::vector<double> gbs, us;
+    for (size_t bytes : sizes) {
+        const double ms = time_ms([&] {
+            if (is_get) nvshmemx_getmem_on_stream(dst, src, bytes, 1, nullptr);
+            else nvshmemx_putmem_on_stream(dst, src, bytes, 1, nullptr);
+            return 0;
+        }, o.iters, o.warmup);
+        gbs.push_back((double)bytes / ms / 1e6);
+        us.push_back(ms * 1e3);
+    }
+    print_table(is_get ? "get_on_stream" : "put_on_stream", "stream", "latency", "us", sizes, us);
+    print_table(is_get ? "get_on_stream" : "put_on_stream", "stream", "BW", "GB/s payload", sizes, gbs);
+    nvshmem_free(src);
+    nvshmem_free(dst);
+    return 0;
+}
+
 // (launch with K + 1 repetitions - launch with 1) / K, like run_device_latency; sig is cleared before
 // every launch because the ping-pong kinds count from zero.
 int run_pt2pt_latency(const Options &o) {
@@ -297,7 +321,8 @@ int main(int argc, char **argv) {
     const Options o = parse(argc, argv);
     const bool device_lat = o.test == "coll_latency" || o.test == "barrier_latency" || o.test == "pt2pt_latency";
     // heap: source and dest of the largest size, times npes for the collectives
-    const bool rma = o.test == "put_bw" || o.test == "get_bw" || o.test == "pt2pt_latency";
+    const bool rma = o.test == "put_bw" || o.test == "get_bw" || o.test == "pt2pt_latency" ||
+                     o.test == "host_put_bw" || o.test == "host_get_bw";
     Options eff = o;
     if (device_lat && o.max_bytes > ((size_t)1 << 20)) eff.max_bytes = (size_t)1 << 20;
     const size_t per_pe = (rma ? 2 * eff.max_bytes : 2 * eff.max_bytes * (size_t)eff.npes) + ((size_t)16 << 20);
@@ -316,6 +341,8 @@ int main(int argc, char **argv) {
     else if (o.test == "coll_latency") rc = run_device_latency(eff, false);
     else if (o.test == "barrier_latency") rc = run_device_latency(eff, true);
     else if (o.test == "pt2pt_latency") rc = run_pt2pt_latency(eff);
+    else if (o.test == "host_put_bw") rc = run_host_rma(eff, false);
+    else if (o.test == "host_get_bw") rc = run_host_rma(eff, true);
     else usage("unknown test");
     if (rc != 0) fprintf(stderr, "nvshmem_perftest: %s\n", nvshmemx_amd_last_error());
     nvshmem_finalize();

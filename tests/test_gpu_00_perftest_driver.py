@@ -51,6 +51,13 @@ def test_put_bw_and_collective_tables():
     assert len(_rows(out, "bcast_on_stream")) == 11
 
 
+def test_host_rma_tables():
+    out = _run("host_put_bw", "--min", "1k", "--max", "1m", "--iters", "10", "--npes", "2")
+    rows = _rows(out, "put_on_stream")
+    assert [r[0] for r in rows] == [1024 << i for i in range(11)] and all(v > 0 for _, _, v in rows)
+    assert len(_rows(_run("host_get_bw", "--min", "64", "--max", "4k", "--iters", "5"), "get_on_stream")) == 7
+
+
 def test_device_latency_tables():
     out = _run("coll_latency", "--min", "8", "--max", "512", "--iters", "50", "--scope", "warp")
     for job in ("reduction_latency", "reducescatter_latency", "fcollect_latency", "alltoall_latency", "bcast_latency"):
