@@ -192,16 +192,13 @@ __global__ __launch_bounds__(kCopyThreads) void segment_copy_kernel(char *base, 
 // ---------------------------------------------------------------------------------------------
 // NPES > 0 fixes the team size at compile time (fold fully unrolled, one wavefront per PE);
 // NPES == 0 takes both from the arguments.
-// SCATTER turns the kernel into reducescatter: blockIdx.y is the destination PE q, the fold runs over
-// block q (nelems elements, a whole number of vectors) of every PE's source with the operands in
-// reducescatter's order, and only PE q's destination is written.  Tiles are then cut on the
-// source's boundaries, because the loads are npes times the stores.
+// fold_next: one step of the fold, in the allreduce's operand order or (SCATTER) the reducescatter's.
 template <typename T, int OP, bool SCATTER>
 __device__ __forceinline__ T fold_next(int p, T acc, T x) {
     return SCATTER ? nvshmemi_amd_reduce_op<T, OP>(acc, x) : nvshmemi_amd_fold_step<T, OP>(p, acc, x);
 }
 
-template <typename T, int OP, int NPES, bool NTL, bool SCATTER = false, int VPT = NVSHMEM_AMD_REDUCE_VPT>
+template <typename T, int OP, int NPES, bool NTL, int VPT = NVSHMEM_AMD_REDUCE_VPT>
 __global__ __launch_bounds__(NPES ? NPES * 64 : 1024) void reduce_vector_kernel(char *base, uint32_t shift,
                                                              const nvshmemi_amd_team_view_t *groups,
                                                              uint32_t lane_shift_arg, uint64_t dst_off,
@@ -211,7 +208,6 @@ __global__ __launch_bounds__(NPES ? NPES * 64 : 1024) void reduce_vector_kernel(
     // this block's team; with NPES > 0 the host has checked that every team has NPES members
     const nvshmemi_amd_team_view_t g = groups[blockIdx.z];
     const int npes = NPES ? NPES : g.size;
-    if (SCATTER && (int)blockIdx.y >= npes) return;
     base += (uint64_t)g.start << shift;
     const uint32_t lane_shift = NPES ? 6u : lane_shift_arg;
     const unsigned lanes = 1u << lane_shift;
@@ -222,11 +218,7 @@ __global__ __launch_bounds__(NPES ? NPES * 64 : 1024) void reduce_vector_kernel(
     // the first tile lie in front of the buffer
     const uint64_t pe_stride = (uint64_t)g.stride << shift;  // from one member to the next
     const bool member = NPES ? true : (int)pe < npes;        // the block is sized for the largest team
-    if (SCATTER) {
-        src_off += (uint64_t)blockIdx.y * nelems * sizeof(T);
-        dst_off += (uint64_t)blockIdx.y * pe_stride;
-    }
-    const uint64_t lead = ((uint64_t)(uintptr_t)(base + (SCATTER ? src_off : dst_off)) >> 4) & (lanes - 1);
+    const uint64_t lead = ((uint64_t)(uintptr_t)(base + dst_off) >> 4) & (lanes - 1);
     // a tile is VPT pieces of `lanes` vectors per PE: thread (pe, i) loads vector i of each piece
     const unsigned tile_vecs = (unsigned)VPT << lane_shift;
     const uint64_t ntiles = (nvec + lead + tile_vecs - 1) / tile_vecs;
@@ -251,7 +243,7 @@ __global__ __launch_bounds__(NPES ? NPES * 64 : 1024) void reduce_vector_kernel(
             T acc = stage_e[e];
 #pragma unroll
             for (int p = 1; p < npes; ++p)
-                acc = fold_next<T, OP, SCATTER>(p, acc, stage_e[(size_t)p * tile_elems + e]);
+                acc = nvshmemi_amd_fold_step<T, OP>(p, acc, stage_e[(size_t)p * tile_elems + e]);
             result_e[e] = acc;
         }
         __syncthreads();
@@ -259,14 +251,9 @@ __global__ __launch_bounds__(NPES ? NPES * 64 : 1024) void reduce_vector_kernel(
         for (int u = 0; u < VPT; ++u) {
             const uint64_t v = v0 + ((uint64_t)u << lane_shift);
             const nvshmemi_v4u r = result[((unsigned)u << lane_shift) + i];
-            if (SCATTER) {
-                if (v < nvec && pe == 0) stream_store(base + dst_off + 16 * v, r);
-            } else {
-                if (v < nvec && member) stream_store(base + (uint64_t)pe * pe_stride + dst_off + 16 * v, r);
-            }
+            if (v < nvec && member) stream_store(base + (uint64_t)pe * pe_stride + dst_off + 16 * v, r);
         }
     }
-    if (SCATTER) return;  // a block of the source is a whole number of vectors
     // elements behind the last full vector
     const uint64_t done = nvec * VEC;
     const uint64_t gid = (uint64_t)blockIdx.x * blockDim.x + threadIdx.x;
@@ -281,19 +268,77 @@ __global__ __launch_bounds__(NPES ? NPES * 64 : 1024) void reduce_vector_kernel(
     }
 }
 
-// reducescatter for teams of at most 8 members without LDS: a block is ONE wavefront, lane i loads
-// vector i of a 1 KiB piece of block q (blockIdx.y) from every member - up to eight independent loads in
-// flight per lane - folds them in member order in registers and stores one vector into member q's
-// destination.  The work is nearly all loads, and for loads this shape measures 7 % faster than the
-// LDS-staged tile (6.3 against 5.9 TB/s for 8 members and 256 MiB of source per member).  NPES > 0 fixes
-// the team size at compile time; NPES == 0 reads it from the team (1..8).
+// Allreduce without LDS, for teams the LDS-staged kernel serves badly (more than 16 members: its block
+// of 1024 threads leaves 32 or 16 lanes per member, i.e. 512 or 256 byte accesses): a block is ONE
+// wavefront, lane i loads vector i of a 1 KiB piece from every member, eight loads in flight at a time,
+// folds in member order and stores the result to every member.
+template <typename T, int OP, bool NTL>
+__global__ __launch_bounds__(64) void reduce_gather_kernel(char *base, uint32_t shift,
+                                                           const nvshmemi_amd_team_view_t *groups,
+                                                           uint64_t dst_off, uint64_t src_off, uint64_t nelems) {
+    constexpr int VEC = 16 / sizeof(T);
+    constexpr int kBatch = 8;
+    union pack_t {
+        nvshmemi_v4u v;
+        T e[VEC];
+    };
+    const nvshmemi_amd_team_view_t g = groups[blockIdx.z];
+    const int npes = g.size;
+    base += (uint64_t)g.start << shift;
+    const uint64_t pe_stride = (uint64_t)g.stride << shift;
+    const uint64_t nvec = nelems / VEC;
+    const uint64_t lead = ((uint64_t)(uintptr_t)(base + dst_off) >> 4) & 63;
+    const uint64_t v = (uint64_t)blockIdx.x * 64 + threadIdx.x - lead;
+    if (v < nvec) {
+        const char *src = base + src_off + 16 * v;
+        pack_t acc;
+        for (int p0 = 0; p0 < npes; p0 += kBatch) {
+            pack_t x[kBatch];
+#pragma unroll
+            for (int k = 0; k < kBatch; ++k)
+                if (p0 + k < npes) x[k].v = stream_load<NTL>(src + (uint64_t)(p0 + k) * pe_stride);
+#pragma unroll
+            for (int k = 0; k < kBatch; ++k)
+                if (p0 + k < npes) {
+                    if (p0 + k == 0) {
+                        acc = x[0];
+                    } else {
+#pragma unroll
+                        for (int j = 0; j < VEC; ++j)
+                            acc.e[j] = nvshmemi_amd_fold_step<T, OP>(p0 + k, acc.e[j], x[k].e[j]);
+                    }
+                }
+        }
+        char *dst = base + dst_off + 16 * v;
+        for (int p = 0; p < npes; ++p) stream_store(dst + (uint64_t)p * pe_stride, acc.v);
+    }
+    // elements behind the last full vector
+    const uint64_t done = nvec * VEC;
+    const uint64_t gid = (uint64_t)blockIdx.x * 64 + threadIdx.x;
+    if (gid < nelems - done) {
+        const uint64_t k = done + gid;
+        const T *s = reinterpret_cast<const T *>(base + src_off);
+        T *d = reinterpret_cast<T *>(base + dst_off);
+        const uint64_t es = pe_stride / sizeof(T);
+        T acc = s[k];
+        for (int p = 1; p < npes; ++p) acc = nvshmemi_amd_fold_step<T, OP>(p, acc, s[(uint64_t)p * es + k]);
+        for (int p = 0; p < npes; ++p) d[(uint64_t)p * es + k] = acc;
+    }
+}
+
+// reducescatter without LDS: a block is ONE wavefront, lane i loads vector i of a 1 KiB piece of block q
+// (blockIdx.y) from every member - eight independent loads in flight per lane at a time - folds them in
+// member order in registers and stores one vector into member q's destination.  The work is nearly all
+// loads, and for loads this shape beats the LDS-staged tile of the allreduce: 6.3 against 5.9 TB/s for
+// 8 members with 256 MiB of source each, 5.9 against 3.7 TB/s for 16 members.  NPES > 0 fixes the team
+// size at compile time; NPES == 0 reads it from the team.
 template <typename T, int OP, int NPES, bool NTL>
 __global__ __launch_bounds__(64) void reducescatter_gather_kernel(char *base, uint32_t shift,
                                                                   const nvshmemi_amd_team_view_t *groups,
                                                                   uint64_t dst_off, uint64_t src_off,
                                                                   uint64_t nelems) {
     constexpr int VEC = 16 / sizeof(T);
-    constexpr int kMax = NPES ? NPES : 8;
+    constexpr int kBatch = 8;  // loads in flight per lane
     union pack_t {
         nvshmemi_v4u v;
         T e[VEC];
@@ -309,17 +354,24 @@ __global__ __launch_bounds__(64) void reducescatter_gather_kernel(char *base, ui
     const uint64_t lead = ((uint64_t)(uintptr_t)(base + src_off) >> 4) & 63;
     const uint64_t v = (uint64_t)blockIdx.x * 64 + threadIdx.x - lead;
     if (v >= nvec) return;  // also the slots in front of the block (wrapped)
-    pack_t x[kMax];
+    const char *src = base + src_off + 16 * v;
+    pack_t acc;
+    for (int p0 = 0; p0 < npes; p0 += kBatch) {
+        pack_t x[kBatch];
 #pragma unroll
-    for (int p = 0; p < kMax; ++p)
-        if (p < npes) x[p].v = stream_load<NTL>(base + (uint64_t)p * pe_stride + src_off + 16 * v);
-    pack_t acc = x[0];
+        for (int k = 0; k < kBatch; ++k)
+            if (p0 + k < npes) x[k].v = stream_load<NTL>(src + (uint64_t)(p0 + k) * pe_stride);
 #pragma unroll
-    for (int p = 1; p < kMax; ++p)
-        if (p < npes) {
+        for (int k = 0; k < kBatch; ++k)
+            if (p0 + k < npes) {
+                if (p0 + k == 0) {
+                    acc = x[0];
+                } else {
 #pragma unroll
-            for (int k = 0; k < VEC; ++k) acc.e[k] = nvshmemi_amd_reduce_op<T, OP>(acc.e[k], x[p].e[k]);
-        }
+                    for (int j = 0; j < VEC; ++j) acc.e[j] = nvshmemi_amd_reduce_op<T, OP>(acc.e[j], x[k].e[j]);
+                }
+            }
+    }
     stream_store(base + (uint64_t)blockIdx.y * pe_stride + dst_off + 16 * v, acc.v);
 }
 
@@ -371,20 +423,26 @@ void launch_reduce(Runtime &rt, const TeamLaunch &tl, uint64_t dst_off, uint64_t
                    uint64_t nelems, hipStream_t stream) {
     const bool vector_ok = ((dst_off | src_off) & 15) == 0;
     const unsigned ngroups = (unsigned)tl.ngroups;
-    if (vector_ok) {
-        // lanes per PE: a full wavefront when the block still fits 1024 threads
-        uint32_t lane_shift = 6;
-        while (((uint32_t)tl.max_size << lane_shift) > 1024) --lane_shift;  // size <= 64 -> >= 16 lanes
-        const unsigned threads = (unsigned)tl.max_size << lane_shift;
+    // Which vector kernel: the LDS-staged one only has the edge for teams of exactly 8 or 16 members
+    // with more than Runtime::lds_reduce_bytes (1 GiB) of sources in all (measured with random fp32 data, 8 members: 6.26 against
+    // 5.71 TB/s at 2 GiB, equal at 1 GiB, 49.6 against 40.8 us at 128 MiB; 16 members: +2..4 % from
+    // 512 MiB up); everything else - other team sizes, smaller messages - goes to the gather kernel
+    // (12 members +14 %, 32 +7 %, 64 +22 %, 4 +7 %).
+    const uint64_t total_bytes = total_members(tl) * nelems * sizeof(T);
+    const int fixed_size = tl.min_size == tl.max_size ? tl.max_size : 0;
+    const bool stream_source = total_bytes > rt.cacheable_source_bytes;
+    // the threshold counts elements (as 4-byte ones): narrow types fold more elements per byte, and the
+    // gather kernel does that arithmetic in one lane per vector (bf16 at 1 GiB: 5.3 against 6.0 TB/s)
+    if (vector_ok && (fixed_size == 8 || fixed_size == 16) &&
+        total_members(tl) * nelems > rt.lds_reduce_bytes / 4) {
+        const uint32_t lane_shift = 6;
+        const unsigned threads = (unsigned)fixed_size << lane_shift;
         const uint64_t nvec = nelems / (16 / sizeof(T));
         const uint64_t tile_vecs = (uint64_t)NVSHMEM_AMD_REDUCE_VPT << lane_shift;
         uint64_t blocks = (nvec + (1u << lane_shift) + tile_vecs - 1) / tile_vecs;  // room for the lead-in
         if (blocks > 0x7fffffffull) blocks = 0x7fffffffull;  // the tile loop covers the rest
-        if (blocks == 0) blocks = 1;                          // only tail elements
-        const size_t lds = ((size_t)tl.max_size + 1) * 16 * tile_vecs;
+        const size_t lds = ((size_t)fixed_size + 1) * 16 * tile_vecs;
         const dim3 grid((unsigned)blocks, 1, ngroups);
-        const bool stream_source =
-            total_members(tl) * nelems * sizeof(T) > rt.cacheable_source_bytes;
 #define NVSHMEM_AMD_LAUNCH_REDUCE(N)                                                              \
     do {                                                                                          \
         if (stream_source)                                                                        \
@@ -396,13 +454,23 @@ void launch_reduce(Runtime &rt, const TeamLaunch &tl, uint64_t dst_off, uint64_t
                                stream, rt.base, rt.heap_shift, tl.groups, lane_shift, dst_off,    \
                                src_off, nelems);                                                  \
     } while (0)
-        // the compile-time sizes need every team of the handle to have that many members
-        switch (tl.min_size == tl.max_size ? tl.max_size : 0) {
-            case 8: NVSHMEM_AMD_LAUNCH_REDUCE(8); break;
-            case 16: NVSHMEM_AMD_LAUNCH_REDUCE(16); break;
-            default: NVSHMEM_AMD_LAUNCH_REDUCE(0); break;
-        }
+        if (fixed_size == 8) NVSHMEM_AMD_LAUNCH_REDUCE(8);
+        else NVSHMEM_AMD_LAUNCH_REDUCE(16);
 #undef NVSHMEM_AMD_LAUNCH_REDUCE
+    } else if (vector_ok) {
+        const uint64_t nvec = nelems / (16 / sizeof(T));
+        uint64_t blocks = (nvec + 63 + 63) / 64;  // room for the lead-in; at least one block for the tail
+        if (blocks > 0x7fffffffull) {
+            set_error("reduce: message too large");
+            return;
+        }
+        const dim3 grid((unsigned)blocks, 1, ngroups);
+        if (stream_source)
+            hipLaunchKernelGGL((reduce_gather_kernel<T, OP, true>), grid, dim3(64), 0, stream, rt.base,
+                               rt.heap_shift, tl.groups, dst_off, src_off, nelems);
+        else
+            hipLaunchKernelGGL((reduce_gather_kernel<T, OP, false>), grid, dim3(64), 0, stream, rt.base,
+                               rt.heap_shift, tl.groups, dst_off, src_off, nelems);
     } else {
         uint64_t blocks = (nelems + kThreads - 1) / kThreads;
         const uint64_t cap = (uint64_t)rt.num_cus * 64 / ngroups + 1;
@@ -419,7 +487,7 @@ void launch_reducescatter(Runtime &rt, const TeamLaunch &tl, uint64_t dst_off, u
                           uint64_t nelems, hipStream_t stream) {
     const bool vector_ok = ((dst_off | src_off | (nelems * sizeof(T))) & 15) == 0;
     const unsigned ngroups = (unsigned)tl.ngroups;
-    if (vector_ok && tl.max_size <= 8) {
+    if (vector_ok) {
         const uint64_t nvec = nelems / (16 / sizeof(T));
         uint64_t blocks = (nvec + 63 + 63) / 64;  // room for the lead-in
         if (blocks > 0x7fffffffull) {
@@ -429,11 +497,10 @@ void launch_reducescatter(Runtime &rt, const TeamLaunch &tl, uint64_t dst_off, u
         const dim3 grid((unsigned)blocks, (unsigned)tl.max_size, ngroups);
         const bool stream_source =
             total_members(tl) * tl.max_size * nelems * sizeof(T) > rt.cacheable_source_bytes;
-        const bool eight = tl.min_size == 8 && tl.max_size == 8;
 #define NVSHMEM_AMD_LAUNCH_GATHER(N, NTL)                                                         \
     hipLaunchKernelGGL((reducescatter_gather_kernel<T, OP, N, NTL>), grid, dim3(64), 0, stream,   \
                        rt.base, rt.heap_shift, tl.groups, dst_off, src_off, nelems)
-        if (eight) {
+        if (tl.min_size == 8 && tl.max_size == 8) {
             if (stream_source) NVSHMEM_AMD_LAUNCH_GATHER(8, true);
             else NVSHMEM_AMD_LAUNCH_GATHER(8, false);
         } else {
@@ -441,25 +508,6 @@ void launch_reducescatter(Runtime &rt, const TeamLaunch &tl, uint64_t dst_off, u
             else NVSHMEM_AMD_LAUNCH_GATHER(0, false);
         }
 #undef NVSHMEM_AMD_LAUNCH_GATHER
-    } else if (vector_ok) {
-        uint32_t lane_shift = 6;
-        while (((uint32_t)tl.max_size << lane_shift) > 1024) --lane_shift;
-        const unsigned threads = (unsigned)tl.max_size << lane_shift;
-        const uint64_t nvec = nelems / (16 / sizeof(T));
-        const uint64_t tile_vecs = (uint64_t)1 << lane_shift;
-        uint64_t blocks = (nvec + (1u << lane_shift) + tile_vecs - 1) / tile_vecs;
-        if (blocks > 0x7fffffffull) blocks = 0x7fffffffull;
-        const size_t lds = ((size_t)tl.max_size + 1) * 16 * tile_vecs;
-        const dim3 grid((unsigned)blocks, (unsigned)tl.max_size, ngroups);
-        const bool stream_source =
-            total_members(tl) * tl.max_size * nelems * sizeof(T) > rt.cacheable_source_bytes;
-#define NVSHMEM_AMD_LAUNCH_SCATTER(N, NTL)                                                        \
-    hipLaunchKernelGGL((reduce_vector_kernel<T, OP, N, NTL, true, 1>), grid, dim3(threads), lds,  \
-                       stream, rt.base, rt.heap_shift, tl.groups, lane_shift, dst_off, src_off,   \
-                       nelems)
-        if (stream_source) NVSHMEM_AMD_LAUNCH_SCATTER(0, true);
-        else NVSHMEM_AMD_LAUNCH_SCATTER(0, false);
-#undef NVSHMEM_AMD_LAUNCH_SCATTER
     } else {
         uint64_t blocks = (nelems + kThreads - 1) / kThreads;
         const uint64_t cap = (uint64_t)rt.num_cus * 64 / ((uint64_t)tl.max_size * ngroups) + 1;

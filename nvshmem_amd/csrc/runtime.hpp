@@ -62,6 +62,10 @@ struct Runtime {
     // Host-launched collectives treat sources of more bytes than this (all PEs together) as too
     // large to stay in the Infinity Cache: NVSHMEM_AMD_CACHEABLE_SOURCE_BYTES, read at init
     uint64_t cacheable_source_bytes = (uint64_t)256 << 20;
+    // Allreduce on teams of exactly 8 or 16 members takes the LDS-staged kernel when the sources of
+    // all PEs together hold more than this many bytes' worth of 4-byte elements:
+    // NVSHMEM_AMD_LDS_REDUCE_BYTES, read at init
+    uint64_t lds_reduce_bytes = (uint64_t)1 << 30;
 
     static Runtime &get();
 

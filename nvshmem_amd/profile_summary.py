@@ -52,7 +52,7 @@ WORKLOADS = {
         "ring_rma_kernel_put_block_8pe_256MiB.txt",
         "put_block: nvshmemx_putmem_block ring, 8 logical PEs x 256 MiB, 262144 blocks x 64 threads per PE (1 KiB per block).\n"
         "Algorithmic bytes per launch: 8 x 256 MiB read + 8 x 256 MiB written = 4 GiB.", 4 << 30),
-    "reduce_vector_kernel<float, 5, 8, true, false,": (
+    "reduce_vector_kernel<float, 5, 8, true,": (
         "reduce_vector_kernel_float_sum_8pe_64Mi.txt",
         "sum_reduce: nvshmemx_float_sum_reduce_on_stream, 8 logical PEs x 2^26 fp32.\n"
         "Algorithmic bytes per launch: 8 sources read once + 8 destinations written once = 4 GiB.", 4 << 30),

@@ -33,10 +33,22 @@ def _random_storage(kind, shape, rng, op):
     return rng.integers(info.min, info.max, size=shape, dtype=dt, endpoint=True)
 
 
-@pytest.fixture(scope="module")
-def rt8():
-    with runtime(8, 1 << 28) as r:
-        yield r
+@pytest.fixture(scope="module", params=["gather", "lds"])
+def rt8(request):
+    """Every test of this module runs with both allreduce kernels: the default choice (the gather
+    kernel at these sizes) and the LDS-staged kernel forced by NVSHMEM_AMD_LDS_REDUCE_BYTES=0."""
+    import os
+    old = os.environ.get("NVSHMEM_AMD_LDS_REDUCE_BYTES")
+    if request.param == "lds":
+        os.environ["NVSHMEM_AMD_LDS_REDUCE_BYTES"] = "0"
+    try:
+        with runtime(8, 1 << 28) as r:
+            yield r
+    finally:
+        if old is None:
+            os.environ.pop("NVSHMEM_AMD_LDS_REDUCE_BYTES", None)
+        else:
+            os.environ["NVSHMEM_AMD_LDS_REDUCE_BYTES"] = old
 
 
 # ---------------------------------------------------------------------------------------------

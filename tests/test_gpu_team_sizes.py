@@ -187,6 +187,7 @@ def test_large_source_policy_of_fcollect_and_broadcast(npes, monkeypatch):
     wavefront).  With the threshold at zero every size takes that path: ragged, misaligned messages
     must come out the same, bytes outside the destination untouched."""
     monkeypatch.setenv("NVSHMEM_AMD_CACHEABLE_SOURCE_BYTES", "0")
+    monkeypatch.setenv("NVSHMEM_AMD_LDS_REDUCE_BYTES", "0")      # 8 and 16 members: the LDS-staged allreduce
     rng = np.random.default_rng(100 + npes)
     with runtime(npes, 1 << 24) as rt:
         cap = 1 << 16
