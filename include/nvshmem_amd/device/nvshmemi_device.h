@@ -780,16 +780,28 @@ NVSHMEMI_DEVICE_INLINE unsigned nvshmemi_amd_ll_lanes() {
 }
 NVSHMEMI_DEVICE_INLINE bool nvshmemi_amd_ll_available() { return nvshmemi_device_state_d.ll_buffers != nullptr; }
 
-/* Next flag of the calling PE for `team`; all threads of the group return the same value. */
+/* The calling PE's count of packet collectives on `team` so far.  Every thread of the group reads
+ * it; no group synchronisation is needed in front: the word only changes in nvshmemi_amd_ll_next_flag,
+ * and every packet collective passes nvshmemi_amd_ll_publish_done's synchronisation after that. */
+NVSHMEMI_DEVICE_INLINE uint64_t nvshmemi_amd_ll_peek_count(nvshmem_team_t team) {
+    return *reinterpret_cast<volatile uint64_t *>(
+        nvshmemi_amd_ll_word(team, nvshmemi_amd_my_pe(), NVSHMEMI_AMD_LL_COUNT_WORD));
+}
+/* Next flag of the calling PE for `team`, from the count peeked earlier; all threads of the group
+ * return the same value.  The synchronisation keeps the first thread's update behind everybody's read. */
 template <int SCOPE>
-NVSHMEMI_DEVICE_INLINE uint32_t nvshmemi_amd_ll_next_flag(nvshmem_team_t team) {
-    uint64_t *count = nvshmemi_amd_ll_word(team, nvshmemi_amd_my_pe(), NVSHMEMI_AMD_LL_COUNT_WORD);
-    nvshmemi_threadgroup_sync<SCOPE>();
-    uint32_t flag = (uint32_t)(*reinterpret_cast<volatile uint64_t *>(count)) + 1u;
+NVSHMEMI_DEVICE_INLINE uint32_t nvshmemi_amd_ll_next_flag(nvshmem_team_t team, uint64_t count_seen) {
+    uint32_t flag = (uint32_t)count_seen + 1u;
     if (flag == 0) flag = 1; /* 0 is what an empty buffer holds */
     nvshmemi_threadgroup_sync<SCOPE>();
-    if (nvshmemi_thread_id_in_threadgroup<SCOPE>() == 0) *reinterpret_cast<volatile uint64_t *>(count) = flag;
+    if (nvshmemi_thread_id_in_threadgroup<SCOPE>() == 0)
+        *reinterpret_cast<volatile uint64_t *>(
+            nvshmemi_amd_ll_word(team, nvshmemi_amd_my_pe(), NVSHMEMI_AMD_LL_COUNT_WORD)) = flag;
     return flag;
+}
+template <int SCOPE>
+NVSHMEMI_DEVICE_INLINE uint32_t nvshmemi_amd_ll_next_flag(nvshmem_team_t team) {
+    return nvshmemi_amd_ll_next_flag<SCOPE>(team, nvshmemi_amd_ll_peek_count(team));
 }
 
 NVSHMEMI_DEVICE_INLINE uint64_t nvshmemi_amd_ll_load_payload(const char *src, size_t left) {
