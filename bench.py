@@ -34,6 +34,9 @@ MEASURED_TRAFFIC_BYTES = {
     "alltoall_1GiB": None,              # not profiled
     "reducescatter": (2048 + 256) << 20,  # profiles/reducescatter_gather_kernel_float_sum_8pe_8Mi.txt
     "broadcast": (256 + 2048) << 20,      # profiles/segment_copy_kernel_broadcast_8pe_256MiB.txt
+    "fcollect": (256 + 4096) << 20,       # profiles/segment_copy_kernel_fcollect_16pe_4Mi_fp32.txt
+    "moe_dispatch": None,                 # not profiled
+    "moe_combine": None,                  # not profiled
 }
 
 # put_block launch shape: each block is one wavefront that moves a contiguous 1 KiB slice, one
@@ -267,6 +270,129 @@ def bench_broadcast(N, O, hip, np, steps, warmup, cpu_budget):
     }
 
 
+def bench_fcollect(N, O, hip, np, steps, warmup, cpu_budget):
+    """Config 4, fp32: 16 PEs x 2^22 elements, every PE ends with all 16 contributions."""
+    npes, n = 16, 1 << 22
+    with _runtime(N, npes, 17 * n * 4 + (16 << 20)) as rt:
+        src = rt.malloc(n * 4); dst = rt.malloc(npes * n * 4)
+        data = O.fill_all("u64", npes, n // 2, 6).view(np.uint8).reshape(npes, -1)
+        rt.upload_all(src, data)
+        from nvshmem_amd import _lib
+        fn = _lib.typed_coll(rt.lib, "nvshmemx_float_fcollect_on_stream", True)
+
+        def step():
+            rc = fn(N.TEAM_WORLD, dst, src, n, None)
+            if rc != 0:
+                raise RuntimeError("fcollect failed: %d %s" % (rc, rt.last_error()))
+        wall, ev = _time_steps(step, steps, warmup, hip)
+        want = data.reshape(-1)                       # every PE: the sources in PE order
+        ok = all(bool(np.array_equal(rt.download(dst, pe, (npes * n * 4,), np.uint8), want)) for pe in (0, 9, 15))
+        rt.free(src); rt.free(dst)
+    alg = (npes + 1) * npes * n * 4
+    cores = min(16, O.lib().oracle_get_threads())
+    O.lib().oracle_set_threads(cores)
+    best, passes = _cpu_time(lambda: O.fcollect(data), cpu_budget, 10)
+    cpu = {"value": round(alg / best / 1e9, 2), "unit": "GB/s", "cores": cores, "kind": "port",
+           "sample": "oracle_fcollect, 16 PEs x %d fp32 (the full workload), best of %d passes" % (n, passes)}
+    return {
+        "name": "fcollect", "dtype": "u8", "verified": ok, "algorithmic_bytes": alg,
+        "wall_ms": wall, "kernel_ms": ev,
+        "config": {"workload": "fcollect: nvshmemx_float_fcollect_on_stream, 16 logical PEs x %d fp32" % n,
+                   "npes": npes, "nelems": n,
+                   "note": "the 256 MiB of sources fit the Infinity Cache and are re-read from it on repeated steps"},
+        "kernel": "segment_copy_kernel<fcollect>",
+        "cpu_baseline": cpu,
+    }
+
+
+def bench_moe(N, O, hip, np, steps, warmup, cpu_budget):
+    """Config 5: 8 PEs x 8192 tokens x 7168 bf16, top-8 of 256 experts, Zipf(1.1).  Returns the
+    dispatch and the combine as two workloads; a step of each is one full pass over all rows."""
+    npes, T, K, E, row = 8, 8192, 8, 256, 7168 * 2
+    ex = O.moe_routing(npes, T, K, E, 1.1, 8)
+    counts, seg_base, dest_pe, dest_row, recv_rows = O.moe_plan(ex, npes, T, K, E)
+    cap, rows = int(recv_rows.max()), T * K
+    steps, warmup = max(1, steps // 5), max(1, warmup // 5)      # a step moves 8 / 14 GiB
+    with _runtime(N, npes, cap * row + rows * row + T * row + (64 << 20)) as rt:
+        perf = rt.perftest()
+        send = rt.malloc(T * row); recv = rt.malloc(cap * row); out = rt.malloc(rows * row)
+        d_pe = rt.malloc(rows * 4); d_row = rt.malloc(rows * 8)
+        expected = rt.malloc(npes * 8); sig = rt.calloc(npes, 8)
+        rt.upload_all(d_pe, dest_pe); rt.upload_all(d_row, dest_row)
+        epp = E // npes
+        exp_tab = np.stack([[counts[s, d * epp:(d + 1) * epp].sum() for s in range(npes)]
+                            for d in range(npes)]).astype(np.uint64)
+        rt.upload_all(expected, exp_tab)
+        payload = O.fill_all("u64", npes, T * row // 8, 7).view(np.uint8).reshape(npes, T, row)
+        rt.upload_all(send, payload)
+
+        def dispatch():
+            perf.nvshmem_perftest_fill_words(sig, 0, npes, None)
+            rc = perf.nvshmem_perftest_moe_dispatch_pieces(recv, cap, send, d_pe, d_row, expected, sig, T, K, row,
+                                                           1024, 256, None)
+            if rc != 0:
+                raise RuntimeError("moe dispatch failed: %d" % rc)
+
+        def combine():
+            rc = perf.nvshmem_perftest_moe_combine_pieces(out, recv, cap, d_pe, d_row, T, K, row, 2048, 262144, 64,
+                                                          N.SCOPE_WARP, None)
+            if rc != 0:
+                raise RuntimeError("moe combine failed: %d" % rc)
+        d_wall, d_ev = _time_steps(dispatch, steps, warmup, hip)
+        c_wall, c_ev = _time_steps(combine, steps, warmup, hip)
+        # parity on samples: signals count the rows exactly, sampled copies sit where the plan says,
+        # and the round trip returns every sampled row
+        ok = bool(np.array_equal(rt.download_all(sig, (npes,), np.uint64), exp_tab))
+        ok = ok and all(rt.read_timeout(pe)[0] == 0 for pe in range(npes))
+        rng = np.random.default_rng(0)
+        for src_pe in range(npes):
+            for r in rng.integers(0, rows, 64):
+                got = rt.download(recv, int(dest_pe[src_pe, r]), (row,), np.uint8, int(dest_row[src_pe, r]) * row)
+                back = rt.download(out, src_pe, (row,), np.uint8, int(r) * row)
+                ok = ok and bool(np.array_equal(got, payload[src_pe, r // K])) and bool(np.array_equal(back, got))
+        for p in (send, recv, out, d_pe, d_row, expected, sig):
+            rt.free(p)
+    moved = npes * rows * row
+    # CPU oracle on a bounded sample: the same shuffle with 1024 tokens per PE
+    Ts = 1024
+    exs = O.moe_routing(npes, Ts, K, E, 1.1, 8)
+    _, _, s_pe, s_row, s_recv = O.moe_plan(exs, npes, Ts, K, E)
+    small = np.ascontiguousarray(payload[:, :Ts])
+    cores = min(16, O.lib().oracle_get_threads())
+    O.lib().oracle_set_threads(cores)
+    held = {}
+
+    def cpu_dispatch():
+        held["recv"] = O.moe_dispatch(small, s_pe, s_row, s_recv, Ts, K)
+    best_d, passes_d = _cpu_time(cpu_dispatch, cpu_budget, 5)
+    best_c, passes_c = _cpu_time(lambda: O.moe_combine(held["recv"], s_pe, s_row, Ts, K, row), cpu_budget, 5)
+    small_moved = npes * Ts * K * row
+    shape = "8 logical PEs x 8192 tokens x 7168 bf16, top-8 of 256 experts, Zipf(1.1)"
+    common = {"npes": npes, "tokens": T, "topk": K, "experts": E, "row_bytes": row}
+    disp = {
+        "name": "moe_dispatch", "dtype": "u8", "verified": ok, "algorithmic_bytes": moved + moved // K,
+        "wall_ms": d_wall, "kernel_ms": d_ev,
+        "config": dict(common, workload="moe_dispatch: 1 KiB work items stored through nvshmem_ptr, ADD signals, "
+                       "signal_wait_until(GE); " + shape,
+                       note="algorithmic bytes = every source row read once and written top-k times "
+                            "(7.875 GiB); the timed step includes clearing the signal words"),
+        "kernel": "moe_dispatch_direct_kernel<1> + moe_dispatch_signal_kernel",
+        "cpu_baseline": {"value": round((small_moved + small_moved // K) / best_d / 1e9, 2), "unit": "GB/s",
+                         "cores": cores, "kind": "port",
+                         "sample": "oracle_moe_dispatch, 1024 tokens per PE, best of %d passes" % passes_d},
+    }
+    comb = {
+        "name": "moe_combine", "dtype": "u8", "verified": ok, "algorithmic_bytes": 2 * moved,
+        "wall_ms": c_wall, "kernel_ms": c_ev,
+        "config": dict(common, workload="moe_combine: nvshmemx_getmem_nbi_warp per 2 KiB of a row; " + shape),
+        "kernel": "moe_combine_kernel<warp, 2048>",
+        "cpu_baseline": {"value": round(2 * small_moved / best_c / 1e9, 2), "unit": "GB/s", "cores": cores,
+                         "kind": "port",
+                         "sample": "oracle_moe_combine, 1024 tokens per PE, best of %d passes" % passes_c},
+    }
+    return disp, comb
+
+
 class _runtime:
     def __init__(self, N, npes, size):
         self.N, self.npes, self.size = N, npes, size
@@ -321,6 +447,8 @@ def main():
                              name="alltoall_1GiB")
     rsc = bench_reducescatter(N, O, hip, np, args.steps, args.warmup, 1.0)
     bca = bench_broadcast(N, O, hip, np, args.steps, args.warmup, 1.0)
+    fco = bench_fcollect(N, O, hip, np, args.steps, args.warmup, 1.0)
+    moe_d, moe_c = bench_moe(N, O, hip, np, args.steps, args.warmup, 1.0)
 
     head = put
     value = head["algorithmic_bytes"] / head["wall_ms"] / 1e6
@@ -344,10 +472,12 @@ def main():
                      "traffic": MEASURED_TRAFFIC_BYTES[head["name"]], "kernel": head["kernel"]},
         "cpu_baseline": head["cpu_baseline"],
         "verified": bool(put["verified"] and red["verified"] and a2a["verified"] and a2a_big["verified"]
-                         and rsc["verified"] and bca["verified"]),
+                         and rsc["verified"] and bca["verified"] and fco["verified"] and moe_d["verified"]),
         "workloads": {"put_block": _summarise(put), "sum_reduce": _summarise(red),
                       "alltoall": _summarise(a2a), "alltoall_1GiB": _summarise(a2a_big),
-                      "reducescatter": _summarise(rsc), "broadcast": _summarise(bca)},
+                      "reducescatter": _summarise(rsc), "broadcast": _summarise(bca),
+                      "fcollect": _summarise(fco), "moe_dispatch": _summarise(moe_d),
+                      "moe_combine": _summarise(moe_c)},
     }
     print(json.dumps(line))
     return 0 if line["verified"] else 1

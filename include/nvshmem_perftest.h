@@ -64,6 +64,10 @@ int nvshmem_perftest_signal_wait(uint64_t *sig, int cmp, uint64_t cmp_value, uin
 int nvshmem_perftest_put_signal_pingpong(void *data, uint64_t *sig, size_t bytes, int iters,
                                          int threads, void *stream);
 
+/* Sets nwords 64-bit words of every PE's copy of `words` to `value` with one kernel on `stream` (for
+ * clearing signal words between timed launches without a host synchronisation per PE). */
+int nvshmem_perftest_fill_words(uint64_t *words, uint64_t value, size_t nwords, void *stream);
+
 /* Latency loops of the reference's perftest/device/pt-to-pt programs, one block per PE, `iters`
  * repetitions inside one launch.  Kinds 0-4: PE 0 acts on PE 1 - PUT: nvshmemx_putmem_block of `bytes`
  * of data + quiet (afterwards PE 1's data equals PE 0's); GET: nvshmemx_getmem_block (PE 0's data

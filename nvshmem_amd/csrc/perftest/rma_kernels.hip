@@ -96,6 +96,13 @@ __global__ void pingpong_kernel(char *data, uint64_t *sig, size_t bytes, int ite
     }
 }
 
+// every PE's copy of `words` := value, in one launch (stream ordered, unlike a memset per PE)
+__global__ void fill_words_kernel(uint64_t *words, uint64_t value, size_t n) {
+    uint64_t *mine = (uint64_t *)nvshmem_ptr(words, nvshmem_my_pe());
+    for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += (size_t)gridDim.x * blockDim.x)
+        mine[i] = value;
+}
+
 // Point-to-point latency loops in the shape of the reference's perftest/device/pt-to-pt programs:
 // PE 0 acts on PE 1 `iters` times (kinds 0-4: shmem_put_latency.cu, shmem_get_latency.cu,
 // shmem_p_latency.cu, shmem_g_latency.cu, shmem_atomic_latency.cu), or PE 0 and PE 1 bounce a word
@@ -302,6 +309,16 @@ int nvshmem_perftest_put_signal_pingpong(void *data, uint64_t *sig, size_t bytes
     void *args[] = {&d, &sig, &bytes, &iters};
     return nvshmemx_collective_launch((const void *)pingpong_kernel, dim3(1), dim3(threads), args,
                                       0, (hipStream_t)stream);
+}
+
+int nvshmem_perftest_fill_words(uint64_t *words, uint64_t value, size_t nwords, void *stream) {
+    if (!perftest::ready() || !perftest::check_range(words, nwords * sizeof(uint64_t)))
+        return NVSHMEMX_ERROR_INVALID_VALUE;
+    if (nwords == 0) return 0;
+    const unsigned blocks = (unsigned)((nwords + 255) / 256 < 1024 ? (nwords + 255) / 256 : 1024);
+    hipLaunchKernelGGL(fill_words_kernel, dim3(blocks, 1, (unsigned)nvshmem_n_pes()), dim3(256), 0,
+                       (hipStream_t)stream, words, value, nwords);
+    return perftest::launch_status("fill_words");
 }
 
 int nvshmem_perftest_pt2pt_latency(int what, void *data, uint64_t *sig, size_t bytes, int iters,

@@ -156,6 +156,18 @@ def test_put_signal_pingpong(rt):
         rt.free(data); rt.free(sig)
 
 
+def test_fill_words_sets_every_pe_copy(rt):
+    perf = rt.perftest()
+    w = rt.malloc(1000 * 8)
+    rt.fill(w, 0xAB, 1000 * 8)
+    assert perf.nvshmem_perftest_fill_words(w + 8, 0x1122334455667788, 998, None) == 0
+    rt.sync()
+    got = rt.download_all(w, (1000,), np.uint64)
+    assert (got[:, 1:999] == 0x1122334455667788).all()
+    assert (got[:, 0] == 0xABABABABABABABAB).all() and (got[:, 999] == 0xABABABABABABABAB).all()
+    rt.free(w)
+
+
 def test_point_to_point_latency_loops_leave_the_documented_state(rt):
     # kinds of nvshmem_perftest_pt2pt_latency (include/nvshmem_perftest.h): what PE 0 and PE 1 hold
     # afterwards is fixed by the loop, so the timing kernels double as functional checks
