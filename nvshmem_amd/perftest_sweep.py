@@ -107,7 +107,7 @@ def sweep_moe(N, hip, iters):
     def timed_dispatch(launch):
         best = None
         for _ in range(iters + 1):
-            rt.fill(sig, 0, npes * 8)
+            perf.nvshmem_perftest_fill_words(sig, 0, npes, None)
             hip.synchronize()
             e0, e1 = hip.Event(), hip.Event()
             e0.record()
