@@ -35,8 +35,9 @@ MEASURED_TRAFFIC_BYTES = {
     "reducescatter": (2048 + 256) << 20,  # profiles/reducescatter_gather_kernel_float_sum_8pe_8Mi.txt
     "broadcast": (256 + 2048) << 20,      # profiles/segment_copy_kernel_broadcast_8pe_256MiB.txt
     "fcollect": (256 + 4096) << 20,       # profiles/segment_copy_kernel_fcollect_16pe_4Mi_fp32.txt
-    "moe_dispatch": None,                 # not profiled
-    "moe_combine": None,                  # not profiled
+    # fabric traffic: two blocks share a piece and both fetch it (the second from the Infinity Cache)
+    "moe_dispatch": (1840 + 7168) << 20,  # profiles/moe_dispatch_direct_kernel_8pe_8192tok_top8.txt
+    "moe_combine": (7216 + 7168) << 20,   # profiles/moe_combine_kernel_8pe_8192tok_top8.txt
 }
 
 # put_block launch shape: each block is one wavefront that moves a contiguous 1 KiB slice, one

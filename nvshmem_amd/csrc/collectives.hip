@@ -398,8 +398,11 @@ __global__ __launch_bounds__(kThreads) void reduce_scalar_kernel(char *base, uin
 }
 
 // fcollect / broadcast of sources too large to stay in the Infinity Cache: a wavefront stores its
-// piece to at most four destinations; the blocks that share a piece are neighbours in the grid, so
-// all but the first find it in the L2.  Measured with random data: broadcast of 512 MiB to 8 PEs
+// piece to at most four destinations; the blocks that share a piece are neighbours in the grid.
+// Neighbouring work-groups run on different XCDs, so the sharers' loads miss in their L2 and are
+// served by the Infinity Cache (FETCH_SIZE counts the piece once per sharer, HBM reads it once).
+// Putting the sharers on one XCD (8 apart in blockIdx.x) makes L2 serve them and halves FETCH_SIZE,
+// but measured slower (broadcast of 512 MiB: 5.4 against 6.0 TB/s), so they stay neighbours.  Measured with random data: broadcast of 512 MiB to 8 PEs
 // 5.05 -> 6.03 TB/s, fcollect of 16 x 32 MiB 5.25 -> 6.10, of 8 x 64 MiB 5.55 -> 6.2; two or eight
 // destinations per wavefront are slower.  Cache-resident sources keep one wavefront per piece: the
 // split costs them up to 9 %.

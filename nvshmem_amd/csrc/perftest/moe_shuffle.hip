@@ -157,8 +157,10 @@ __global__ void moe_dispatch_pieces_kernel(char *recv, const char *send, const i
 
 // The same work items moved with nvshmem_ptr and plain vector accesses: the piece is loaded into
 // registers (V 16-byte vectors per lane) and stored to up to four of the topk destinations from there;
-// the blocks that share a piece are neighbours in the grid and all but the first find it in the cache,
-// so a source byte crosses the HBM interface once instead of topk times.  Needs 16-byte aligned buffers and
+// the blocks that share a piece are neighbours in the grid; they run on different XCDs, so the second
+// one's load is served by the Infinity Cache rather than by L2 (measured: FETCH_SIZE 1840 MiB for
+// 896 MiB of rows), and a source byte still crosses the HBM interface once instead of topk times.
+// Sharers placed on one XCD hit in L2 (FETCH_SIZE 944 MiB) but the kernel is 11 % slower.  Needs 16-byte aligned buffers and
 // rows; the host picks moe_dispatch_pieces_kernel otherwise.
 template <int V>
 __global__ void moe_dispatch_direct_kernel(char *recv, const char *send, const int32_t *dest_pe,

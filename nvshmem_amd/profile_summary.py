@@ -77,6 +77,20 @@ WORKLOADS = {
         "segment_copy_kernel_broadcast_8pe_256MiB.txt",
         "broadcast: nvshmemx_broadcastmem_on_stream, 8 logical PEs, 256 MiB from PE 3.\n"
         "Algorithmic bytes per launch: 256 MiB read + 8 x 256 MiB written = 2.25 GiB.", (9 * 256) << 20),
+    "moe_dispatch_direct_kernel<1>": (
+        "moe_dispatch_direct_kernel_8pe_8192tok_top8.txt",
+        "MoE dispatch (config 5): 8 logical PEs x 8192 tokens x 7168 bf16, top-8 of 256 experts, Zipf(1.1);\n"
+        "1 KiB work items, at most four copies per wavefront: two neighbouring blocks share a piece.  They run on\n"
+        "different XCDs, so both fetch it through the fabric (FETCH_SIZE counts it twice); the second fetch is\n"
+        "served by the Infinity Cache, not by HBM.  The signalling kernel that follows\n"
+        "(moe_dispatch_signal_kernel) is not part of this figure.\n"
+        "Algorithmic bytes per launch: every row read once (896 MiB) + written 8 times (7 GiB) = 7.875 GiB.",
+        (896 + 7168) << 20),
+    "moe_combine_kernel<true, 2048>": (
+        "moe_combine_kernel_8pe_8192tok_top8.txt",
+        "MoE combine (config 5): every one of the 8 x 65536 row copies fetched back with nvshmemx_getmem_nbi_warp,\n"
+        "2 KiB per single-wavefront block.\n"
+        "Algorithmic bytes per launch: 7 GiB read + 7 GiB written = 14 GiB.", 14 << 30),
     "plain_copy_kernel": (
         "plain_copy_kernel_calibration_1GiB.txt",
         "Counter calibration: plain one-vector-per-thread copy, 1 GiB read + 1 GiB written.", 2 << 30),

@@ -18,6 +18,71 @@ ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
 sys.path.insert(0, ROOT)
 
 
+def moe_plan(np, rng, npes, tokens, topk, experts, zipf_s):
+    """Routing and receive layout of the MoE shuffle: top-k distinct experts per token with
+    P(expert k) ~ (k + 1)^-s (drawn without replacement through Gumbel keys), rows grouped on the
+    destination PE by (expert, source PE, token order).  -> dest_pe, dest_row [npes, tokens * topk],
+    expected [dst, src] row counts, rows received per PE."""
+    logp = -zipf_s * np.log(np.arange(1, experts + 1))
+    per_pe = experts // npes
+    picks = np.empty((npes, tokens, topk), np.int64)
+    for pe in range(npes):
+        keys = logp[None, :] + rng.gumbel(size=(tokens, experts))
+        picks[pe] = np.argsort(-keys, axis=1)[:, :topk]
+    counts = np.stack([np.bincount(picks[pe].reshape(-1), minlength=experts) for pe in range(npes)])  # [src, expert]
+    # segment (expert, src) starts after all segments in front of it on the expert's PE
+    seg = np.zeros((experts, npes), np.int64)
+    recv_rows = np.zeros(npes, np.int64)
+    for d in range(npes):
+        run = 0
+        for e in range(d * per_pe, (d + 1) * per_pe):
+            for src in range(npes):
+                seg[e, src] = run
+                run += counts[src, e]
+        recv_rows[d] = run
+    dest_pe = (picks // per_pe).reshape(npes, -1).astype(np.int32)
+    dest_row = np.empty((npes, tokens * topk), np.int64)
+    for pe in range(npes):
+        flat = picks[pe].reshape(-1)
+        order = np.argsort(flat, kind="stable")                       # copies of one expert in token order
+        rank = np.empty_like(order)
+        starts = np.concatenate(([0], np.cumsum(counts[pe])[:-1]))
+        rank[order] = np.arange(flat.size) - starts[flat[order]]
+        dest_row[pe] = seg[flat, pe] + rank
+    expected = np.stack([[counts[src, d * per_pe:(d + 1) * per_pe].sum() for src in range(npes)]
+                         for d in range(npes)]).astype(np.uint64)
+    return dest_pe, dest_row, expected, recv_rows
+
+
+def moe_shuffle(N, hip, np, rng, noise, iters):
+    """Config 5: 8 PEs x 8192 tokens x 7168 bf16, top-8 of 256 experts, Zipf(1.1): dispatch, then combine."""
+    npes, T, K, E, row = 8, 8192, 8, 256, 7168 * 2
+    dest_pe, dest_row, expected, recv_rows = moe_plan(np, rng, npes, T, K, E, 1.1)
+    cap, rows = int(recv_rows.max()), T * K
+    rt = N.Runtime(npes=npes, symmetric_size=cap * row + rows * row + T * row + (64 << 20))
+    perf = rt.perftest()
+    send = rt.malloc(T * row); recv = rt.malloc(cap * row); out = rt.malloc(rows * row)
+    d_pe = rt.malloc(rows * 4); d_row = rt.malloc(rows * 8)
+    d_expected = rt.malloc(npes * 8); sig = rt.calloc(npes, 8)
+    for pe in range(npes):
+        rt.upload(send, pe, np.roll(noise[:T * row], 4096 * (pe + 1)))
+    rt.upload_all(d_pe, dest_pe); rt.upload_all(d_row, dest_row); rt.upload_all(d_expected, expected)
+    for _ in range(iters):
+        assert perf.nvshmem_perftest_fill_words(sig, 0, npes, None) == 0
+        assert perf.nvshmem_perftest_moe_dispatch_pieces(recv, cap, send, d_pe, d_row, d_expected, sig, T, K, row,
+                                                         1024, 256, None) == 0
+        assert perf.nvshmem_perftest_moe_combine_pieces(out, recv, cap, d_pe, d_row, T, K, row, 2048, 262144, 64,
+                                                        N.SCOPE_WARP, None) == 0
+    hip.synchronize()
+    assert all(rt.read_timeout(pe)[0] == 0 for pe in range(npes)), "a receiver gave up waiting"
+    # the round trip gives every row back: spot check
+    for pe in (0, npes - 1):
+        got = rt.download(out, pe, (64, row), np.uint8)
+        want = np.repeat(np.roll(noise[:T * row], 4096 * (pe + 1)).reshape(T, row)[:8], K, axis=0)
+        assert np.array_equal(got, want), "combine(dispatch(x)) != x"
+    rt.finalize()
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--iters", type=int, default=10)
@@ -110,6 +175,7 @@ def main():
         rt.fcollect("float", dst, src, n, stream=None)
     hip.synchronize()
     rt.finalize()
+    moe_shuffle(N, hip, np, rng, noise, max(2, args.iters // 2))
     print("profile_workloads: done (%d iterations each)" % args.iters)
 
 
