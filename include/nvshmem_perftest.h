@@ -215,8 +215,8 @@ int nvshmem_perftest_moe_combine_ex(void *out, const void *recv, size_t recv_cap
  * 2048 or 4096) of one token's row, pushed to all of its topk destinations - then one block per PE
  * that publishes the row counts through the signal words and waits for the expected ones.  A block of
  * `threads` (a multiple of 64) takes threads / 64 tokens.  With 16-byte aligned buffers and rows the
- * piece is loaded once and stored through nvshmem_ptr; otherwise it is moved with topk
- * nvshmemx_putmem_nbi_warp calls. */
+ * piece is loaded once and stored through nvshmem_ptr; otherwise (or when the environment variable
+ * NVSHMEM_PERFTEST_MOE_PUTS is set) it is moved with topk nvshmemx_putmem_nbi_warp calls. */
 int nvshmem_perftest_moe_dispatch_pieces(void *recv, size_t recv_cap_rows, const void *send,
                                          const int32_t *dest_pe, const int64_t *dest_row,
                                          const uint64_t *expected, uint64_t *sig, int tokens, int topk,

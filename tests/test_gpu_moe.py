@@ -108,6 +108,14 @@ def test_moe_shuffle_small(scope):
         _shuffle(rt, 8, 33, 3, 64, 200 + 6, 2, 128, scope, check_exchange=False)   # ragged rows
 
 
+def test_moe_dispatch_pieces_through_the_put_api(monkeypatch):
+    """NVSHMEM_PERFTEST_MOE_PUTS selects the nvshmemx_putmem_nbi_warp form of the short work items also
+    for aligned rows (without it only rows that are not 16-byte aligned take it)."""
+    monkeypatch.setenv("NVSHMEM_PERFTEST_MOE_PUTS", "1")
+    with runtime(8, 1 << 28) as rt:
+        _shuffle(rt, 8, 128, 8, 64, 4096 + 1024, 4, 256, N.SCOPE_WARP, check_exchange=False)
+
+
 def test_moe_routing_table_outside_the_buffer_is_skipped_not_written():
     with runtime(4, 1 << 24) as rt:
         perf = rt.perftest()
