@@ -166,6 +166,29 @@ def test_ring_put_get_256MiB_16_blocks(rt, is_get):
     rt.free(src); rt.free(dst)
 
 
+def test_ring_put_get_8MiB_to_128MiB_and_the_gpu_filling_shape(rt):
+    # the upper half of the sweep (config 2: 8 B ... 256 MiB), block counts 1 / 4 / 16 in turn, and
+    # the launch shape the benchmark uses (one wavefront per KiB) at 256 MiB
+    perf = rt.perftest()
+    size_max = 1 << 28
+    src = rt.malloc(size_max); dst = rt.malloc(size_max)
+    data = O.fill_all("bytes", NPES, size_max, 3)
+    rt.upload_all(src, data)
+    cases = [(1 << p, (1, 4, 16)[p % 3], 1024, p % 2) for p in range(23, 28)]
+    cases += [(size_max, size_max >> 10, 64, 0), (size_max, size_max >> 10, 64, 1), ((1 << 27) + 12345, 1 << 17, 64, 0)]
+    for size, blocks, threads, is_get in cases:
+        rt.fill(dst, 0, size_max)
+        note("ring_rma size=%d blocks=%d threads=%d get=%d" % (size, blocks, threads, is_get))
+        assert perf.nvshmem_perftest_ring_rma(dst, src, size, blocks, threads, N.SCOPE_BLOCK, is_get, 1, None) == 0
+        rt.sync()
+        for pe in (0, 3, NPES - 1):
+            got = rt.download(dst, pe, (min(size + 4096, size_max),), np.uint8)
+            want = data[(pe + 1) % NPES] if is_get else data[(pe - 1) % NPES]
+            assert np.array_equal(got[:size], want[:size]), (size, blocks, pe)
+            assert (got[size:] == 0).all(), (size, blocks, pe)
+    rt.free(src); rt.free(dst)
+
+
 def test_ring_rejects_ranges_outside_the_heap(rt):
     perf = rt.perftest()
     a = rt.malloc(4096)
