@@ -408,6 +408,10 @@ NVSHMEMI_STAMP_MEM_COLL(nvshmemx, _block, NVSHMEMI_THREADGROUP_BLOCK)
 NVSHMEMI_REPT_FOR_ALL_REDUCE_TYPES_AND_OPS(NVSHMEMI_STAMP_REDUCE)
 #undef NVSHMEMI_STAMP_REDUCE
 
+/* barrier among the PEs of `team`, called by one warpgroup (256 threads: four wavefronts) per PE
+ * (reference nvshmemx_coll_api.h:118, nvshmemx_coll_defines.cuh:52) */
+NVSHMEMI_DEV int nvshmemx_barrier_warpgroup(nvshmem_team_t team) { return nvshmemi_barrier_warpgroup(team); }
+
 /* (value, location) maximum, block scope only (reference nvshmemx_coll_defines.cuh:210-214) */
 NVSHMEMI_DEV int nvshmemx_double2_maxloc_reduce_block(nvshmem_team_t team, double2 *dest,
                                                       const double2 *source, size_t nreduce) {

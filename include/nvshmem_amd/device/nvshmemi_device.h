@@ -676,6 +676,50 @@ NVSHMEMI_DEVICE_INLINE void nvshmemi_barrier_threadgroup(nvshmem_team_t team = N
     nvshmemi_sync_threadgroup<SCOPE>(team);
 }
 
+/* Barrier called by one warpgroup per PE (reference nvshmemx_barrier_warpgroup, its fourth thread
+ * group scope: four warps that meet at a named hardware barrier, threadgroup/
+ * nvshmemi_common_device_defines.cuh:76-110).  gfx950 has no barrier for part of a work-group, so the
+ * wavefronts of the warpgroup - threads [256 g, 256 g + 256) of the block - meet at two words of
+ * the team's sync row instead, an arrival count and a generation: every wavefront reads the
+ * generation and adds one to the count; the last one to arrive puts the count back to zero and
+ * advances the generation, the others wait for the generation to change.  The count is zero between
+ * meetings, so groups of different sizes (a short last group) can follow each other.  The
+ * warpgroup's first thread then runs the thread-scope barrier among the PEs, and a second meeting
+ * releases the others.  As with the warp scope, only one warpgroup per PE may be inside a barrier
+ * on a given team at a time. */
+NVSHMEMI_DEVICE_INLINE void nvshmemi_amd_warpgroup_meet(nvshmem_team_t team) {
+    const unsigned tid = nvshmemi_amd_block_tid(), nthr = nvshmemi_amd_block_size();
+    const unsigned first = tid & ~(unsigned)(NVSHMEMI_AMD_WARPGROUP_SIZE - 1);
+    const unsigned members = nthr - first < NVSHMEMI_AMD_WARPGROUP_SIZE ? nthr - first : NVSHMEMI_AMD_WARPGROUP_SIZE;
+    const uint64_t waves = (members + NVSHMEMI_WARP_SIZE - 1) / NVSHMEMI_WARP_SIZE;
+    uint64_t *count = nvshmemi_device_state_d.team_sync +
+                      ((size_t)team * NVSHMEMI_AMD_MAX_PES + (size_t)nvshmemi_amd_my_pe()) * NVSHMEMI_AMD_TEAM_SYNC_WORDS +
+                      NVSHMEMI_AMD_WARPGROUP_ARRIVE_WORD;
+    uint64_t *generation = count + 1;
+    const uint64_t seen = __hip_atomic_load(generation, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    /* the generation is read, and this wavefront's earlier memory operations are done, before it
+     * reports its arrival */
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
+    if ((tid & (NVSHMEMI_WARP_SIZE - 1)) == 0) {
+        if (__hip_atomic_fetch_add(count, (uint64_t)1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) + 1 == waves) {
+            __hip_atomic_store(count, (uint64_t)0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            /* release: the count is back at zero before anyone sees the new generation */
+            __hip_atomic_store(generation, seen + 1, __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_AGENT);
+        } else {
+            nvshmemi_wait_until<uint64_t>(generation, NVSHMEM_CMP_NE, seen);
+        }
+    }
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup");
+}
+NVSHMEMI_DEVICE_INLINE int nvshmemi_barrier_warpgroup(nvshmem_team_t team) {
+    if (nvshmemi_amd_team_view(team).size <= 0) return 1; /* the calling PE is not a member */
+    nvshmemi_amd_warpgroup_meet(team);
+    if ((nvshmemi_amd_block_tid() & (NVSHMEMI_AMD_WARPGROUP_SIZE - 1)) == 0)
+        nvshmemi_barrier_threadgroup<NVSHMEMI_THREADGROUP_THREAD>(team);
+    nvshmemi_amd_warpgroup_meet(team);
+    return 0;
+}
+
 /* ------------------------------------------------------------------------------------------------
  * Reduction operator (reference perform_gpu_rdxn, coll/reduce.cuh:49-105): computed in the element
  * type; 16-bit floats add/multiply in fp32 and round to nearest-even once per step, which equals

@@ -216,6 +216,10 @@ typedef struct {
 #define NVSHMEMI_AMD_LL_BCAST_MAX_BYTES 16384 /* broadcast: one contribution, up to a whole buffer */
 #define NVSHMEMI_AMD_LL_COUNT_WORD (NVSHMEMI_AMD_MAX_PES + 1)
 #define NVSHMEMI_AMD_LL_DONE_WORD (NVSHMEMI_AMD_MAX_PES + 2)
+/* Words of a PE's team sync row where the wavefronts of nvshmemx_barrier_warpgroup meet: the
+ * arrival count (zero between meetings) and, one word on, the generation. */
+#define NVSHMEMI_AMD_WARPGROUP_ARRIVE_WORD (NVSHMEMI_AMD_MAX_PES + 3)
+#define NVSHMEMI_AMD_WARPGROUP_SIZE 256 /* four wavefronts, as the reference's warpgroup is four warps */
 
 typedef struct nvshmemi_device_state {
     uint32_t version;     /* (1 << 16) + sizeof(struct) */

@@ -172,6 +172,11 @@ int nvshmem_perftest_team_query(int *out, int team_a, int team_b, void *stream);
 /* device_barrier among the members of `team` (nvshmem_barrier(team) / nvshmem_team_sync(team)). */
 int nvshmem_perftest_device_team_barrier(uint64_t *counter, uint64_t *errors, int rounds, int team,
                                          int scope, int threads, void *stream);
+/* The same rounds run by ONE warpgroup of every member through nvshmemx_barrier_warpgroup: warpgroup
+ * `group` = threads [256 group, 256 group + 256) of the one block per PE (the last group may be
+ * shorter); the block's other threads leave at once. */
+int nvshmem_perftest_device_warpgroup_barrier(uint64_t *counter, uint64_t *errors, int rounds, int team,
+                                              int group, int threads, void *stream);
 /* `rounds` barriers; before round r each PE stores r into its `counter`, after the barrier it reads
  * every PE's counter and adds to its own errors[0] the number that are < r.  counter and errors
  * hold one uint64 each. */

@@ -144,6 +144,7 @@ def load_perftest():
         "nvshmem_perftest_device_team_coll": [i32, i32, vp, vp, sz, i32, i32, i32, vp],
         "nvshmem_perftest_device_team_coll_loop": [i32, i32, vp, vp, sz, i32, i32, i32, i32, vp],
         "nvshmem_perftest_team_query": [vp, i32, i32, vp],
+        "nvshmem_perftest_device_warpgroup_barrier": [vp, vp, i32, i32, i32, i32, vp],
         "nvshmem_perftest_device_team_barrier": [vp, vp, i32, i32, i32, i32, vp],
         "nvshmem_perftest_device_reducescatter": [i32, i32, vp, vp, sz, i32, i32, vp],
         "nvshmem_perftest_device_broadcast": [vp, vp, sz, i32, i32, i32, vp],

@@ -154,6 +154,32 @@ __global__ void team_barrier_kernel(uint64_t *counter, uint64_t *errors, int rou
     if (threadIdx.x == 0) *(uint64_t *)nvshmem_ptr(errors, me) += bad;
 }
 
+// nvshmemx_barrier_warpgroup: warpgroup `group` (threads [256 group, 256 group + 256) of the block) of
+// every member runs the rounds of team_barrier_kernel; the other threads of the block leave at once.
+__global__ void warpgroup_barrier_kernel(uint64_t *counter, uint64_t *errors, int rounds, nvshmem_team_t team,
+                                         int group) {
+    const int idx = nvshmem_team_my_pe(team), np = nvshmem_team_n_pes(team);
+    if (idx < 0 || (int)(threadIdx.x / NVSHMEMI_AMD_WARPGROUP_SIZE) != group) return;
+    const unsigned local = threadIdx.x % NVSHMEMI_AMD_WARPGROUP_SIZE;
+    const unsigned rest = blockDim.x - group * NVSHMEMI_AMD_WARPGROUP_SIZE;
+    const unsigned members = rest < NVSHMEMI_AMD_WARPGROUP_SIZE ? rest : NVSHMEMI_AMD_WARPGROUP_SIZE;
+    const bool leader = local == 0;
+    const int me = nvshmem_my_pe();
+    uint64_t *my_counter = (uint64_t *)nvshmem_ptr(counter, me);
+    uint64_t bad = 0;
+    for (int r = 1; r <= rounds; ++r) {
+        // the LAST thread of the warpgroup writes and the first one checks: the barrier has to order the
+        // wavefronts of the group as well as the PEs
+        if (local == members - 1) *my_counter = (uint64_t)r;
+        nvshmemx_barrier_warpgroup(team);
+        if (leader)
+            for (int q = 0; q < np; ++q)
+                bad += nvshmem_uint64_g(counter, nvshmem_team_translate_pe(team, q, NVSHMEM_TEAM_WORLD)) < (uint64_t)r;
+        nvshmemx_barrier_warpgroup(team);
+    }
+    if (leader) *(uint64_t *)nvshmem_ptr(errors, me) += bad;
+}
+
 // Many collectives back to back without any barrier in between (sync_between = 0) or with one
 // after every check (1): round r fills src[i] = gen(me, r, i), then runs an int32 sum reduce of n
 // elements, a broadcast of the same n elements from member r % npes, an fcollect of fc_bytes per
@@ -381,6 +407,18 @@ int nvshmem_perftest_device_team_barrier(uint64_t *counter, uint64_t *errors, in
         scope, team_barrier_kernel<NVSHMEM_PERFTEST_SCOPE_BLOCK>,
         team_barrier_kernel<NVSHMEM_PERFTEST_SCOPE_WARP>, team_barrier_kernel<NVSHMEM_PERFTEST_SCOPE_THREAD>,
         threads, stream, counter, errors, rounds, (nvshmem_team_t)team);
+}
+
+int nvshmem_perftest_device_warpgroup_barrier(uint64_t *counter, uint64_t *errors, int rounds, int team,
+                                              int group, int threads, void *stream) {
+    if (!perftest::ready() || !perftest::check_launch(1, threads) || group < 0 ||
+        group * NVSHMEMI_AMD_WARPGROUP_SIZE >= threads ||
+        !perftest::check_range(counter, sizeof(uint64_t)) || !perftest::check_range(errors, sizeof(uint64_t)))
+        return NVSHMEMX_ERROR_INVALID_VALUE;
+    nvshmem_team_t t = team;
+    void *args[] = {(void *)&counter, (void *)&errors, (void *)&rounds, (void *)&t, (void *)&group};
+    return nvshmemx_collective_launch((const void *)warpgroup_barrier_kernel, dim3(1), dim3(threads), args, 0,
+                                      (hipStream_t)stream);
 }
 
 int nvshmem_perftest_coll_sequence(int32_t *src, int32_t *dst, uint64_t *check, int n, int fc_bytes,

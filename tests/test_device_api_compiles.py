@@ -42,7 +42,7 @@ def _names():
               "nvshmem_int_broadcast", "nvshmem_int_fcollect", "nvshmem_int_sum_reduce",
               "nvshmem_int_sum_reducescatter", "nvshmem_quiet", "nvshmem_fence", "nvshmem_ptr", "nvshmem_my_pe",
               "nvshmem_n_pes", "nvshmem_team_my_pe", "nvshmem_team_n_pes", "nvshmem_team_translate_pe",
-              "nvshmemx_double2_maxloc_reduce_block"]
+              "nvshmemx_double2_maxloc_reduce_block", "nvshmemx_barrier_warpgroup"]
     for f in ("wait_until", "wait_until_all", "wait_until_any", "wait_until_some", "wait_until_all_vector",
               "wait_until_any_vector", "wait_until_some_vector", "test", "test_all", "test_any", "test_some",
               "test_all_vector", "test_any_vector", "test_some_vector"):

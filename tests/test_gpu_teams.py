@@ -348,6 +348,30 @@ def test_device_scope_collectives_on_teams(rt, scope, threads, n):
         rt.team_destroy(t)
 
 
+def test_warpgroup_barrier_on_world_and_strided_teams(rt):
+    """nvshmemx_barrier_warpgroup: one group of up to 256 threads of every member's block runs the
+    barrier rounds while the block's other threads have left; first, middle and short last group."""
+    perf = rt.perftest()
+    odd = rt.team_split_strided(N.TEAM_WORLD, 1, 2, NPES // 2)
+    for team, members in ((N.TEAM_WORLD, list(range(NPES))), (odd, list(range(1, NPES, 2)))):
+        for threads, group in ((256, 0), (512, 1), (768, 1), (640, 2), (1024, 3), (64, 0)):
+            note("warpgroup barrier team=%d threads=%d group=%d" % (team, threads, group))
+            counter = rt.calloc(1, 8); errors = rt.calloc(1, 8)
+            assert perf.nvshmem_perftest_device_warpgroup_barrier(counter, errors, 40, team, group, threads, None) == 0
+            rt.sync()
+            assert (rt.download_all(errors, (1,), np.uint64) == 0).all()
+            cnt = rt.download_all(counter, (1,), np.uint64)
+            for pe in range(NPES):
+                assert cnt[pe, 0] == (40 if pe in members else 0)
+            flag, rec = rt.read_timeout(0)
+            assert flag == 0, rec
+            rt.free(counter); rt.free(errors)
+    counter = rt.calloc(1, 8); errors = rt.calloc(1, 8)
+    assert perf.nvshmem_perftest_device_warpgroup_barrier(counter, errors, 1, N.TEAM_WORLD, 2, 512, None) != 0
+    rt.free(counter); rt.free(errors)
+    rt.team_destroy(odd)
+
+
 def test_maxloc_reduce_and_device_identification(rt):
     """nvshmemx_double2_maxloc_reduce_block on the world team, a strided team and the rows of a 2-D
     split, with ties and NaNs in the values; plus what the device-side identification calls report."""
