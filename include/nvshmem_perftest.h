@@ -90,6 +90,22 @@ enum {
 int nvshmem_perftest_pt2pt_latency(int what, void *data, uint64_t *sig, size_t bytes, int iters,
                                    int threads, void *stream);
 
+/* Element-wise bandwidth kernels in the shape of perftest/device/pt-to-pt/shmem_p_bw.cu:43-84,
+ * shmem_g_bw.cu, shmem_st_bw.cu and shmem_atomic_bw.cu: every thread handles single elements of
+ * elem_bytes (1, 2, 4 or 8; ADD: 4 or 8), consecutive threads consecutive elements, grid-stride over
+ * nelems.  P: nvshmem_<uintN>_p(dest + i, src[i], right neighbour); G: dest[i] = nvshmem_<uintN>_g(src
+ * + i, right neighbour); ST: the same as P by a plain store through nvshmem_ptr; ADD:
+ * nvshmem_<uintN>_atomic_add(dest + i, src[i], right neighbour).  After P / ST / ADD PE p's dest holds
+ * (ADD: has grown by) PE p-1's src, after G PE p+1's. */
+enum {
+    NVSHMEM_PERFTEST_ELEMENT_P = 0,
+    NVSHMEM_PERFTEST_ELEMENT_G = 1,
+    NVSHMEM_PERFTEST_ELEMENT_ST = 2,
+    NVSHMEM_PERFTEST_ELEMENT_ADD = 3
+};
+int nvshmem_perftest_element_bw(int what, int elem_bytes, void *dest, const void *src, size_t nelems,
+                                int blocks_per_pe, int threads, void *stream);
+
 /* Ring allreduce of int32 built from put_signal_nbi + signal_wait_until, the algorithm of
  * examples/ring-reduce.cu:88-144: reduce phase around the ring, then broadcast phase.  nreduce must
  * be a multiple of blocks*chunk_elems.  signal holds `blocks` words (zero before the call; the

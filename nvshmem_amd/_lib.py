@@ -153,6 +153,7 @@ def load_perftest():
         "nvshmem_perftest_device_maxloc": [i32, vp, vp, sz, i32, i32, vp, vp],
         "nvshmem_perftest_fill_words": [vp, u64, sz, vp],
         "nvshmem_perftest_pt2pt_latency": [i32, vp, vp, sz, i32, i32, vp],
+        "nvshmem_perftest_element_bw": [i32, i32, vp, vp, sz, i32, i32, vp],
         "nvshmem_perftest_moe_dispatch": [vp, sz, vp, vp, vp, vp, vp, i32, i32, sz, i32, i32, vp],
         "nvshmem_perftest_moe_dispatch_ex": [vp, sz, vp, vp, vp, vp, vp, i32, i32, sz, i32, i32, i32, vp],
         "nvshmem_perftest_moe_dispatch_pieces": [vp, sz, vp, vp, vp, vp, vp, i32, i32, sz, i32, i32, vp],

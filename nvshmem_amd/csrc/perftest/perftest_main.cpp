@@ -5,9 +5,12 @@
 // perftest/device/coll/*_latency.cu).
 //
 //   nvshmem_perftest <test> [--npes N] [--min BYTES] [--max BYTES] [--iters K] [--warmup W]
-//                           [--blocks B] [--threads T] [--scope thread|warp|block]
+//                           [--blocks B] [--threads T] [--scope thread|warp|block] [--elem 1|2|4|8]
 //
 // tests: put_bw get_bw                      device put/get, every PE to its right neighbour
+//        p_bw g_bw st_bw atomic_bw          one element per thread and call (--elem 1|2|4|8 bytes):
+//                                           nvshmem_<T>_p / _g, a plain store through nvshmem_ptr,
+//                                           nvshmem_<T>_atomic_add
 //        reduce reducescatter fcollect alltoall broadcast
 //                                           host-launched collectives on a stream (fp32 sum for the
 //                                           reductions); size = bytes each PE contributes
@@ -39,12 +42,13 @@ struct Options {
     int iters = 20, warmup = 5;
     int blocks = 0, threads = 0;  // 0: a shape that fills the GPU
     int scope = NVSHMEM_PERFTEST_SCOPE_BLOCK;
+    int elem = 8;  // element size of the element-wise tests
 };
 
 [[noreturn]] void usage(const char *why) {
-    fprintf(stderr, "nvshmem_perftest: %s\nusage: nvshmem_perftest <put_bw|get_bw|reduce|reducescatter|fcollect|"
+    fprintf(stderr, "nvshmem_perftest: %s\nusage: nvshmem_perftest <put_bw|get_bw|p_bw|g_bw|st_bw|atomic_bw|reduce|reducescatter|fcollect|"
                     "alltoall|broadcast|coll_latency|barrier_latency|pt2pt_latency|host_put_bw|host_get_bw> [--npes N] [--min B] [--max B] [--iters K] "
-                    "[--warmup W] [--blocks B] [--threads T] [--scope thread|warp|block]\n", why);
+                    "[--warmup W] [--blocks B] [--threads T] [--scope thread|warp|block] [--elem 1|2|4|8]\n", why);
     exit(2);
 }
 
@@ -78,6 +82,7 @@ Options parse(int argc, char **argv) {
         else if (a == "--warmup") o.warmup = atoi(next());
         else if (a == "--blocks") o.blocks = atoi(next());
         else if (a == "--threads") o.threads = atoi(next());
+        else if (a == "--elem") o.elem = atoi(next());
         else if (a == "--scope") {
             const std::string s = next();
             if (s == "thread") o.scope = NVSHMEM_PERFTEST_SCOPE_THREAD;
@@ -87,6 +92,8 @@ Options parse(int argc, char **argv) {
         } else usage(("unknown option " + a).c_str());
     }
     if (o.iters < 1 || o.warmup < 0 || o.min_bytes < 1 || o.max_bytes < o.min_bytes) usage("bad range");
+    if (o.elem != 1 && o.elem != 2 && o.elem != 4 && o.elem != 8) usage("bad element size");
+    if (o.test == "atomic_bw" && o.elem < 4) usage("atomics are 4 or 8 bytes wide");
     return o;
 }
 
@@ -162,6 +169,34 @@ int run_rma(const Options &o, bool is_get) {
     }
     print_table(is_get ? "shmem_get_bw" : "shmem_put_bw", scope_name(o.scope), "BW", "GB/s per PE", sizes, gbs);
     printf("# %d PEs move that payload at once: aggregate payload = npes x BW, HBM traffic = 2 x that\n", o.npes);
+    nvshmem_free(src);
+    nvshmem_free(dst);
+    return 0;
+}
+
+// shmem_p_bw / shmem_g_bw / shmem_st_bw / shmem_atomic_bw: size = bytes one PE moves per launch
+int run_element(const Options &o, int what) {
+    static const char *jobs[] = {"shmem_p_bw", "shmem_g_bw", "shmem_st_bw", "shmem_atomic_bw"};
+    void *src = nvshmem_malloc(o.max_bytes), *dst = nvshmem_malloc(o.max_bytes);
+    if (!src || !dst) return 1;
+    std::vector<size_t> sizes = sweep(o, (size_t)o.elem);
+    std::vector<double> gbs;
+    for (size_t bytes : sizes) {
+        const size_t nelems = bytes / (size_t)o.elem;
+        // default: 256 threads, four elements per thread, at most 2^20 blocks per PE
+        const int threads = o.threads ? o.threads : 256;
+        long blocks = o.blocks ? o.blocks : (long)((nelems + 4 * (size_t)threads - 1) / (4 * (size_t)threads));
+        if (blocks < 1) blocks = 1;
+        if (blocks > (1 << 20)) blocks = 1 << 20;
+        const double ms = time_ms([&] {
+            return nvshmem_perftest_element_bw(what, o.elem, dst, src, nelems, (int)blocks, threads, nullptr);
+        }, o.iters, o.warmup);
+        gbs.push_back((double)bytes / ms / 1e6);
+    }
+    char scope[32];
+    snprintf(scope, sizeof scope, "%d-byte", o.elem);
+    print_table(jobs[what], scope, "BW", "GB/s per PE", sizes, gbs);
+    printf("# %d PEs move that payload at once: aggregate payload = npes x BW\n", o.npes);
     nvshmem_free(src);
     nvshmem_free(dst);
     return 0;
@@ -321,7 +356,8 @@ int main(int argc, char **argv) {
     const Options o = parse(argc, argv);
     const bool device_lat = o.test == "coll_latency" || o.test == "barrier_latency" || o.test == "pt2pt_latency";
     // heap: source and dest of the largest size, times npes for the collectives
-    const bool rma = o.test == "put_bw" || o.test == "get_bw" || o.test == "pt2pt_latency" ||
+    const bool rma = o.test == "put_bw" || o.test == "get_bw" || o.test == "pt2pt_latency" || o.test == "p_bw" ||
+                     o.test == "g_bw" || o.test == "st_bw" || o.test == "atomic_bw" ||
                      o.test == "host_put_bw" || o.test == "host_get_bw";
     Options eff = o;
     if (device_lat && o.max_bytes > ((size_t)1 << 20)) eff.max_bytes = (size_t)1 << 20;
@@ -333,6 +369,10 @@ int main(int argc, char **argv) {
     int rc;
     if (o.test == "put_bw") rc = run_rma(eff, false);
     else if (o.test == "get_bw") rc = run_rma(eff, true);
+    else if (o.test == "p_bw") rc = run_element(eff, NVSHMEM_PERFTEST_ELEMENT_P);
+    else if (o.test == "g_bw") rc = run_element(eff, NVSHMEM_PERFTEST_ELEMENT_G);
+    else if (o.test == "st_bw") rc = run_element(eff, NVSHMEM_PERFTEST_ELEMENT_ST);
+    else if (o.test == "atomic_bw") rc = run_element(eff, NVSHMEM_PERFTEST_ELEMENT_ADD);
     else if (o.test == "reduce") rc = run_host_collective(eff, kReduce);
     else if (o.test == "reducescatter") rc = run_host_collective(eff, kReducescatter);
     else if (o.test == "fcollect") rc = run_host_collective(eff, kFcollect);

@@ -1,5 +1,5 @@
 // Point-to-point kernels written against the public device API: ring put/get in the three scopes,
-// scalar p/g, signal operations, bounded waits, put_signal ping-pong and the ring allreduce built
+// scalar p/g, element-wise p/g/store/atomic-add bandwidth, signal operations, bounded waits, put_signal ping-pong and the ring allreduce built
 // from put_signal + signal_wait_until.
 //
 // Counterparts in the reference tree: perftest/device/pt-to-pt/shmem_put_bw.cu:21-60,
@@ -209,6 +209,59 @@ __global__ void plain_copy_kernel(nvshmemi_v4u *dst, const nvshmemi_v4u *src, si
     if (i < nvec) dst[i] = src[i];
 }
 
+// Element-wise bandwidth in the shape of the reference's shmem_p_bw.cu:43-84, shmem_g_bw.cu,
+// shmem_st_bw.cu and shmem_atomic_bw.cu: every thread moves single elements, consecutive threads
+// consecutive elements, every PE to (P, ST, ADD) or from (G) its right neighbour.
+template <typename T> struct element_api;
+#define ELEMENT_API(T, NAME)                                                                          \
+    template <> struct element_api<T> {                                                               \
+        static __device__ __forceinline__ void p(T *d, T v, int pe) { nvshmem_##NAME##_p(d, v, pe); } \
+        static __device__ __forceinline__ T g(const T *s, int pe) { return nvshmem_##NAME##_g(s, pe); } \
+    };
+ELEMENT_API(uint8_t, uint8)
+ELEMENT_API(uint16_t, uint16)
+ELEMENT_API(uint32_t, uint32)
+ELEMENT_API(uint64_t, uint64)
+#undef ELEMENT_API
+__device__ __forceinline__ void element_add(uint8_t *, uint8_t, int) {}
+__device__ __forceinline__ void element_add(uint16_t *, uint16_t, int) {}
+__device__ __forceinline__ void element_add(uint32_t *d, uint32_t v, int pe) { nvshmem_uint32_atomic_add(d, v, pe); }
+__device__ __forceinline__ void element_add(uint64_t *d, uint64_t v, int pe) { nvshmem_uint64_atomic_add(d, v, pe); }
+
+template <typename T, int WHAT>
+__global__ void element_bw_kernel(T *dest, const T *src, size_t n) {
+    const int me = nvshmem_my_pe();
+    const int peer = (me + 1 == nvshmem_n_pes()) ? 0 : me + 1;
+    const size_t stride = (size_t)gridDim.x * blockDim.x;
+    const T *my_src = (const T *)nvshmem_ptr(src, me);
+    for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += stride) {
+        if (WHAT == NVSHMEM_PERFTEST_ELEMENT_P) element_api<T>::p(dest + i, my_src[i], peer);
+        else if (WHAT == NVSHMEM_PERFTEST_ELEMENT_G) ((T *)nvshmem_ptr(dest, me))[i] = element_api<T>::g(src + i, peer);
+        else if (WHAT == NVSHMEM_PERFTEST_ELEMENT_ST) ((T *)nvshmem_ptr(dest, peer))[i] = my_src[i];
+        else element_add(dest + i, my_src[i], peer);
+    }
+}
+
+template <typename T>
+int launch_element(int what, void *dest, const void *src, size_t n, int blocks, int threads, hipStream_t stream) {
+    const dim3 grid((unsigned)blocks, 1, (unsigned)nvshmem_n_pes());
+    switch (what) {
+        case NVSHMEM_PERFTEST_ELEMENT_P:
+            hipLaunchKernelGGL((element_bw_kernel<T, NVSHMEM_PERFTEST_ELEMENT_P>), grid, dim3(threads), 0, stream, (T *)dest, (const T *)src, n);
+            break;
+        case NVSHMEM_PERFTEST_ELEMENT_G:
+            hipLaunchKernelGGL((element_bw_kernel<T, NVSHMEM_PERFTEST_ELEMENT_G>), grid, dim3(threads), 0, stream, (T *)dest, (const T *)src, n);
+            break;
+        case NVSHMEM_PERFTEST_ELEMENT_ST:
+            hipLaunchKernelGGL((element_bw_kernel<T, NVSHMEM_PERFTEST_ELEMENT_ST>), grid, dim3(threads), 0, stream, (T *)dest, (const T *)src, n);
+            break;
+        default:
+            hipLaunchKernelGGL((element_bw_kernel<T, NVSHMEM_PERFTEST_ELEMENT_ADD>), grid, dim3(threads), 0, stream, (T *)dest, (const T *)src, n);
+            break;
+    }
+    return perftest::launch_status("element_bw");
+}
+
 template <int SCOPE>
 int launch_ring(bool is_get, char *dest, const char *src, size_t bytes, int blocks, int threads,
                 hipStream_t stream) {
@@ -256,6 +309,24 @@ int nvshmem_perftest_ring_rma(void *dest, const void *src, size_t bytes, int blo
         }
     }
     return rc;
+}
+
+int nvshmem_perftest_element_bw(int what, int elem_bytes, void *dest, const void *src, size_t nelems,
+                                int blocks_per_pe, int threads, void *stream) {
+    const bool size_ok = elem_bytes == 1 || elem_bytes == 2 || elem_bytes == 4 || elem_bytes == 8;
+    if (!perftest::ready() || what < 0 || what > NVSHMEM_PERFTEST_ELEMENT_ADD || !size_ok ||
+        (what == NVSHMEM_PERFTEST_ELEMENT_ADD && elem_bytes < 4) ||
+        ((uintptr_t)dest % elem_bytes) || ((uintptr_t)src % elem_bytes) ||
+        !perftest::check_launch(blocks_per_pe, threads) ||
+        !perftest::check_range(dest, nelems * elem_bytes) || !perftest::check_range(src, nelems * elem_bytes))
+        return NVSHMEMX_ERROR_INVALID_VALUE;
+    if (nelems == 0) return 0;
+    switch (elem_bytes) {
+        case 1: return launch_element<uint8_t>(what, dest, src, nelems, blocks_per_pe, threads, (hipStream_t)stream);
+        case 2: return launch_element<uint16_t>(what, dest, src, nelems, blocks_per_pe, threads, (hipStream_t)stream);
+        case 4: return launch_element<uint32_t>(what, dest, src, nelems, blocks_per_pe, threads, (hipStream_t)stream);
+        default: return launch_element<uint64_t>(what, dest, src, nelems, blocks_per_pe, threads, (hipStream_t)stream);
+    }
 }
 
 int nvshmem_perftest_plain_copy(void *dst, const void *src, size_t bytes, void *stream) {

@@ -69,6 +69,16 @@ def test_device_latency_tables():
     assert "barrier_latency" in out
 
 
+def test_element_wise_bandwidth_tables():
+    for test, job, elem in (("p_bw", "shmem_p_bw", "8"), ("g_bw", "shmem_g_bw", "4"), ("st_bw", "shmem_st_bw", "1"),
+                            ("atomic_bw", "shmem_atomic_bw", "8")):
+        rows = _rows(_run(test, "--min", "1k", "--max", "4m", "--iters", "5", "--elem", elem), job)
+        assert [r[0] for r in rows] == [1024 << i for i in range(13)] and all(r[1] == elem + "-byte" for r in rows)
+        assert all(v > 0 for _, _, v in rows), (job, rows)
+    proc = subprocess.run([DRIVER, "atomic_bw", "--elem", "2"], stdout=subprocess.PIPE, stderr=subprocess.PIPE, timeout=100)
+    assert proc.returncode == 2 and b"atomics" in proc.stderr
+
+
 def test_bad_arguments_are_refused():
     proc = subprocess.run([DRIVER, "nonsense"], stdout=subprocess.PIPE, stderr=subprocess.PIPE, timeout=100)
     assert proc.returncode == 2 and b"usage" in proc.stderr

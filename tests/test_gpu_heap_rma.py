@@ -189,6 +189,39 @@ def test_ring_put_get_8MiB_to_128MiB_and_the_gpu_filling_shape(rt):
     rt.free(src); rt.free(dst)
 
 
+@pytest.mark.parametrize("elem", [1, 2, 4, 8])
+def test_element_wise_p_g_store_and_atomic_add(rt, elem):
+    """One element per thread and call (the reference's shmem_p_bw / g_bw / st_bw / atomic_bw shape):
+    the ring shift of the oracle for p, g and the plain store; element-wise wrapping sums for add."""
+    perf = rt.perftest()
+    kinds = [(0, "p"), (1, "g"), (2, "st")] + ([(3, "add")] if elem >= 4 else [])
+    for nelems, blocks, threads in ((1, 1, 64), (1000, 3, 64), (70001, 16, 256), (1 << 18, 64, 1024)):
+        size = nelems * elem
+        src = rt.malloc(size + 64); dst = rt.malloc(size + 64)
+        data = O.fill_all("bytes", NPES, size, 20 + elem)[:, :size]
+        start = O.fill_all("bytes", NPES, size + 64, 30 + elem)[:, :size + 64]
+        rt.upload_all(src, data)
+        for what, name in kinds:
+            rt.upload_all(dst, start)
+            note("element_bw %s elem=%d nelems=%d blocks=%d threads=%d" % (name, elem, nelems, blocks, threads))
+            assert perf.nvshmem_perftest_element_bw(what, elem, dst, src, nelems, blocks, threads, None) == 0
+            rt.sync()
+            whole = rt.download_all(dst, (size + 64,), np.uint8)
+            assert np.array_equal(whole[:, size:], start[:, size:]), "wrote past the range"
+            if name == "add":
+                ty = np.uint32 if elem == 4 else np.uint64
+                want = (start[:, :size].copy().view(ty) + O.ring_put(data).copy().view(ty)).view(np.uint8)
+            else:
+                want = O.ring_get(data) if name == "g" else O.ring_put(data)
+            assert np.array_equal(whole[:, :size], want), (name, nelems)
+        rt.free(src); rt.free(dst)
+    a = rt.malloc(64)
+    assert perf.nvshmem_perftest_element_bw(3, 2, a, a, 4, 1, 64, None) != 0      # no 2-byte atomics
+    assert perf.nvshmem_perftest_element_bw(0, 8, a + 4, a, 4, 1, 64, None) != 0  # misaligned for the type
+    assert perf.nvshmem_perftest_element_bw(0, 3, a, a, 4, 1, 64, None) != 0
+    rt.free(a)
+
+
 def test_ring_rejects_ranges_outside_the_heap(rt):
     perf = rt.perftest()
     a = rt.malloc(4096)
