@@ -169,7 +169,7 @@ int nvshmem_perftest_coll_sequence(int32_t *src, int32_t *dst, uint64_t *check, 
 int nvshmem_perftest_device_team_coll(int what, int team, void *dest, const void *src, size_t n,
                                       int root, int scope, int threads, void *stream);
 /* The same call repeated `iters` times inside one kernel (the launch is paid once), for latency
- * measurements; what = 5 adds nvshmem_barrier(team). */
+ * measurements; what = 5 adds nvshmem_barrier(team), what = 6 nvshmem_team_sync(team). */
 int nvshmem_perftest_device_team_coll_loop(int what, int team, void *dest, const void *src,
                                            size_t n, int root, int iters, int scope, int threads,
                                            void *stream);

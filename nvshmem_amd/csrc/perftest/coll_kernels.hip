@@ -79,7 +79,7 @@ __global__ void barrier_kernel(uint64_t *counter, uint64_t *errors, int rounds) 
 
 // Collectives and queries on a team handle; PEs that are not members of `team` return at once.
 enum { kTeamReduce = 0, kTeamReducescatter = 1, kTeamFcollect = 2, kTeamAlltoall = 3, kTeamBroadcast = 4,
-       kTeamBarrier = 5 };
+       kTeamBarrier = 5, kTeamSync = 6 };
 
 // `iters` > 1 repeats the call inside the kernel, which is how the reference's device perftests
 // time a collective (perftest/device/coll/*_latency.cu): the launch is paid once.
@@ -97,6 +97,7 @@ __global__ void team_coll_kernel(int what, nvshmem_team_t team, void *dest, cons
         case kTeamFcollect: SCOPED_CALL(SCOPE, fcollectmem, team, dest, src, n); break;
         case kTeamAlltoall: SCOPED_CALL(SCOPE, alltoallmem, team, dest, src, n); break;
         case kTeamBarrier: SCOPED_CALL(SCOPE, barrier, team); break;
+        case kTeamSync: SCOPED_CALL(SCOPE, team_sync, team); break;
         default: SCOPED_CALL(SCOPE, broadcastmem, team, dest, src, n, root); break;
     }
 }
@@ -355,7 +356,7 @@ int nvshmem_perftest_device_barrier(uint64_t *counter, uint64_t *errors, int rou
 int nvshmem_perftest_device_team_coll_loop(int what, int team, void *dest, const void *src,
                                            size_t n, int root, int iters, int scope, int threads,
                                            void *stream) {
-    if (!perftest::ready() || scope < 0 || scope > 2 || what < kTeamReduce || what > kTeamBarrier ||
+    if (!perftest::ready() || scope < 0 || scope > 2 || what < kTeamReduce || what > kTeamSync ||
         iters < 1 || !perftest::check_launch(1, threads) || !perftest::check_range(dest, 1) ||
         !perftest::check_range(src, 1))
         return NVSHMEMX_ERROR_INVALID_VALUE;
@@ -367,7 +368,7 @@ int nvshmem_perftest_device_team_coll_loop(int what, int team, void *dest, const
 
 int nvshmem_perftest_device_team_coll(int what, int team, void *dest, const void *src, size_t n,
                                       int root, int scope, int threads, void *stream) {
-    if (what == kTeamBarrier) return NVSHMEMX_ERROR_INVALID_VALUE;
+    if (what >= kTeamBarrier) return NVSHMEMX_ERROR_INVALID_VALUE;
     return nvshmem_perftest_device_team_coll_loop(what, team, dest, src, n, root, 1, scope, threads,
                                                   stream);
 }

@@ -16,7 +16,11 @@
 //                                           reductions); size = bytes each PE contributes
 //        coll_latency                       the same five calls made inside a kernel, the call
 //                                           repeated --iters times in one launch
-//        barrier_latency                    nvshmem_barrier_all inside a kernel
+//        barrier_latency sync_latency       nvshmem_barrier_all / nvshmem_sync_all inside a kernel
+//        barrier_on_stream sync_on_stream   nvshmemx_barrier_all_on_stream / nvshmemx_sync_all_on_stream and
+//                                           their team forms (perftest/host/coll/barrier_on_stream.cpp)
+//        malloc                             nvshmem_malloc / nvshmem_free of doubling sizes
+//                                           (perftest/host/init/malloc.cpp)
 //        host_put_bw host_get_bw            nvshmemx_putmem_on_stream / getmem_on_stream from PE 0 to
 //                                           PE 1 (perftest/host/pt-to-pt/bw.cpp)
 //        pt2pt_latency                      put / get (+ put_signal ping-pong) latency per size and
@@ -27,6 +31,7 @@
 #include <cstdio>
 #include <cstdlib>
 #include <cstring>
+#include <ctime>
 #include <string>
 #include <vector>
 
@@ -47,7 +52,7 @@ struct Options {
 
 [[noreturn]] void usage(const char *why) {
     fprintf(stderr, "nvshmem_perftest: %s\nusage: nvshmem_perftest <put_bw|get_bw|p_bw|g_bw|st_bw|atomic_bw|reduce|reducescatter|fcollect|"
-                    "alltoall|broadcast|coll_latency|barrier_latency|pt2pt_latency|host_put_bw|host_get_bw> [--npes N] [--min B] [--max B] [--iters K] "
+                    "alltoall|broadcast|coll_latency|barrier_latency|sync_latency|barrier_on_stream|sync_on_stream|pt2pt_latency|host_put_bw|host_get_bw|malloc> [--npes N] [--min B] [--max B] [--iters K] "
                     "[--warmup W] [--blocks B] [--threads T] [--scope thread|warp|block] [--elem 1|2|4|8]\n", why);
     exit(2);
 }
@@ -244,7 +249,7 @@ int run_host_collective(const Options &o, int what) {
     return 0;
 }
 
-int run_device_latency(const Options &o, bool barrier_only) {
+int run_device_latency(const Options &o, bool barrier_only, bool sync = false) {
     const size_t n = (size_t)o.npes;
     const size_t cap = barrier_only ? 64 : o.max_bytes;
     void *src = nvshmem_malloc(cap * n), *dst = nvshmem_malloc(cap * n);
@@ -258,8 +263,8 @@ int run_device_latency(const Options &o, bool barrier_only) {
         return (tk - t1) * 1e3 / o.iters;
     };
     if (barrier_only) {
-        printf("#barrier_latency\n%-8s  %-16s\n%-8s  %-16.6f\n", "scope", "latency (us)", scope_name(o.scope),
-               latency_us(5, 0));
+        printf("#%s\n%-8s  %-16s\n%-8s  %-16.6f\n", sync ? "sync_latency" : "barrier_latency", "scope", "latency (us)",
+               scope_name(o.scope), latency_us(sync ? 6 : 5, 0));
     } else {
         std::vector<size_t> sizes = sweep(o, 4);
         static const struct { int what; const char *job; } calls[] = {
@@ -301,6 +306,52 @@ int run_host_rma(const Options &o, bool is_get) {
     nvshmem_free(src);
     nvshmem_free(dst);
     return 0;
+}
+
+// barrier_all_on_stream.cpp / barrier_on_stream.cpp / sync_all_on_stream.cpp / sync_on_stream.cpp:
+// microseconds per call, calls queued back to back on the default stream
+int run_host_sync(const Options &o, bool sync) {
+    const double all = time_ms([&] {
+        if (sync) nvshmemx_sync_all_on_stream(nullptr); else nvshmemx_barrier_all_on_stream(nullptr);
+        return 0;
+    }, o.iters, o.warmup);
+    const double team = time_ms([&] {
+        return sync ? nvshmemx_team_sync_on_stream(NVSHMEM_TEAM_WORLD, nullptr)
+                    : nvshmemx_barrier_on_stream(NVSHMEM_TEAM_WORLD, nullptr);
+    }, o.iters, o.warmup);
+    printf("#%s\n%-8s  %-16s\n%-8s  %-16.6f\n", sync ? "sync_all_on_stream" : "barrier_all_on_stream", "scope",
+           "latency (us)", "stream", all * 1e3);
+    printf("#%s\n%-8s  %-16s\n%-8s  %-16.6f\n", sync ? "sync_on_stream" : "barrier_on_stream", "scope",
+           "latency (us)", "stream", team * 1e3);
+    return 0;
+}
+
+// perftest/host/init/malloc.cpp: allocations of doubling size until the heap is full, then all
+// freed; microseconds of host time per call (the allocator touches no device memory)
+int run_malloc(const Options &o) {
+    std::vector<void *> held;
+    std::vector<size_t> sizes;
+    std::vector<double> alloc_us, free_us;
+    for (size_t bytes = o.min_bytes; bytes <= o.max_bytes; bytes *= 2) {
+        timespec a, b;
+        clock_gettime(CLOCK_MONOTONIC, &a);
+        void *p = nvshmem_malloc(bytes);
+        clock_gettime(CLOCK_MONOTONIC, &b);
+        if (!p) break;
+        held.push_back(p);
+        sizes.push_back(bytes);
+        alloc_us.push_back((b.tv_sec - a.tv_sec) * 1e6 + (b.tv_nsec - a.tv_nsec) * 1e-3);
+    }
+    for (void *p : held) {
+        timespec a, b;
+        clock_gettime(CLOCK_MONOTONIC, &a);
+        nvshmem_free(p);
+        clock_gettime(CLOCK_MONOTONIC, &b);
+        free_us.push_back((b.tv_sec - a.tv_sec) * 1e6 + (b.tv_nsec - a.tv_nsec) * 1e-3);
+    }
+    print_table("nvshmem_malloc", "host", "latency", "us", sizes, alloc_us);
+    print_table("nvshmem_free", "host", "latency", "us", sizes, free_us);
+    return sizes.empty() ? 1 : 0;
 }
 
 // (launch with K + 1 repetitions - launch with 1) / K, like run_device_latency; sig is cleared before
@@ -354,10 +405,11 @@ int run_pt2pt_latency(const Options &o) {
 
 int main(int argc, char **argv) {
     const Options o = parse(argc, argv);
-    const bool device_lat = o.test == "coll_latency" || o.test == "barrier_latency" || o.test == "pt2pt_latency";
+    const bool device_lat = o.test == "coll_latency" || o.test == "barrier_latency" || o.test == "sync_latency" ||
+                            o.test == "pt2pt_latency" || o.test == "barrier_on_stream" || o.test == "sync_on_stream";
     // heap: source and dest of the largest size, times npes for the collectives
     const bool rma = o.test == "put_bw" || o.test == "get_bw" || o.test == "pt2pt_latency" || o.test == "p_bw" ||
-                     o.test == "g_bw" || o.test == "st_bw" || o.test == "atomic_bw" ||
+                     o.test == "g_bw" || o.test == "st_bw" || o.test == "atomic_bw" || o.test == "malloc" ||
                      o.test == "host_put_bw" || o.test == "host_get_bw";
     Options eff = o;
     if (device_lat && o.max_bytes > ((size_t)1 << 20)) eff.max_bytes = (size_t)1 << 20;
@@ -380,6 +432,10 @@ int main(int argc, char **argv) {
     else if (o.test == "broadcast") rc = run_host_collective(eff, kBroadcast);
     else if (o.test == "coll_latency") rc = run_device_latency(eff, false);
     else if (o.test == "barrier_latency") rc = run_device_latency(eff, true);
+    else if (o.test == "sync_latency") rc = run_device_latency(eff, true, true);
+    else if (o.test == "barrier_on_stream") rc = run_host_sync(eff, false);
+    else if (o.test == "sync_on_stream") rc = run_host_sync(eff, true);
+    else if (o.test == "malloc") rc = run_malloc(eff);
     else if (o.test == "pt2pt_latency") rc = run_pt2pt_latency(eff);
     else if (o.test == "host_put_bw") rc = run_host_rma(eff, false);
     else if (o.test == "host_get_bw") rc = run_host_rma(eff, true);

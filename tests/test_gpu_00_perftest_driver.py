@@ -67,6 +67,20 @@ def test_device_latency_tables():
     assert 0.0 < _rows(out, "redmaxloc_latency")[0][2] < 1000.0
     out = _run("barrier_latency", "--iters", "100")
     assert "barrier_latency" in out
+    out = _run("sync_latency", "--iters", "100", "--scope", "thread")
+    assert 0.0 < float(out.split()[-1]) < 1000.0 and out.split()[0] == "#sync_latency"
+
+
+def test_host_synchronisation_and_allocator_tables():
+    for test, jobs in (("barrier_on_stream", ("#barrier_all_on_stream", "#barrier_on_stream")),
+                       ("sync_on_stream", ("#sync_all_on_stream", "#sync_on_stream"))):
+        lines = _run(test, "--iters", "50", "--npes", "4").splitlines()
+        assert (lines[0], lines[3]) == jobs
+        assert all(0.0 < float(lines[i].split()[-1]) < 10000.0 for i in (2, 5))
+    out = _run("malloc", "--min", "512", "--max", "64m", "--npes", "2")
+    for job in ("nvshmem_malloc", "nvshmem_free"):
+        rows = _rows(out, job)
+        assert [r[0] for r in rows] == [512 << i for i in range(18)] and all(0.0 <= v < 1e5 for _, _, v in rows)
 
 
 def test_element_wise_bandwidth_tables():
