@@ -151,14 +151,25 @@ uint16_t oracle_f32_to_f16(float f) {
 /* ------------------------------------------------------------------------------------------- */
 void oracle_copy(void *dst, const void *src, size_t bytes) { memmove(dst, src, bytes); }
 
-/* ring pattern of the reference's put example (examples/put-block.cu:39, :93-104) */
-void oracle_ring_put(uint8_t *dst, const uint8_t *src, int npes, size_t bytes) {
+/* ring pattern of the reference's put example (examples/put-block.cu:39, :93-104); the copies are
+ * cut into 1 MiB pieces so that the threads set with oracle_set_threads share them */
+#define ORC_RING_PIECE ((size_t)1 << 20)
+static void ring_copy(uint8_t *dst, const uint8_t *src, int npes, size_t bytes, int dst_step, int src_step) {
+    const long pieces = (long)((bytes + ORC_RING_PIECE - 1) / ORC_RING_PIECE);
+#pragma omp parallel for collapse(2) schedule(static)
     for (int p = 0; p < npes; ++p)
-        memcpy(dst + (size_t)((p + 1) % npes) * bytes, src + (size_t)p * bytes, bytes);
+        for (long k = 0; k < pieces; ++k) {
+            const size_t off = (size_t)k * ORC_RING_PIECE;
+            const size_t len = bytes - off < ORC_RING_PIECE ? bytes - off : ORC_RING_PIECE;
+            memcpy(dst + (size_t)((p + dst_step) % npes) * bytes + off, src + (size_t)((p + src_step) % npes) * bytes + off,
+                   len);
+        }
+}
+void oracle_ring_put(uint8_t *dst, const uint8_t *src, int npes, size_t bytes) {
+    ring_copy(dst, src, npes, bytes, 1, 0);
 }
 void oracle_ring_get(uint8_t *dst, const uint8_t *src, int npes, size_t bytes) {
-    for (int p = 0; p < npes; ++p)
-        memcpy(dst + (size_t)p * bytes, src + (size_t)((p + 1) % npes) * bytes, bytes);
+    ring_copy(dst, src, npes, bytes, 0, 1);
 }
 
 /* reference nvshmemi_signal_op, nvshmemi_common_device.cuh:507-527; SET = 9, ADD = 10

@@ -205,9 +205,11 @@ def alltoall(src_bytes):
     return out
 
 
-def ring_put(src_bytes):
+def ring_put(src_bytes, out=None):
     src = np.ascontiguousarray(src_bytes, dtype=np.uint8)
-    out = np.empty_like(src)
+    if out is None:
+        out = np.empty_like(src)
+    assert out.shape == src.shape and out.dtype == np.uint8 and out.flags.c_contiguous
     lib().oracle_ring_put(_p(out), _p(src), src.shape[0], src.shape[1])
     return out
 
