@@ -5,7 +5,7 @@
 // perftest/device/coll/*_latency.cu).
 //
 //   nvshmem_perftest <test> [--npes N] [--min BYTES] [--max BYTES] [--iters K] [--warmup W]
-//                           [--blocks B] [--threads T] [--scope thread|warp|block] [--elem 1|2|4|8]
+//                           [--blocks B] [--threads T] [--scope thread|warp|block] [--elem 1|2|4|8] [--graph]
 //
 // tests: put_bw get_bw                      device put/get, every PE to its right neighbour
 //        p_bw g_bw st_bw atomic_bw          one element per thread and call (--elem 1|2|4|8 bytes):
@@ -13,7 +13,8 @@
 //                                           nvshmem_<T>_atomic_add
 //        reduce reducescatter fcollect alltoall broadcast
 //                                           host-launched collectives on a stream (fp32 sum for the
-//                                           reductions); size = bytes each PE contributes
+//                                           reductions); size = bytes each PE contributes; --graph
+//                                           captures the timed calls in one HIP graph and replays it
 //        coll_latency                       the same five calls made inside a kernel, the call
 //                                           repeated --iters times in one launch
 //        barrier_latency sync_latency       nvshmem_barrier_all / nvshmem_sync_all inside a kernel
@@ -48,12 +49,13 @@ struct Options {
     int blocks = 0, threads = 0;  // 0: a shape that fills the GPU
     int scope = NVSHMEM_PERFTEST_SCOPE_BLOCK;
     int elem = 8;  // element size of the element-wise tests
+    bool graph = false;  // host collectives: capture the timed calls in one HIP graph
 };
 
 [[noreturn]] void usage(const char *why) {
     fprintf(stderr, "nvshmem_perftest: %s\nusage: nvshmem_perftest <put_bw|get_bw|p_bw|g_bw|st_bw|atomic_bw|reduce|reducescatter|fcollect|"
                     "alltoall|broadcast|coll_latency|barrier_latency|sync_latency|barrier_on_stream|sync_on_stream|pt2pt_latency|host_put_bw|host_get_bw|malloc> [--npes N] [--min B] [--max B] [--iters K] "
-                    "[--warmup W] [--blocks B] [--threads T] [--scope thread|warp|block] [--elem 1|2|4|8]\n", why);
+                    "[--warmup W] [--blocks B] [--threads T] [--scope thread|warp|block] [--elem 1|2|4|8] [--graph]\n", why);
     exit(2);
 }
 
@@ -88,6 +90,7 @@ Options parse(int argc, char **argv) {
         else if (a == "--blocks") o.blocks = atoi(next());
         else if (a == "--threads") o.threads = atoi(next());
         else if (a == "--elem") o.elem = atoi(next());
+        else if (a == "--graph") o.graph = true;
         else if (a == "--scope") {
             const std::string s = next();
             if (s == "thread") o.scope = NVSHMEM_PERFTEST_SCOPE_THREAD;
@@ -136,6 +139,39 @@ double time_ms(Fn fn, int iters, int warmup) {
     CHECK_HIP(hipEventDestroy(a));
     CHECK_HIP(hipEventDestroy(b));
     return (double)ms / iters;
+}
+
+// The same measurement with the `iters` calls captured once into a HIP graph on `stream` and replayed
+// (the graph variant of the reference's host collective tests, perftest/host/coll/coll_test.h:128-186):
+// average milliseconds per captured call over `replays` replays after one warm-up replay.
+template <typename Fn>
+double time_graph_ms(Fn fn, int iters, hipStream_t stream, int replays = 5) {
+    hipGraph_t graph;
+    hipGraphExec_t exec;
+    CHECK_HIP(hipStreamBeginCapture(stream, hipStreamCaptureModeGlobal));
+    for (int i = 0; i < iters; ++i)
+        if (fn() != 0) {
+            fprintf(stderr, "nvshmem_perftest: call failed under capture: %s\n", nvshmemx_amd_last_error());
+            exit(1);
+        }
+    CHECK_HIP(hipStreamEndCapture(stream, &graph));
+    CHECK_HIP(hipGraphInstantiate(&exec, graph, nullptr, nullptr, 0));
+    CHECK_HIP(hipGraphLaunch(exec, stream));
+    CHECK_HIP(hipStreamSynchronize(stream));
+    hipEvent_t a, b;
+    CHECK_HIP(hipEventCreate(&a));
+    CHECK_HIP(hipEventCreate(&b));
+    CHECK_HIP(hipEventRecord(a, stream));
+    for (int r = 0; r < replays; ++r) CHECK_HIP(hipGraphLaunch(exec, stream));
+    CHECK_HIP(hipEventRecord(b, stream));
+    CHECK_HIP(hipEventSynchronize(b));
+    float ms = 0;
+    CHECK_HIP(hipEventElapsedTime(&ms, a, b));
+    CHECK_HIP(hipEventDestroy(a));
+    CHECK_HIP(hipEventDestroy(b));
+    CHECK_HIP(hipGraphExecDestroy(exec));
+    CHECK_HIP(hipGraphDestroy(graph));
+    return (double)ms / replays / iters;
 }
 
 void print_table(const char *job, const char *scope, const char *what, const char *units,
@@ -216,34 +252,38 @@ int run_host_collective(const Options &o, int what) {
     if (!src || !dst) return 1;
     std::vector<size_t> sizes = sweep(o, 4);
     std::vector<double> us, gbs;
+    hipStream_t stream = nullptr;
+    if (o.graph) CHECK_HIP(hipStreamCreate(&stream));
     for (size_t bytes : sizes) {
         double alg = 0;
-        const double ms = time_ms([&]() -> int {
+        auto call = [&]() -> int {
             switch (what) {
                 case kReduce:
                     alg = 2.0 * n * bytes;
-                    return nvshmemx_float_sum_reduce_on_stream(NVSHMEM_TEAM_WORLD, (float *)dst, (const float *)src, bytes / 4, nullptr);
+                    return nvshmemx_float_sum_reduce_on_stream(NVSHMEM_TEAM_WORLD, (float *)dst, (const float *)src, bytes / 4, stream);
                 case kReducescatter:  // every PE holds npes blocks of `bytes`
                     alg = (double)(n + 1) * n * bytes;
-                    return nvshmemx_float_sum_reducescatter_on_stream(NVSHMEM_TEAM_WORLD, (float *)dst, (const float *)src, bytes / 4, nullptr);
+                    return nvshmemx_float_sum_reducescatter_on_stream(NVSHMEM_TEAM_WORLD, (float *)dst, (const float *)src, bytes / 4, stream);
                 case kFcollect:
                     alg = (double)(n + 1) * n * bytes;
-                    return nvshmemx_fcollectmem_on_stream(NVSHMEM_TEAM_WORLD, dst, src, bytes, nullptr);
+                    return nvshmemx_fcollectmem_on_stream(NVSHMEM_TEAM_WORLD, dst, src, bytes, stream);
                 case kAlltoall:  // `bytes` per destination
                     alg = 2.0 * n * n * bytes;
-                    return nvshmemx_alltoallmem_on_stream(NVSHMEM_TEAM_WORLD, dst, src, bytes, nullptr);
+                    return nvshmemx_alltoallmem_on_stream(NVSHMEM_TEAM_WORLD, dst, src, bytes, stream);
                 default:
                     alg = (double)(n + 1) * bytes;
-                    return nvshmemx_broadcastmem_on_stream(NVSHMEM_TEAM_WORLD, dst, src, bytes, 0, nullptr);
+                    return nvshmemx_broadcastmem_on_stream(NVSHMEM_TEAM_WORLD, dst, src, bytes, 0, stream);
             }
-        }, o.iters, o.warmup);
+        };
+        const double ms = o.graph ? time_graph_ms(call, o.iters, stream) : time_ms(call, o.iters, o.warmup);
         us.push_back(ms * 1e3);
         gbs.push_back(alg / ms / 1e6);
     }
     static const char *names[] = {"reduction_on_stream", "reducescatter_on_stream", "fcollect_on_stream",
                                   "alltoall_on_stream", "bcast_on_stream"};
-    print_table(names[what], "stream", "latency", "us", sizes, us);
-    print_table(names[what], "stream", "algorithmic BW", "GB/s", sizes, gbs);
+    print_table(names[what], o.graph ? "graph" : "stream", "latency", "us", sizes, us);
+    print_table(names[what], o.graph ? "graph" : "stream", "algorithmic BW", "GB/s", sizes, gbs);
+    if (stream) CHECK_HIP(hipStreamDestroy(stream));
     nvshmem_free(src);
     nvshmem_free(dst);
     return 0;

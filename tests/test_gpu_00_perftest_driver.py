@@ -49,6 +49,10 @@ def test_put_bw_and_collective_tables():
     assert len(lat) == 11 and all(v > 0 for _, _, v in lat)
     out = _run("broadcast", "--min", "64", "--max", "64k", "--iters", "5", "--npes", "4")
     assert len(_rows(out, "bcast_on_stream")) == 11
+    # the same calls captured in a HIP graph and replayed
+    for test, job in (("reduce", "reduction_on_stream"), ("fcollect", "fcollect_on_stream"), ("alltoall", "alltoall_on_stream")):
+        rows = _rows(_run(test, "--min", "64", "--max", "1m", "--iters", "10", "--graph"), job)
+        assert len(rows) == 15 and all(r[1] == "graph" and 0.0 < r[2] < 1e4 for r in rows), rows
 
 
 def test_host_rma_tables():
