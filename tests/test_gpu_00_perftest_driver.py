@@ -115,7 +115,9 @@ def test_point_to_point_latency_tables():
 
 
 @pytest.mark.parametrize("name,npes", [("put_block", 8), ("ring_bcast", 8), ("ring_bcast", 3), ("allreduce", 8),
-                                       ("allreduce", 5), ("on_stream", 8), ("on_stream", 16), ("moe_shuffle", 8), ("moe_shuffle", 3)])
+                                       ("allreduce", 5), ("on_stream", 8), ("on_stream", 16), ("moe_shuffle", 8), ("moe_shuffle", 3),
+                                       ("collective_launch", 8), ("collective_launch", 5), ("thread_group", 8),
+                                       ("thread_group", 3), ("simple_shift", 8), ("simple_shift", 2)])
 def test_example_programs_reach_their_known_answers(name, npes):
     """nvshmem_amd/examples/*.hip are user programs built with one hipcc command against include/ and
     libnvshmem_amd.so; each checks the closed-form answer of the reference example it models on every
