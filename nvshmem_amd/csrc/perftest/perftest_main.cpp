@@ -197,10 +197,11 @@ int run_rma(const Options &o, bool is_get) {
     std::vector<size_t> sizes = sweep(o, 1);
     std::vector<double> gbs;
     for (size_t bytes : sizes) {
-        // default: 1 KiB per block of one wavefront (one 16-byte vector per lane), the shape that
-        // measures fastest on large messages (bounded below by 1 block)
+        // default: a block of one wavefront and one 16-byte vector per lane (1 KiB per block), the
+        // shape that measures fastest on large messages (bounded below by 1 block)
         int threads = o.threads ? o.threads : 64;
-        long blocks = o.blocks ? o.blocks : (long)((bytes + 1023) / 1024);
+        const size_t per_block = (size_t)threads * 16;
+        long blocks = o.blocks ? o.blocks : (long)((bytes + per_block - 1) / per_block);
         if (blocks < 1) blocks = 1;
         if (blocks > (1 << 22)) blocks = 1 << 22;
         const double ms = time_ms([&] {

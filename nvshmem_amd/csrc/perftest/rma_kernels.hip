@@ -50,8 +50,11 @@ __global__ void ring_rma_kernel(char *dest, const char *src, size_t bytes, size_
         else nvshmemx_putmem_block(dest + off, src + off, len, peer);
     } else if (SCOPE == NVSHMEM_PERFTEST_SCOPE_WARP) {
         const size_t waves = (blockDim.x + NVSHMEMI_WARP_SIZE - 1) / NVSHMEMI_WARP_SIZE;
-        size_t woff, wlen;
-        if (!slice_of(len, waves, threadIdx.x / NVSHMEMI_WARP_SIZE, &woff, &wlen)) return;
+        // the wavefront's index as a scalar: the slice bounds and the copy's branches on them then
+        // stay in scalar registers, as they do in the block scope
+        const unsigned wave = __builtin_amdgcn_readfirstlane(threadIdx.x / NVSHMEMI_WARP_SIZE);
+        size_t woff = 0, wlen = len;
+        if (waves > 1 && !slice_of(len, waves, wave, &woff, &wlen)) return;
         if (GET) nvshmemx_getmem_warp(dest + off + woff, src + off + woff, wlen, peer);
         else nvshmemx_putmem_warp(dest + off + woff, src + off + woff, wlen, peer);
     } else {

@@ -125,7 +125,9 @@ def test_ring_put_get_block_sizes_8B_to_4MiB(rt, blocks, is_get):
         assert np.array_equal(got, want), "size 2^%d" % p
 
 
-@pytest.mark.parametrize("scope,threads", [(N.SCOPE_THREAD, 64), (N.SCOPE_WARP, 256), (N.SCOPE_BLOCK, 1024)])
+# 96 and 160 threads: the block's last wavefront has 32 lanes only
+@pytest.mark.parametrize("scope,threads", [(N.SCOPE_THREAD, 64), (N.SCOPE_WARP, 256), (N.SCOPE_BLOCK, 1024),
+                                           (N.SCOPE_WARP, 96), (N.SCOPE_WARP, 160), (N.SCOPE_BLOCK, 96)])
 def test_ring_put_get_scopes_ragged_sizes(rt, scope, threads):
     for size in (0, 1, 7, 100, 1000, 4097, 65536 + 13, (1 << 20) + 5):
         for is_get in (0, 1):
