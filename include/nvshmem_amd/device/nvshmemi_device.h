@@ -900,6 +900,47 @@ NVSHMEMI_DEVICE_INLINE uint64_t nvshmemi_amd_ll_recv_packet(const char *packet, 
     }
     return (uint64_t)v.x | ((uint64_t)v.z << 32);
 }
+/* The same for NVSHMEMI_AMD_LL_BATCH packets at once: all loads are issued before the first is looked
+ * at, so a lane that owns several packets pays one memory round trip per poll and not one per packet.
+ * Packets whose bit in `pending` is clear are loaded too (the caller passes any valid packet address
+ * for them) and ignored.  Returns the bits still missing when a bounded wait gave up, else 0. */
+#define NVSHMEMI_AMD_LL_BATCH 4
+NVSHMEMI_DEVICE_INLINE unsigned nvshmemi_amd_ll_recv_batch(const char *const (&packet)[NVSHMEMI_AMD_LL_BATCH],
+                                                           uint64_t (&payload)[NVSHMEMI_AMD_LL_BATCH],
+                                                           unsigned pending, uint32_t flag) {
+    const uint64_t limit = nvshmemi_device_state_d.spin_limit;
+    uint64_t polls = 0;
+    while (pending) {
+        nvshmemi_v4u v[NVSHMEMI_AMD_LL_BATCH];
+        asm volatile(
+            "global_load_dwordx4 %0, %4, off sc1\n\t"
+            "global_load_dwordx4 %1, %5, off sc1\n\t"
+            "global_load_dwordx4 %2, %6, off sc1\n\t"
+            "global_load_dwordx4 %3, %7, off sc1\n\t"
+            "s_waitcnt vmcnt(0)"
+            : "=&v"(v[0]), "=&v"(v[1]), "=&v"(v[2]), "=&v"(v[3])
+            : "v"(packet[0]), "v"(packet[1]), "v"(packet[2]), "v"(packet[3])
+            : "memory");
+#pragma unroll
+        for (int k = 0; k < NVSHMEMI_AMD_LL_BATCH; ++k)
+            if (((pending >> k) & 1u) && v[k].y == flag && v[k].w == flag) {
+                payload[k] = (uint64_t)v[k].x | ((uint64_t)v[k].z << 32);
+                pending &= ~(1u << k);
+            }
+        if (!pending) break;
+        if (limit && ++polls > limit) {
+#pragma unroll
+            for (int k = 0; k < NVSHMEMI_AMD_LL_BATCH; ++k)
+                if ((pending >> k) & 1u) {
+                    nvshmemi_amd_record_timeout(packet[k], v[k].y, flag);
+                    break;
+                }
+            break;
+        }
+        __builtin_amdgcn_s_sleep(1);
+    }
+    return pending;
+}
 /* Sends npk chunks to each other member of the team, chunk j into slot slot0 + j of its buffers:
  * the chunks of src for everybody (dest_stride 0), or those of src + idx * dest_stride for member
  * idx.  The (member, chunk) pairs are spread over the lanes. */
@@ -934,6 +975,62 @@ NVSHMEMI_DEVICE_INLINE bool nvshmemi_amd_ll_fits(size_t nbytes, int size) {
     return nbytes > 0 && nbytes <= NVSHMEMI_AMD_LL_MAX_BYTES && nvshmemi_amd_ll_available() &&
            npk * 8 * (size_t)size <= NVSHMEMI_AMD_LL_PAYLOAD_BYTES &&
            npk * (size_t)(size - 1) <= nvshmemi_amd_ll_lanes<SCOPE>();
+}
+/* fcollect / alltoall: a wavefront or block lets every lane own up to NVSHMEMI_AMD_LL_BATCH packets,
+ * which it polls together (measured among 8 PEs with 256 threads: 3.9 against 5.0 us at 512 bytes per
+ * member and 4.7 against 4.9 at 1 KiB; more packets per lane lose against the copy-and-barrier path) */
+template <int SCOPE>
+NVSHMEMI_DEVICE_INLINE bool nvshmemi_amd_ll_fits_batched(size_t nbytes, int size) {
+    const size_t npk = (nbytes + 7) >> 3;
+    const size_t per_lane = SCOPE == NVSHMEMI_THREADGROUP_THREAD ? 1 : NVSHMEMI_AMD_LL_BATCH;
+    return nbytes > 0 && nbytes <= NVSHMEMI_AMD_LL_MAX_BYTES && nvshmemi_amd_ll_available() &&
+           npk * 8 * (size_t)size <= NVSHMEMI_AMD_LL_PAYLOAD_BYTES &&
+           npk * (size_t)(size - 1) <= per_lane * nvshmemi_amd_ll_lanes<SCOPE>();
+}
+/* Reception for fcollect and alltoall: the packets of the other members, chunk j of member idx in slot
+ * idx * npk + j of `mine`, go to dst + idx * nbytes + 8 j; the (member, chunk) pairs are spread over the
+ * lanes, NVSHMEMI_AMD_LL_BATCH of them per lane and round. */
+template <int SCOPE>
+NVSHMEMI_DEVICE_INLINE void nvshmemi_amd_ll_unpack(const char *mine, char *dst, size_t nbytes, unsigned npk, int me,
+                                                   int npes, uint32_t flag) {
+    const unsigned tid = (unsigned)nvshmemi_thread_id_in_threadgroup<SCOPE>();
+    const unsigned nthr = (unsigned)nvshmemi_threadgroup_size<SCOPE>();
+    const unsigned total = (unsigned)(npes - 1) * npk;
+    if (total <= nthr) { /* at most one packet per lane */
+        if (tid < total) {
+            const unsigned off = tid / npk, j = tid - off * npk;
+            int idx = me + 1 + (int)off;
+            if (idx >= npes) idx -= npes;
+            const uint64_t v = nvshmemi_amd_ll_recv_packet(mine + ((size_t)idx * npk + j) * 16, flag);
+            nvshmemi_amd_ll_store_payload(dst + (size_t)idx * nbytes + 8 * (size_t)j, v, nbytes - 8 * (size_t)j);
+        }
+        return;
+    }
+    for (unsigned w0 = tid; w0 < total; w0 += NVSHMEMI_AMD_LL_BATCH * nthr) {
+        const char *packet[NVSHMEMI_AMD_LL_BATCH];
+        char *out[NVSHMEMI_AMD_LL_BATCH];
+        size_t left[NVSHMEMI_AMD_LL_BATCH];
+        uint64_t payload[NVSHMEMI_AMD_LL_BATCH];
+        unsigned pending = 0;
+#pragma unroll
+        for (int k = 0; k < NVSHMEMI_AMD_LL_BATCH; ++k) {
+            const unsigned w = w0 + (unsigned)k * nthr;
+            const unsigned wc = w < total ? w : w0; /* out of range: this lane's first packet once more */
+            const unsigned off = wc / npk, j = wc - off * npk;
+            int idx = me + 1 + (int)off;
+            if (idx >= npes) idx -= npes;
+            packet[k] = mine + ((size_t)idx * npk + j) * 16;
+            out[k] = dst + (size_t)idx * nbytes + 8 * (size_t)j;
+            left[k] = nbytes - 8 * (size_t)j;
+            payload[k] = 0;
+            if (w < total) pending |= 1u << k;
+        }
+        const unsigned wanted = pending;
+        const unsigned missing = nvshmemi_amd_ll_recv_batch(packet, payload, pending, flag);
+#pragma unroll
+        for (int k = 0; k < NVSHMEMI_AMD_LL_BATCH; ++k)
+            if (((wanted & ~missing) >> k) & 1u) nvshmemi_amd_ll_store_payload(out[k], payload[k], left[k]);
+    }
 }
 
 /* Small allreduce in one hop: every member sends its source to every other member as packets and
@@ -1100,26 +1197,19 @@ NVSHMEMI_DEVICE_INLINE int nvshmemi_fcollect_threadgroup(nvshmem_team_t team, T 
     const int me = tv.my_pe;
     const int npes = tv.size;
     const size_t nbytes = nelems * sizeof(T);
-    if (nvshmemi_amd_ll_fits<SCOPE>(nbytes, npes)) {
+    if (nvshmemi_amd_ll_fits_batched<SCOPE>(nbytes, npes)) {
         /* small contributions: packets to every member's buffer, then unpack what arrived here;
          * the (member, chunk) pairs are spread over the lanes both ways */
         const unsigned tid = (unsigned)nvshmemi_thread_id_in_threadgroup<SCOPE>();
         const unsigned nthr = (unsigned)nvshmemi_threadgroup_size<SCOPE>();
         const uint32_t flag = nvshmemi_amd_ll_next_flag<SCOPE>(team);
         const unsigned npk = nvshmemi_amd_ll_packets(nbytes);
-        const unsigned total = (unsigned)(npes - 1) * npk;
         const char *src = nvshmemi_amd_local(source);
         char *dst = nvshmemi_amd_local(dest);
         nvshmemi_amd_ll_send_to_all<SCOPE>(team, tv, src, nbytes, npk, (unsigned)me * npk, flag);
         for (size_t b = tid; b < nbytes; b += nthr) dst[(size_t)me * nbytes + b] = src[b];
-        const char *mine = nvshmemi_amd_ll_buffer(team, nvshmemi_amd_my_pe(), flag);
-        for (unsigned w = tid; w < total; w += nthr) {
-            const unsigned off = w / npk, j = w - off * npk;
-            int idx = me + 1 + (int)off;
-            if (idx >= npes) idx -= npes;
-            const uint64_t v = nvshmemi_amd_ll_recv_packet(mine + ((size_t)idx * npk + j) * 16, flag);
-            nvshmemi_amd_ll_store_payload(dst + (size_t)idx * nbytes + 8 * (size_t)j, v, nbytes - 8 * (size_t)j);
-        }
+        nvshmemi_amd_ll_unpack<SCOPE>(nvshmemi_amd_ll_buffer(team, nvshmemi_amd_my_pe(), flag), dst, nbytes, npk, me,
+                                      npes, flag);
         nvshmemi_amd_ll_publish_done<SCOPE>(team, flag);
         return 0;
     }
@@ -1141,25 +1231,18 @@ NVSHMEMI_DEVICE_INLINE int nvshmemi_alltoall_threadgroup(nvshmem_team_t team, T 
     const int me = tv.my_pe;
     const int npes = tv.size;
     const size_t nbytes = nelems * sizeof(T);
-    if (nvshmemi_amd_ll_fits<SCOPE>(nbytes, npes)) {
+    if (nvshmemi_amd_ll_fits_batched<SCOPE>(nbytes, npes)) {
         /* small blocks: like the fcollect packets, but member idx is sent block idx */
         const unsigned tid = (unsigned)nvshmemi_thread_id_in_threadgroup<SCOPE>();
         const unsigned nthr = (unsigned)nvshmemi_threadgroup_size<SCOPE>();
         const uint32_t flag = nvshmemi_amd_ll_next_flag<SCOPE>(team);
         const unsigned npk = nvshmemi_amd_ll_packets(nbytes);
-        const unsigned total = (unsigned)(npes - 1) * npk;
         const char *src = nvshmemi_amd_local(source);
         char *dst = nvshmemi_amd_local(dest);
         nvshmemi_amd_ll_send_to_all<SCOPE>(team, tv, src, nbytes, npk, (unsigned)me * npk, flag, nbytes);
         for (size_t b = tid; b < nbytes; b += nthr) dst[(size_t)me * nbytes + b] = src[(size_t)me * nbytes + b];
-        const char *mine = nvshmemi_amd_ll_buffer(team, nvshmemi_amd_my_pe(), flag);
-        for (unsigned w = tid; w < total; w += nthr) {
-            const unsigned off = w / npk, j = w - off * npk;
-            int idx = me + 1 + (int)off;
-            if (idx >= npes) idx -= npes;
-            const uint64_t v = nvshmemi_amd_ll_recv_packet(mine + ((size_t)idx * npk + j) * 16, flag);
-            nvshmemi_amd_ll_store_payload(dst + (size_t)idx * nbytes + 8 * (size_t)j, v, nbytes - 8 * (size_t)j);
-        }
+        nvshmemi_amd_ll_unpack<SCOPE>(nvshmemi_amd_ll_buffer(team, nvshmemi_amd_my_pe(), flag), dst, nbytes, npk, me,
+                                      npes, flag);
         nvshmemi_amd_ll_publish_done<SCOPE>(team, flag);
         return 0;
     }

@@ -56,13 +56,15 @@ def _expected_checks(npes, n, fc_bytes, rounds):
 
 def _uses_packets(what, nbytes, npes, scope, threads):
     """The library's rule for taking the packet path: one packet per lane of the thread group (a
-    single thread takes up to 8), nvshmemi_amd_ll_fits / nvshmemi_amd_ll_reduce_group."""
+    single thread takes up to 8; fcollect and alltoall in the wavefront and block scope up to four per
+    lane), nvshmemi_amd_ll_fits / nvshmemi_amd_ll_fits_batched / nvshmemi_amd_ll_reduce_group."""
     nthr = {N.SCOPE_BLOCK: threads, N.SCOPE_WARP: 64, N.SCOPE_THREAD: 1}[scope]
     lanes = max(nthr, 8)
     npk = (nbytes + 7) // 8
     if what == "broadcast":
         return nbytes <= 16384 and npk * (npes - 1 if scope == N.SCOPE_THREAD else 1) <= lanes
-    ok = nbytes <= 2048 and npk * 8 * npes <= 16384 and npk * (npes - 1) <= lanes
+    per_lane = 4 if what in ("fcollect", "alltoall") and scope != N.SCOPE_THREAD else 1
+    ok = nbytes <= 2048 and npk * 8 * npes <= 16384 and npk * (npes - 1) <= per_lane * lanes
     if what in ("reduce", "reducescatter") and scope != N.SCOPE_THREAD:
         group = 1
         while group < npes:
@@ -152,7 +154,9 @@ def test_sizes_around_the_switch_over(rt8, scope, threads):
                 rt8.sync()
                 assert bits_equal(rt8.download_all(dst, (n,), data.dtype, off), O.reducescatter(kind, op, data)), \
                     (kind, op, n, off)
-    for nbytes in (1, 7, 8, 9, 63, 72, 73, 288, 289, 511, 512, 513, 2047, 2048, 2049, 16384, 16385):
+    # 72 | 73 and 288 | 289: one packet per lane of a wavefront / a 256-thread block; 289 (wavefront) and
+    # 1168 | 1169 (block): four per lane
+    for nbytes in (1, 7, 8, 9, 63, 72, 73, 288, 289, 511, 512, 513, 1167, 1168, 1169, 2047, 2048, 2049, 16384, 16385):
         for soff, doff in ((0, 0), (3, 5)):
             data = rng.integers(0, 256, (8, nbytes), dtype=np.uint8)
             rt8.fill(dst, 0xCD, 1 << 18)
