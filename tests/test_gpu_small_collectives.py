@@ -56,15 +56,17 @@ def _expected_checks(npes, n, fc_bytes, rounds):
 
 def _uses_packets(what, nbytes, npes, scope, threads):
     """The library's rule for taking the packet path: one packet per lane of the thread group (a
-    single thread takes up to 8; fcollect and alltoall in the wavefront and block scope up to four per
-    lane), nvshmemi_amd_ll_fits / nvshmemi_amd_ll_fits_batched / nvshmemi_amd_ll_reduce_group."""
+    single thread takes up to 8), nvshmemi_amd_ll_fits / nvshmemi_amd_ll_reduce_group."""
     nthr = {N.SCOPE_BLOCK: threads, N.SCOPE_WARP: 64, N.SCOPE_THREAD: 1}[scope]
     lanes = max(nthr, 8)
     npk = (nbytes + 7) // 8
     if what == "broadcast":
-        return nbytes <= 16384 and npk * (npes - 1 if scope == N.SCOPE_THREAD else 1) <= lanes
-    per_lane = 4 if what in ("fcollect", "alltoall") and scope != N.SCOPE_THREAD else 1
-    ok = nbytes <= 2048 and npk * 8 * npes <= 16384 and npk * (npes - 1) <= per_lane * lanes
+        # (a wavefront or block whose (member, chunk) pairs need more than one round over its lanes pushes
+        # with the fan-out copy instead when source and dest share their offset within 16 bytes, as the
+        # buffers of these tests do)
+        return nbytes <= 16384 and npk * (npes - 1 if scope == N.SCOPE_THREAD else 1) <= lanes and \
+            (npk * (npes - 1) <= lanes or scope == N.SCOPE_THREAD)
+    ok = nbytes <= 2048 and npk * 8 * npes <= 16384 and npk * (npes - 1) <= lanes
     if what in ("reduce", "reducescatter") and scope != N.SCOPE_THREAD:
         group = 1
         while group < npes:
@@ -154,8 +156,8 @@ def test_sizes_around_the_switch_over(rt8, scope, threads):
                 rt8.sync()
                 assert bits_equal(rt8.download_all(dst, (n,), data.dtype, off), O.reducescatter(kind, op, data)), \
                     (kind, op, n, off)
-    # 72 | 73 and 288 | 289: one packet per lane of a wavefront / a 256-thread block; 289 (wavefront) and
-    # 1168 | 1169 (block): four per lane
+    # 72 | 73 and 288 | 289: one packet per lane of a wavefront / a 256-thread block; beyond, and up to
+    # 16384 bytes, the fan-out copy (whole vectors from 16 bytes on, edge bytes around them)
     for nbytes in (1, 7, 8, 9, 63, 72, 73, 288, 289, 511, 512, 513, 1167, 1168, 1169, 2047, 2048, 2049, 16384, 16385):
         for soff, doff in ((0, 0), (3, 5)):
             data = rng.integers(0, 256, (8, nbytes), dtype=np.uint8)
