@@ -214,6 +214,12 @@ typedef struct {
 #define NVSHMEMI_AMD_LL_PAYLOAD_BYTES 16384
 #define NVSHMEMI_AMD_LL_MAX_BYTES 2048
 #define NVSHMEMI_AMD_LL_BCAST_MAX_BYTES 16384 /* broadcast: one contribution, up to a whole buffer */
+/* Behind the packet buffers of all teams every (team, PE) owns NVSHMEMI_AMD_STAGE_BUFFERS staging
+ * buffers of NVSHMEMI_AMD_STAGE_BYTES: the members of a small in-kernel reduction push their whole
+ * contributions there (member i into slot i) and every PE folds its own copy after ONE barrier; the
+ * parity of the team's barrier count picks the buffer. */
+#define NVSHMEMI_AMD_STAGE_BUFFERS 2
+#define NVSHMEMI_AMD_STAGE_BYTES 32768
 #define NVSHMEMI_AMD_LL_COUNT_WORD (NVSHMEMI_AMD_MAX_PES + 1)
 #define NVSHMEMI_AMD_LL_DONE_WORD (NVSHMEMI_AMD_MAX_PES + 2)
 /* Words of a PE's team sync row where the wavefronts of nvshmemx_barrier_warpgroup meet: the
@@ -235,7 +241,8 @@ typedef struct nvshmemi_device_state {
     const nvshmemi_amd_team_view_t *team_views; /* [NVSHMEMI_AMD_MAX_TEAMS][NVSHMEMI_AMD_MAX_PES] */
     uint64_t *team_sync; /* [MAX_TEAMS][MAX_PES][NVSHMEMI_AMD_TEAM_SYNC_WORDS]: barrier rows of the teams
                             other than WORLD, low-latency counters of all teams */
-    char *ll_buffers;    /* [MAX_TEAMS][npes][NVSHMEMI_AMD_LL_BUFFERS][2 * NVSHMEMI_AMD_LL_PAYLOAD_BYTES] */
+    char *ll_buffers;    /* [MAX_TEAMS][npes][NVSHMEMI_AMD_LL_BUFFERS][2 * NVSHMEMI_AMD_LL_PAYLOAD_BYTES], then
+                            [MAX_TEAMS][npes][NVSHMEMI_AMD_STAGE_BUFFERS][NVSHMEMI_AMD_STAGE_BYTES] */
 } nvshmemi_device_state_t;
 
 #endif

@@ -27,6 +27,11 @@ size_t ll_bytes_per_team(const Runtime &rt) {
     return (size_t)rt.npes * NVSHMEMI_AMD_LL_BUFFERS * 2 * NVSHMEMI_AMD_LL_PAYLOAD_BYTES;
 }
 
+// the staging buffers of all teams follow the packet buffers of all teams in one allocation
+size_t stage_bytes_per_team(const Runtime &rt) {
+    return (size_t)rt.npes * NVSHMEMI_AMD_STAGE_BUFFERS * NVSHMEMI_AMD_STAGE_BYTES;
+}
+
 // distinct member sets of the handle, in order of their first PE
 void rebuild_groups(Runtime &rt, int team) {
     TeamTable &tt = rt.teams;
@@ -137,7 +142,7 @@ bool teams_init(Runtime &rt) {
     // every in-kernel collective takes its copy-and-barrier path
     const char *no_ll = getenv("NVSHMEM_AMD_DISABLE_LL");
     if (!(no_ll && no_ll[0] == '1')) {
-        const size_t ll_bytes = ll_bytes_per_team(rt) * kMaxTeams;
+        const size_t ll_bytes = (ll_bytes_per_team(rt) + stage_bytes_per_team(rt)) * kMaxTeams;
         e = hipMalloc(&mem, ll_bytes);
         if (e != hipSuccess || !mem) {
             (void)hipGetLastError();
