@@ -97,12 +97,12 @@ WORKLOADS = {
 }
 
 COMMANDS = """Commands (from the repository root on the GPU box; every file they run is committed):
-  cd /tmp && export TMPDIR=/tmp
-  rocprofv3 --kernel-trace --stats -d $REPO/gpurun_out/prof_stats -- python3 $REPO/nvshmem_amd/profile_workloads.py
-  rocprofv3 --pmc FETCH_SIZE -d $REPO/gpurun_out/prof_fetch -- python3 $REPO/nvshmem_amd/profile_workloads.py --iters 5
-  rocprofv3 --pmc WRITE_SIZE -d $REPO/gpurun_out/prof_write -- python3 $REPO/nvshmem_amd/profile_workloads.py --iters 5
-  python3 nvshmem_amd/profile_summary.py --stats gpurun_out/prof_stats --fetch gpurun_out/prof_fetch \\
-          --write gpurun_out/prof_write --profiles-dir profiles
+  cd /tmp && export TMPDIR=/tmp OUT=<a scratch directory>
+  rocprofv3 --kernel-trace --stats -d $OUT/prof_stats -- python3 $REPO/nvshmem_amd/profile_workloads.py
+  rocprofv3 --pmc FETCH_SIZE -d $OUT/prof_fetch -- python3 $REPO/nvshmem_amd/profile_workloads.py --iters 5
+  rocprofv3 --pmc WRITE_SIZE -d $OUT/prof_write -- python3 $REPO/nvshmem_amd/profile_workloads.py --iters 5
+  python3 nvshmem_amd/profile_summary.py --stats $OUT/prof_stats --fetch $OUT/prof_fetch \\
+          --write $OUT/prof_write --profiles-dir profiles
 Hardware: one MI355X (gfx950), ROCm 7.2.  Durations are per dispatch from the kernel trace."""
 
 
