@@ -347,7 +347,7 @@ NVSHMEMI_DEVICE_INLINE void nvshmemi_quiet() {
     nvshmemi_amd_wait_vm();
     nvshmemi_threadgroup_sync<SCOPE>();
     if (nvshmemi_thread_id_in_threadgroup<SCOPE>() == 0)
-        __builtin_amdgcn_fence(__ATOMIC_SEQ_CST, "agent");
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "agent");
     nvshmemi_threadgroup_sync<SCOPE>();
 }
 
