@@ -159,14 +159,16 @@ def test_sizes_around_the_switch_over(rt8, scope, threads):
     # 72 | 73 and 288 | 289: one packet per lane of a wavefront / a 256-thread block; beyond, and up to
     # 16384 bytes, the fan-out copy (whole vectors from 16 bytes on, edge bytes around them)
     for nbytes in (1, 7, 8, 9, 63, 72, 73, 288, 289, 511, 512, 513, 1167, 1168, 1169, 2047, 2048, 2049, 16384, 16385):
-        for soff, doff in ((0, 0), (3, 5)):
+        # (3, 5): no common offset within 16 bytes, a copy per member; (5, 21): a common one, the fan-out
+        # copy with bytes in front of its first whole vector
+        for soff, doff in ((0, 0), (3, 5), (5, 21)):
             data = rng.integers(0, 256, (8, nbytes), dtype=np.uint8)
             rt8.fill(dst, 0xCD, 1 << 18)
             rt8.upload_all(src, data, soff)
             note("device fcollect / broadcast bytes=%d soff=%d doff=%d scope=%d" % (nbytes, soff, doff, scope))
             assert perf.nvshmem_perftest_device_fcollect(dst + doff, src + soff, nbytes, scope, threads, None) == 0
             rt8.sync()
-            got = rt8.download_all(dst, (8 * nbytes + 16,), np.uint8)
+            got = rt8.download_all(dst, (8 * nbytes + 32,), np.uint8)
             assert np.array_equal(got[:, doff:doff + 8 * nbytes], O.fcollect(data))
             assert (got[:, :doff] == 0xCD).all() and (got[:, doff + 8 * nbytes:] == 0xCD).all()
             if 8 * nbytes + soff <= (1 << 16):
@@ -175,14 +177,14 @@ def test_sizes_around_the_switch_over(rt8, scope, threads):
                 rt8.upload_all(src, data8, soff)
                 assert perf.nvshmem_perftest_device_alltoall(dst + doff, src + soff, nbytes, scope, threads, None) == 0
                 rt8.sync()
-                got = rt8.download_all(dst, (8 * nbytes + 16,), np.uint8)
+                got = rt8.download_all(dst, (8 * nbytes + 32,), np.uint8)
                 assert np.array_equal(got[:, doff:doff + 8 * nbytes], O.alltoall(data8))
                 assert (got[:, :doff] == 0xCD).all() and (got[:, doff + 8 * nbytes:] == 0xCD).all()
                 rt8.upload_all(src, data, soff)
             rt8.fill(dst, 0xCD, 1 << 18)
             assert perf.nvshmem_perftest_device_broadcast(dst + doff, src + soff, nbytes, 6, scope, threads, None) == 0
             rt8.sync()
-            got = rt8.download_all(dst, (nbytes + 16,), np.uint8)
+            got = rt8.download_all(dst, (nbytes + 32,), np.uint8)
             assert np.array_equal(got[:, doff:doff + nbytes], O.broadcast(data, 6))
             assert (got[:, :doff] == 0xCD).all() and (got[:, doff + nbytes:] == 0xCD).all()
     rt8.free(src); rt8.free(dst)
