@@ -188,8 +188,11 @@ NVSHMEMI_REPT_FOR_SIZES(NVSHMEMI_STAMP_SIZED_RMA)
 #undef NVSHMEMI_STAMP_SIZED_RMA_SCOPE
 
 /* ---- signals ---- */
+/* As in the reference (nvshmemi_signal_op, common/nvshmemi_common_device.cuh:507-527: a bare store or
+ * atomic add), a standalone signal orders nothing by itself: a caller that publishes data with it
+ * calls nvshmem_fence or nvshmem_quiet first, or uses a put-with-signal. */
 NVSHMEMI_DEV void nvshmemx_signal_op(uint64_t *sig_addr, uint64_t signal, int sig_op, int pe) {
-    nvshmemi_signal_op_release(sig_addr, signal, sig_op, pe);
+    nvshmemi_signal_op(sig_addr, signal, sig_op, pe);
 }
 NVSHMEMI_DEV uint64_t nvshmem_signal_fetch(uint64_t *sig_addr) {
     return nvshmemi_amd_poll(reinterpret_cast<const uint64_t *>(nvshmemi_amd_local(sig_addr)));

@@ -363,7 +363,7 @@ NVSHMEMI_DEVICE_INLINE void nvshmemi_signal_op(uint64_t *sig_addr, uint64_t sign
         __hip_atomic_fetch_add(p, signal, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 }
 
-/* A standalone signal publishes everything its caller wrote before it. */
+/* The signal of a put-with-signal publishes the data that the group wrote before it. */
 NVSHMEMI_DEVICE_INLINE void nvshmemi_signal_op_release(uint64_t *sig_addr, uint64_t signal,
                                                        int sig_op, int pe) {
     __builtin_amdgcn_fence(__ATOMIC_RELEASE, "agent");
