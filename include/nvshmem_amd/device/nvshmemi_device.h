@@ -946,6 +946,38 @@ template <int SCOPE>
 NVSHMEMI_DEVICE_INLINE void nvshmemi_amd_ll_send_to_all(nvshmem_team_t team, const nvshmemi_amd_team_view_t &tv,
                                                         const char *src, size_t nbytes, unsigned npk,
                                                         unsigned slot0, uint32_t flag, size_t dest_stride = 0) {
+    if (SCOPE == NVSHMEMI_THREADGROUP_THREAD) {
+        /* a single thread: chunk by chunk, the chunk loaded once (dest_stride 0) or for eight members in
+         * one go, then the stores to the members one behind the other with no load in between (member
+         * by member every store waited for the load in front of it: 8 bytes among 8 PEs, fcollect 7.0 us
+         * against 5.2 us, allreduce 5.9 against 3.6) */
+        for (unsigned j = 0; j < npk; ++j) {
+            const uint64_t same =
+                dest_stride ? 0 : nvshmemi_amd_ll_load_payload(src + 8 * (size_t)j, nbytes - 8 * (size_t)j);
+            for (int o0 = 0; o0 < tv.size - 1; o0 += 8) {
+                uint64_t x[8];
+#pragma unroll
+                for (int k = 0; k < 8; ++k) {
+                    const int off = o0 + k < tv.size - 1 ? o0 + k : o0;
+                    int idx = tv.my_pe + 1 + off;
+                    if (idx >= tv.size) idx -= tv.size;
+                    x[k] = dest_stride ? nvshmemi_amd_ll_load_payload(src + (size_t)idx * dest_stride + 8 * (size_t)j,
+                                                                      nbytes - 8 * (size_t)j)
+                                       : same;
+                }
+#pragma unroll
+                for (int k = 0; k < 8; ++k) {
+                    if (o0 + k >= tv.size - 1) break;
+                    int idx = tv.my_pe + 1 + o0 + k;
+                    if (idx >= tv.size) idx -= tv.size;
+                    nvshmemi_amd_ll_store_packet(
+                        nvshmemi_amd_ll_buffer(team, nvshmemi_amd_team_pe(tv, idx), flag) + (size_t)(slot0 + j) * 16, x[k],
+                        flag);
+                }
+            }
+        }
+        return;
+    }
     const unsigned nthr = (unsigned)nvshmemi_threadgroup_size<SCOPE>();
     const unsigned total = (unsigned)(tv.size - 1) * npk;
     for (unsigned w = (unsigned)nvshmemi_thread_id_in_threadgroup<SCOPE>(); w < total; w += nthr) {
