@@ -1371,7 +1371,15 @@ NVSHMEMI_DEVICE_INLINE int nvshmemi_fcollect_threadgroup(nvshmem_team_t team, T 
         const char *src = nvshmemi_amd_local(source);
         char *dst = nvshmemi_amd_local(dest);
         nvshmemi_amd_ll_send_to_all<SCOPE>(team, tv, src, nbytes, npk, (unsigned)me * npk, flag);
-        for (size_t b = tid; b < nbytes; b += nthr) dst[(size_t)me * nbytes + b] = src[b];
+        /* the caller's own block: a single thread moves it eight bytes at a time (byte by byte every
+         * store waited for a load), the lanes of a group a byte each */
+        if (SCOPE == NVSHMEMI_THREADGROUP_THREAD)
+            for (unsigned j = 0; j < npk; ++j)
+                nvshmemi_amd_ll_store_payload(dst + (size_t)me * nbytes + 8 * (size_t)j,
+                                              nvshmemi_amd_ll_load_payload(src + 8 * (size_t)j, nbytes - 8 * (size_t)j),
+                                              nbytes - 8 * (size_t)j);
+        else
+            for (size_t b = tid; b < nbytes; b += nthr) dst[(size_t)me * nbytes + b] = src[b];
         const char *mine = nvshmemi_amd_ll_buffer(team, nvshmemi_amd_my_pe(), flag);
         for (unsigned w = tid; w < total; w += nthr) {
             const unsigned off = w / npk, j = w - off * npk;
@@ -1412,7 +1420,14 @@ NVSHMEMI_DEVICE_INLINE int nvshmemi_alltoall_threadgroup(nvshmem_team_t team, T 
         const char *src = nvshmemi_amd_local(source);
         char *dst = nvshmemi_amd_local(dest);
         nvshmemi_amd_ll_send_to_all<SCOPE>(team, tv, src, nbytes, npk, (unsigned)me * npk, flag, nbytes);
-        for (size_t b = tid; b < nbytes; b += nthr) dst[(size_t)me * nbytes + b] = src[(size_t)me * nbytes + b];
+        if (SCOPE == NVSHMEMI_THREADGROUP_THREAD)
+            for (unsigned j = 0; j < npk; ++j)
+                nvshmemi_amd_ll_store_payload(
+                    dst + (size_t)me * nbytes + 8 * (size_t)j,
+                    nvshmemi_amd_ll_load_payload(src + (size_t)me * nbytes + 8 * (size_t)j, nbytes - 8 * (size_t)j),
+                    nbytes - 8 * (size_t)j);
+        else
+            for (size_t b = tid; b < nbytes; b += nthr) dst[(size_t)me * nbytes + b] = src[(size_t)me * nbytes + b];
         const char *mine = nvshmemi_amd_ll_buffer(team, nvshmemi_amd_my_pe(), flag);
         for (unsigned w = tid; w < total; w += nthr) {
             const unsigned off = w / npk, j = w - off * npk;
@@ -1467,11 +1482,39 @@ NVSHMEMI_DEVICE_INLINE int nvshmemi_broadcast_threadgroup(nvshmem_team_t team, T
             char *dst = nvshmemi_amd_local(dest);
             /* nothing else orders a root against its receivers: all of them must have finished
              * reading call flag - 2 before anybody may be sent call flag */
-            for (unsigned i = tid; i < (unsigned)npes; i += nthr)
-                if ((int)i != me && flag > 2)
+            if (flag > 2 && nthr >= (unsigned)npes) {
+                if (tid < (unsigned)npes && (int)tid != me)
                     nvshmemi_wait_until<uint64_t>(
-                        nvshmemi_amd_ll_word(team, nvshmemi_amd_team_pe(tv, (int)i), NVSHMEMI_AMD_LL_DONE_WORD),
+                        nvshmemi_amd_ll_word(team, nvshmemi_amd_team_pe(tv, (int)tid), NVSHMEMI_AMD_LL_DONE_WORD),
                         NVSHMEM_CMP_GE, (uint64_t)(flag - 2));
+            } else if (flag > 2) {
+                /* a lane that answers for several members reads eight of their words per round trip (the
+                 * root's own word is past flag - 2 as well, so nobody is left out) */
+                const uint64_t limit = nvshmemi_device_state_d.spin_limit;
+                uint64_t polls = 0;
+                for (;;) {
+                    uint64_t lowest = ~(uint64_t)0;
+                    for (unsigned i0 = tid; i0 < (unsigned)npes; i0 += 8 * nthr) {
+                        uint64_t x[8];
+#pragma unroll
+                        for (unsigned k = 0; k < 8; ++k) {
+                            const unsigned i = i0 + k * nthr < (unsigned)npes ? i0 + k * nthr : i0;
+                            x[k] = nvshmemi_amd_poll(reinterpret_cast<const uint64_t *>(
+                                nvshmemi_amd_ll_word(team, nvshmemi_amd_team_pe(tv, (int)i), NVSHMEMI_AMD_LL_DONE_WORD)));
+                        }
+#pragma unroll
+                        for (unsigned k = 0; k < 8; ++k) lowest = x[k] < lowest ? x[k] : lowest;
+                    }
+                    if (lowest >= (uint64_t)(flag - 2)) break;
+                    if (limit && ++polls > limit) {
+                        nvshmemi_amd_record_timeout(
+                            nvshmemi_amd_ll_word(team, nvshmemi_amd_team_pe(tv, (int)tid), NVSHMEMI_AMD_LL_DONE_WORD), lowest,
+                            (uint64_t)(flag - 2));
+                        break;
+                    }
+                    __builtin_amdgcn_s_sleep(1);
+                }
+            }
             nvshmemi_threadgroup_sync<SCOPE>();
             nvshmemi_amd_ll_send_to_all<SCOPE>(team, tv, src, nbytes, npk, 0, flag);
             if (dst != src)
