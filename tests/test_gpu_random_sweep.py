@@ -185,3 +185,39 @@ def test_random_in_kernel_collectives(npes, seed):
             if team != N.TEAM_WORLD:
                 rt.team_destroy(team)
         rt.free(src); rt.free(dst)
+
+
+@pytest.mark.parametrize("scope,threads", [(N.SCOPE_WARP, 64), (N.SCOPE_BLOCK, 256), (N.SCOPE_BLOCK, 1024)])
+def test_large_in_kernel_pushes(scope, threads):
+    """In-kernel fcollect / alltoall / broadcast from 32 KiB to 256 KiB per member: a common source is
+    fanned out at any size, different sources up to 32 KiB each, beyond that a copy per member; with
+    and without a common offset of source and dest within 16 bytes."""
+    npes = 8
+    rng = np.random.default_rng(300 + threads)
+    top = (256 << 10) + 48
+    with runtime(npes, 10 * npes * top + (16 << 20)) as rt:
+        perf = rt.perftest()
+        src = rt.malloc(npes * top + 64); dst = rt.malloc(npes * top + 64)
+        for nbytes in (32768, 32784, 100003, top):
+            for soff, doff in ((0, 0), (5, 21), (3, 5)):
+                data = rng.integers(0, 256, (npes, npes * nbytes), dtype=np.uint8)
+                rt.upload_all(src, data, soff)
+                for what in (2, 3, 4):
+                    rt.fill(dst, 0xCD, npes * top + 64)
+                    note("large push what=%d bytes=%d soff=%d doff=%d scope=%d threads=%d" % (what, nbytes, soff, doff, scope, threads))
+                    assert perf.nvshmem_perftest_device_team_coll(what, N.TEAM_WORLD, dst + doff, src + soff, nbytes, 5,
+                                                                  scope, threads, None) == 0
+                    rt.sync()
+                    out_bytes = nbytes if what == 4 else npes * nbytes
+                    got = rt.download_all(dst, (npes * top + 64,), np.uint8)
+                    if what == 2:
+                        want = O.fcollect(data[:, :nbytes])
+                    elif what == 3:
+                        want = O.alltoall(data)
+                    else:
+                        want = np.broadcast_to(data[5, :nbytes], (npes, nbytes))
+                    assert np.array_equal(got[:, doff:doff + out_bytes], want), (what, nbytes, soff, doff)
+                    assert (got[:, :doff] == 0xCD).all() and (got[:, doff + out_bytes:] == 0xCD).all()
+        flag, rec = rt.read_timeout(0)
+        assert flag == 0, rec
+        rt.free(src); rt.free(dst)
