@@ -1110,6 +1110,9 @@ NVSHMEMI_DEVICE_INLINE unsigned nvshmemi_amd_ll_reduce_group(size_t nbytes, int 
  * at every size: 64 KiB per member among 8 PEs with 256 threads 8.6 against 12.9 us, 1 MiB 98 against
  * 131 us). */
 #define NVSHMEMI_AMD_FANOUT_MAX_BYTES 32768
+/* in-kernel broadcasts from this size on are fetched by every PE instead of pushed by the root */
+#define NVSHMEMI_AMD_BCAST_PULL_BYTES 32768
+#define NVSHMEMI_AMD_BCAST_PULL_BYTES_PER_LANE 128
 /* (every PE's slice starts on a multiple of 16 bytes and more, so a symmetric address and its
  * translations share their low bits and every PE decides alike) */
 template <int SCOPE>
@@ -1529,6 +1532,20 @@ NVSHMEMI_DEVICE_INLINE int nvshmemi_broadcast_threadgroup(nvshmem_team_t team, T
                                               nbytes - 8 * (size_t)j);
         }
         nvshmemi_amd_ll_publish_done<SCOPE>(team, flag);
+        return 0;
+    }
+    if (nbytes >= NVSHMEMI_AMD_BCAST_PULL_BYTES ||
+        nbytes >= (size_t)NVSHMEMI_AMD_BCAST_PULL_BYTES_PER_LANE * (size_t)nvshmemi_threadgroup_size<SCOPE>()) {
+        /* long messages: a root that pushes does all the work alone (1 MiB to 8 PEs from one block:
+         * 98 us).  Instead everybody meets - the root's source is complete and written back by then -
+         * and every PE fetches the message itself, all blocks at once (17 us), and meets again, after
+         * which the root may reuse its source.  Two barriers instead of one pay off from 32 KiB on for a
+         * block and from 128 bytes per lane for smaller groups (a wavefront: 8 KiB, 4.5 against 5.3 us). */
+        nvshmemi_barrier_threadgroup<SCOPE>(team);
+        const char *from = nvshmemi_amd_remote(source, nvshmemi_amd_team_pe(tv, PE_root));
+        char *to = nvshmemi_amd_local(dest);
+        if (to != from) nvshmemi_memcpy_threadgroup<SCOPE>(to, from, nbytes);
+        nvshmemi_barrier_threadgroup<SCOPE>(team);
         return 0;
     }
     if (me == PE_root) {

@@ -187,11 +187,13 @@ def test_random_in_kernel_collectives(npes, seed):
         rt.free(src); rt.free(dst)
 
 
-@pytest.mark.parametrize("scope,threads", [(N.SCOPE_WARP, 64), (N.SCOPE_BLOCK, 256), (N.SCOPE_BLOCK, 1024)])
+@pytest.mark.parametrize("scope,threads", [(N.SCOPE_WARP, 64), (N.SCOPE_BLOCK, 256), (N.SCOPE_BLOCK, 1024),
+                                           (N.SCOPE_THREAD, 64)])
 def test_large_in_kernel_pushes(scope, threads):
     """In-kernel fcollect / alltoall / broadcast from 32 KiB to 256 KiB per member: a common source is
     fanned out at any size, different sources up to 32 KiB each, beyond that a copy per member; with
-    and without a common offset of source and dest within 16 bytes."""
+    and without a common offset of source and dest within 16 bytes.  Broadcasts of this length are
+    fetched by every PE between two barriers instead of pushed by the root."""
     npes = 8
     rng = np.random.default_rng(300 + threads)
     top = (256 << 10) + 48
