@@ -496,29 +496,57 @@ NVSHMEMI_DEVICE_INLINE void nvshmemi_wait_until_all(T *ivars, size_t nelems, con
     }
     __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "agent");
 }
+/* One pass over the set, eight variables per memory round trip: visit(i, satisfied) is called for the
+ * members in index order until it returns false.  The caller acquires once if it reports success. */
+template <typename T, bool VECTOR, typename Visit>
+NVSHMEMI_DEVICE_INLINE void nvshmemi_amd_scan_set(T *ivars, size_t nelems, const int *status, int cmp,
+                                                  const T *values, Visit visit) {
+    if (nelems == 0) return;
+    const T *addr = reinterpret_cast<const T *>(nvshmemi_amd_local(ivars));
+    for (size_t first = 0; first < nelems; first += 8) {
+        T x[8];
+#pragma unroll
+        for (size_t k = 0; k < 8; ++k) x[k] = nvshmemi_amd_poll(addr + (first + k < nelems ? first + k : nelems - 1));
+#pragma unroll
+        for (size_t k = 0; k < 8; ++k) {
+            const size_t i = first + k;
+            if (i >= nelems) return;
+            if (status && status[i]) continue;
+            if (!visit(i, nvshmemi_amd_compare(x[k], cmp, nvshmemi_amd_cmp_value<T, VECTOR>(values, i)))) return;
+        }
+    }
+}
 template <typename T, bool VECTOR>
 NVSHMEMI_DEVICE_INLINE int nvshmemi_test_all(T *ivars, size_t nelems, const int *status, int cmp,
                                              const T *values) {
-    for (size_t i = 0; i < nelems; ++i)
-        if ((!status || !status[i]) && !nvshmemi_test<T>(ivars + i, cmp, nvshmemi_amd_cmp_value<T, VECTOR>(values, i)))
-            return 0;
-    return 1;
+    bool all = true;
+    nvshmemi_amd_scan_set<T, VECTOR>(ivars, nelems, status, cmp, values, [&](size_t, bool ok) {
+        all = ok;
+        return ok;
+    });
+    if (all) __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "agent");
+    return all ? 1 : 0;
 }
 template <typename T, bool VECTOR>
 NVSHMEMI_DEVICE_INLINE size_t nvshmemi_test_any(T *ivars, size_t nelems, const int *status, int cmp,
                                                 const T *values) {
-    for (size_t i = 0; i < nelems; ++i)
-        if ((!status || !status[i]) && nvshmemi_test<T>(ivars + i, cmp, nvshmemi_amd_cmp_value<T, VECTOR>(values, i)))
-            return i;
-    return SIZE_MAX;
+    size_t hit = SIZE_MAX;
+    nvshmemi_amd_scan_set<T, VECTOR>(ivars, nelems, status, cmp, values, [&](size_t i, bool ok) {
+        if (ok) hit = i;
+        return !ok;
+    });
+    if (hit != SIZE_MAX) __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "agent");
+    return hit;
 }
 template <typename T, bool VECTOR>
 NVSHMEMI_DEVICE_INLINE size_t nvshmemi_test_some(T *ivars, size_t nelems, size_t *indices, const int *status,
                                                  int cmp, const T *values) {
     size_t found = 0;
-    for (size_t i = 0; i < nelems; ++i)
-        if ((!status || !status[i]) && nvshmemi_test<T>(ivars + i, cmp, nvshmemi_amd_cmp_value<T, VECTOR>(values, i)))
-            indices[found++] = i;
+    nvshmemi_amd_scan_set<T, VECTOR>(ivars, nelems, status, cmp, values, [&](size_t i, bool ok) {
+        if (ok) indices[found++] = i;
+        return true;
+    });
+    if (found) __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "agent");
     return found;
 }
 template <typename T, bool VECTOR>
