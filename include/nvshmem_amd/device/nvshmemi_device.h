@@ -144,25 +144,49 @@ NVSHMEMI_DEVICE_INLINE void *nvshmemi_ptr(const void *ptr, int pe) {
  *
  * Byte-exact copy by the lanes of one thread group.  Where the reference picks the widest element
  * both pointers are aligned to and cascades, this version always stores 16-byte vectors: a byte
- * head brings dst to a 16-byte boundary, the body issues four independent dwordx4 loads per lane
- * before the first store (gfx950 accepts unaligned vector loads, so a src that is not co-aligned
- * only costs extra cache-line touches, not narrower instructions), and a byte tail finishes.
+ * head brings dst to a 16-byte boundary, the body issues four (long copies: sixteen) independent
+ * dwordx4 loads per lane before the first store (gfx950 accepts unaligned vector loads, so a src that
+ * is not co-aligned only costs extra cache-line touches, not narrower instructions), and a byte tail
+ * finishes.
  * ---------------------------------------------------------------------------------------------- */
 typedef unsigned int nvshmemi_v4u __attribute__((ext_vector_type(4)));
 typedef nvshmemi_v4u __attribute__((aligned(1))) nvshmemi_v4u_unaligned;
 
+/* Vectors per lane and round of the ordinary body. */
 #ifndef NVSHMEMI_AMD_COPY_UNROLL
 #define NVSHMEMI_AMD_COPY_UNROLL 4
 #endif
-/* bit 0: non-temporal loads, bit 1: non-temporal stores in the vector body.  Stores stream (the
- * copy never reads its destination back).  Loads stay cacheable by default because callers often
- * push the same source to several PEs (top-k token dispatch, all-push collectives) and the repeats
- * then hit in L2: measured 1.4x on the MoE dispatch.  A translation unit whose kernels only stream
- * bulk data once may define NVSHMEMI_AMD_COPY_NT 3 before including nvshmem.h: measured +5 % on a
- * 256 MiB put. */
-#ifndef NVSHMEMI_AMD_COPY_NT
-#define NVSHMEMI_AMD_COPY_NT 2
+/* Long copies - a lane owns at least NVSHMEMI_AMD_COPY_DEEP_MIN vectors - run rounds of
+ * NVSHMEMI_AMD_COPY_DEEP_UNROLL vectors per lane first (0 switches the deep rounds off).  A thread group
+ * that streams a long slice on its own compute unit is bound by the bytes it keeps in flight: 1024
+ * threads x 4 vectors are 64 KiB, which at the loaded memory latency is about 33 GB/s. */
+#ifndef NVSHMEMI_AMD_COPY_DEEP_UNROLL
+#define NVSHMEMI_AMD_COPY_DEEP_UNROLL 16
 #endif
+#ifndef NVSHMEMI_AMD_COPY_DEEP_MIN
+#define NVSHMEMI_AMD_COPY_DEEP_MIN 32
+#endif
+/* Cache policy of the vector body.  Stores stream (non-temporal): a copy never reads its destination
+ * back.  Loads stay cacheable for short and medium copies, because callers often push the same source
+ * to several PEs (top-k token dispatch, all-push collectives) and the repeats then hit in L2 (measured
+ * 1.4x on the MoE dispatch); a single copy of NVSHMEMI_AMD_COPY_NT_BYTES or more streams its loads
+ * too (measured +5 % on a 256 MiB put).  NVSHMEMI_AMD_COPY_NT overrides the choice for a translation
+ * unit: bit 0 set = always non-temporal loads, 0 = never; bit 1 = non-temporal stores. */
+#ifndef NVSHMEMI_AMD_COPY_NT_BYTES
+#define NVSHMEMI_AMD_COPY_NT_BYTES (1u << 20)
+#endif
+
+/* A 16-byte store at agent scope (written through the L2).  The compiler has no such store, so it is
+ * written as inline assembly, and the compiler does not know that the statement is a vector memory
+ * store: it would not keep the one wait state this GPU needs between a store of more than 8 bytes
+ * and a write to the registers that hold the store's data, so the s_nop supplies it (without it a
+ * following address computation that reused the data registers corrupted the stored value). */
+NVSHMEMI_DEVICE_INLINE void nvshmemi_amd_store16_agent(char *p, nvshmemi_v4u v) {
+#ifndef NVSHMEMI_AMD_AGENT_STORE_MODS
+#define NVSHMEMI_AMD_AGENT_STORE_MODS "sc1"
+#endif
+    asm volatile("global_store_dwordx4 %0, %1, off " NVSHMEMI_AMD_AGENT_STORE_MODS "\n\ts_nop 1" : : "v"(p), "v"(v) : "memory");
+}
 
 template <bool SRC_ALIGNED>
 NVSHMEMI_DEVICE_INLINE nvshmemi_v4u nvshmemi_amd_load16(const char *p) {
@@ -170,56 +194,130 @@ NVSHMEMI_DEVICE_INLINE nvshmemi_v4u nvshmemi_amd_load16(const char *p) {
     return *reinterpret_cast<const nvshmemi_v4u_unaligned *>(p);
 }
 
-template <bool SRC_ALIGNED>
+template <bool SRC_ALIGNED, bool NT_LOAD>
 NVSHMEMI_DEVICE_INLINE nvshmemi_v4u nvshmemi_amd_stream_load16(const char *p) {
-    if ((NVSHMEMI_AMD_COPY_NT & 1) && SRC_ALIGNED)
-        return __builtin_nontemporal_load(reinterpret_cast<const nvshmemi_v4u *>(p));
+    if (NT_LOAD && SRC_ALIGNED) return __builtin_nontemporal_load(reinterpret_cast<const nvshmemi_v4u *>(p));
     return nvshmemi_amd_load16<SRC_ALIGNED>(p);
 }
+/* Where the stores of a copy go: streamed (non-temporal; the lines stay dirty in this XCD's L2 until
+ * they are evicted or a release writes the L2 back) or written through the L2 to memory at agent scope,
+ * which leaves nothing for a later release to write back. */
+enum nvshmemi_amd_store_policy_t { NVSHMEMI_AMD_STORE_STREAM = 0, NVSHMEMI_AMD_STORE_WRITE_THROUGH = 1 };
+
+template <int STORE = NVSHMEMI_AMD_STORE_STREAM>
 NVSHMEMI_DEVICE_INLINE void nvshmemi_amd_stream_store16(char *p, nvshmemi_v4u v) {
-    if (NVSHMEMI_AMD_COPY_NT & 2) __builtin_nontemporal_store(v, reinterpret_cast<nvshmemi_v4u *>(p));
-    else *reinterpret_cast<nvshmemi_v4u *>(p) = v;
+    if (STORE == NVSHMEMI_AMD_STORE_WRITE_THROUGH) {
+        nvshmemi_amd_store16_agent(p, v);
+        return;
+    }
+#if defined(NVSHMEMI_AMD_COPY_NT) && !(NVSHMEMI_AMD_COPY_NT & 2)
+    *reinterpret_cast<nvshmemi_v4u *>(p) = v;
+#else
+    __builtin_nontemporal_store(v, reinterpret_cast<nvshmemi_v4u *>(p));
+#endif
+}
+template <int STORE>
+NVSHMEMI_DEVICE_INLINE void nvshmemi_amd_store_byte(char *p, char v) {
+    if (STORE == NVSHMEMI_AMD_STORE_WRITE_THROUGH)
+        __hip_atomic_store(reinterpret_cast<unsigned char *>(p), (unsigned char)v, __ATOMIC_RELAXED,
+                           __HIP_MEMORY_SCOPE_AGENT);
+    else
+        *p = v;
 }
 
 /* Lane `tid` of `nthr` owns vectors tid, tid+nthr, ...  Rounds of U vectors per lane are straight-line
  * code - U independent loads issued before the first store - and run while the lane still has U
- * vectors left; the remainder is handled by the same code at U/2, U/4, ... 1, so a short copy (a
- * 14 KiB row moved by one wavefront is 14 vectors per lane: 4 + 4 + 4 + 2) keeps most of its loads in
- * flight.  No per-vector predicates: branches between the loads would make them wait for each
+ * vectors left; with CASCADE the remainder is handled by the same code at U/2, U/4, ... 1, so a short
+ * copy (a 14 KiB row moved by one wavefront is 14 vectors per lane: 4 + 4 + 4 + 2) keeps most of its
+ * loads in flight.  No per-vector predicates: branches between the loads would make them wait for each
  * other. */
-template <bool SRC_ALIGNED, int U>
+template <bool SRC_ALIGNED, bool NT_LOAD, int STORE, int U, bool CASCADE>
 NVSHMEMI_DEVICE_INLINE size_t nvshmemi_amd_copy_rounds(char *__restrict__ dst,
                                                       const char *__restrict__ src, size_t nvec,
                                                       size_t i, size_t nthr) {
     for (; i + (U - 1) * nthr < nvec; i += U * nthr) {
         nvshmemi_v4u v[U];
 #pragma unroll
-        for (int u = 0; u < U; ++u) v[u] = nvshmemi_amd_stream_load16<SRC_ALIGNED>(src + 16 * (i + u * nthr));
+        for (int u = 0; u < U; ++u)
+            v[u] = nvshmemi_amd_stream_load16<SRC_ALIGNED, NT_LOAD>(src + 16 * (i + u * nthr));
 #pragma unroll
-        for (int u = 0; u < U; ++u) nvshmemi_amd_stream_store16(dst + 16 * (i + u * nthr), v[u]);
+        for (int u = 0; u < U; ++u) nvshmemi_amd_stream_store16<STORE>(dst + 16 * (i + u * nthr), v[u]);
     }
-    if constexpr (U > 1) return nvshmemi_amd_copy_rounds<SRC_ALIGNED, U / 2>(dst, src, nvec, i, nthr);
+    if constexpr (CASCADE && U > 1)
+        return nvshmemi_amd_copy_rounds<SRC_ALIGNED, NT_LOAD, STORE, U / 2, true>(dst, src, nvec, i, nthr);
     return i;
 }
 
-template <bool SRC_ALIGNED>
-NVSHMEMI_DEVICE_INLINE void nvshmemi_amd_copy_vectors(char *__restrict__ dst,
-                                                     const char *__restrict__ src, size_t nvec,
-                                                     size_t tid, size_t nthr) {
-    nvshmemi_amd_copy_rounds<SRC_ALIGNED, NVSHMEMI_AMD_COPY_UNROLL>(dst, src, nvec, tid, nthr);
+/* The translation unit's fixed choice for the loads of the ordinary rounds; the deep rounds of a long
+ * copy choose at run time. */
+#if defined(NVSHMEMI_AMD_COPY_NT) && (NVSHMEMI_AMD_COPY_NT & 1)
+#define NVSHMEMI_AMD_COPY_NT_ALWAYS true
+#else
+#define NVSHMEMI_AMD_COPY_NT_ALWAYS false
+#endif
+
+/* Deep rounds of a long copy by whole wavefronts: per round the group moves U * nthr consecutive
+ * vectors, of which wavefront w owns the U KiB [w * U, (w + 1) * U) and moves them with U loads issued
+ * back to back, then U stores.  The wavefront's base addresses are wave-uniform (scalar registers) and a
+ * lane adds its 16 * lane and a constant u * 1024, so the U vectors in flight cost 4 U vector registers
+ * and no address registers of their own (one address pair per vector made the compiler serialise the
+ * round to stay within its register budget).  Returns the number of vectors moved, a multiple of
+ * U * nthr. */
+template <bool NT_LOAD, int STORE, int U>
+NVSHMEMI_DEVICE_INLINE size_t nvshmemi_amd_copy_deep_rounds(char *__restrict__ dst, const char *__restrict__ src,
+                                                           size_t nvec, unsigned tid, size_t nthr) {
+    const size_t per_round = (size_t)U * nthr;
+    const size_t rounds = nvec / per_round;
+    const size_t wave = (size_t)__builtin_amdgcn_readfirstlane(tid >> 6);
+    const unsigned lane_off = (tid & 63u) * 16u;
+    const char *s = src + wave * (size_t)(U * 1024);
+    char *d = dst + wave * (size_t)(U * 1024);
+    for (size_t r = 0; r < rounds; ++r, s += 16 * per_round, d += 16 * per_round) {
+        nvshmemi_v4u v[U];
+#pragma unroll
+        for (int u = 0; u < U; ++u) v[u] = nvshmemi_amd_stream_load16<true, NT_LOAD>(s + u * 1024 + lane_off);
+#pragma unroll
+        for (int u = 0; u < U; ++u) nvshmemi_amd_stream_store16<STORE>(d + u * 1024 + lane_off, v[u]);
+    }
+    return rounds * per_round;
 }
 
-template <int SCOPE>
+template <bool SRC_ALIGNED, int STORE>
+NVSHMEMI_DEVICE_INLINE void nvshmemi_amd_copy_vectors(char *__restrict__ dst,
+                                                     const char *__restrict__ src, size_t nvec,
+                                                     size_t tid, size_t nthr, bool stream_loads) {
+#if NVSHMEMI_AMD_COPY_DEEP_UNROLL > NVSHMEMI_AMD_COPY_UNROLL
+    if (SRC_ALIGNED && (nthr & 63) == 0 && nvec >= (size_t)NVSHMEMI_AMD_COPY_DEEP_MIN * nthr) {
+        const size_t done =
+            stream_loads ? nvshmemi_amd_copy_deep_rounds<true, STORE, NVSHMEMI_AMD_COPY_DEEP_UNROLL>(
+                               dst, src, nvec, (unsigned)tid, nthr)
+                         : nvshmemi_amd_copy_deep_rounds<false, STORE, NVSHMEMI_AMD_COPY_DEEP_UNROLL>(
+                               dst, src, nvec, (unsigned)tid, nthr);
+        dst += 16 * done;
+        src += 16 * done;
+        nvec -= done;
+    }
+#endif
+    nvshmemi_amd_copy_rounds<SRC_ALIGNED, NVSHMEMI_AMD_COPY_NT_ALWAYS, STORE, NVSHMEMI_AMD_COPY_UNROLL, true>(
+        dst, src, nvec, tid, nthr);
+}
+
+template <int SCOPE, int STORE = NVSHMEMI_AMD_STORE_STREAM>
 NVSHMEMI_DEVICE_INLINE void nvshmemi_memcpy_threadgroup(void *__restrict__ dst_v,
                                                        const void *__restrict__ src_v, size_t len) {
     char *dst = static_cast<char *>(dst_v);
     const char *src = static_cast<const char *>(src_v);
     const size_t tid = (size_t)nvshmemi_thread_id_in_threadgroup<SCOPE>();
     const size_t nthr = (size_t)nvshmemi_threadgroup_size<SCOPE>();
+#if defined(NVSHMEMI_AMD_COPY_NT)
+    const bool stream_loads = (NVSHMEMI_AMD_COPY_NT & 1) != 0;
+#else
+    const bool stream_loads = len >= NVSHMEMI_AMD_COPY_NT_BYTES;
+#endif
 
     size_t head = (size_t)(-(uintptr_t)dst & 15);
     if (head > len) head = len;
-    for (size_t i = tid; i < head; i += nthr) dst[i] = src[i];
+    for (size_t i = tid; i < head; i += nthr) nvshmemi_amd_store_byte<STORE>(dst + i, src[i]);
     dst += head;
     src += head;
     len -= head;
@@ -232,16 +330,16 @@ NVSHMEMI_DEVICE_INLINE void nvshmemi_memcpy_threadgroup(void *__restrict__ dst_v
         size_t pre = 0;
         if (nvec >= 256) {
             pre = (size_t)((-(uintptr_t)dst >> 4) & 63);
-            if (((uintptr_t)src & 15) == 0) nvshmemi_amd_copy_vectors<true>(dst, src, pre, tid, nthr);
-            else nvshmemi_amd_copy_vectors<false>(dst, src, pre, tid, nthr);
+            if (((uintptr_t)src & 15) == 0) nvshmemi_amd_copy_vectors<true, STORE>(dst, src, pre, tid, nthr, false);
+            else nvshmemi_amd_copy_vectors<false, STORE>(dst, src, pre, tid, nthr, false);
         }
         if (((uintptr_t)src & 15) == 0)
-            nvshmemi_amd_copy_vectors<true>(dst + 16 * pre, src + 16 * pre, nvec - pre, tid, nthr);
+            nvshmemi_amd_copy_vectors<true, STORE>(dst + 16 * pre, src + 16 * pre, nvec - pre, tid, nthr, stream_loads);
         else
-            nvshmemi_amd_copy_vectors<false>(dst + 16 * pre, src + 16 * pre, nvec - pre, tid, nthr);
+            nvshmemi_amd_copy_vectors<false, STORE>(dst + 16 * pre, src + 16 * pre, nvec - pre, tid, nthr, stream_loads);
     }
     const size_t done = nvec * 16;
-    for (size_t i = done + tid; i < len; i += nthr) dst[i] = src[i];
+    for (size_t i = done + tid; i < len; i += nthr) nvshmemi_amd_store_byte<STORE>(dst + i, src[i]);
 }
 
 /* ------------------------------------------------------------------------------------------------
@@ -357,7 +455,7 @@ NVSHMEMI_DEVICE_INLINE void nvshmemi_quiet() {
 NVSHMEMI_DEVICE_INLINE void nvshmemi_signal_op(uint64_t *sig_addr, uint64_t signal, int sig_op,
                                                int pe) {
     uint64_t *p = reinterpret_cast<uint64_t *>(nvshmemi_amd_remote(sig_addr, pe));
-    if (sig_op == NVSHMEM_SIGNAL_SET)
+    if ((sig_op & NVSHMEMI_AMD_SIGNAL_OP_MASK) == NVSHMEM_SIGNAL_SET)
         __hip_atomic_store(p, signal, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     else
         __hip_atomic_fetch_add(p, signal, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
@@ -370,19 +468,40 @@ NVSHMEMI_DEVICE_INLINE void nvshmemi_signal_op_release(uint64_t *sig_addr, uint6
     nvshmemi_signal_op(sig_addr, signal, sig_op, pe);
 }
 
+/* put-with-signal.  Two orderings, chosen by the caller through sig_op:
+ *  - default, the reference's (a full fence in front of the signal,
+ *    common/nvshmemi_common_device.cuh:541-545): the payload streams into the L2, every wavefront waits
+ *    for its stores, and the one lane that signals first releases at agent scope, which writes the
+ *    XCD's L2 back - the payload and whatever else the group wrote before the call (a ring allreduce
+ *    that accumulates into its destination with plain stores and is overwritten by a neighbour later
+ *    relies on that);
+ *  - NVSHMEMX_AMD_SIGNAL_PAYLOAD_ONLY, OpenSHMEM's: the payload is written through the L2 with
+ *    agent-scope stores, so it is in memory once every wavefront has counted its stores down, and the
+ *    signal follows with no fence at all.  An L2 write-back walks the whole L2, the write-backs of an
+ *    XCD run one after the other, dirty lines leave at about 60 GB/s per XCD and other traffic crawls
+ *    meanwhile: a token dispatch that signals each 14 KiB row took 17-24 ms with a release per row
+ *    (whether the payload was streamed or written through, and also when the wavefronts of an XCD
+ *    shared write-backs through a ticket lock: a write-back under that load takes some 20 us), against
+ *    1.7 ms with one release per block.  Without the fence the per-row form takes a few ms. */
 template <typename T, int SCOPE>
 NVSHMEMI_DEVICE_INLINE void nvshmemi_put_signal(T *dest, const T *source, size_t nelems,
                                                 uint64_t *sig_addr, uint64_t signal, int sig_op,
                                                 int pe) {
     nvshmemi_threadgroup_sync<SCOPE>();
-    nvshmemi_memcpy_threadgroup<SCOPE>(nvshmemi_amd_remote(dest, pe), nvshmemi_amd_local(source),
-                                       nelems * sizeof(T));
-    /* Every wavefront's stores have reached the L2 before the group meets; the one lane that
-     * signals then releases at agent scope, which writes the L2 back for the other XCDs. */
-    nvshmemi_amd_wait_vm();
-    nvshmemi_threadgroup_sync<SCOPE>();
-    if (nvshmemi_thread_id_in_threadgroup<SCOPE>() == 0)
-        nvshmemi_signal_op_release(sig_addr, signal, sig_op, pe);
+    if (sig_op & NVSHMEMX_AMD_SIGNAL_PAYLOAD_ONLY) {
+        nvshmemi_memcpy_threadgroup<SCOPE, NVSHMEMI_AMD_STORE_WRITE_THROUGH>(
+            nvshmemi_amd_remote(dest, pe), nvshmemi_amd_local(source), nelems * sizeof(T));
+        nvshmemi_amd_wait_vm();
+        nvshmemi_threadgroup_sync<SCOPE>();
+        if (nvshmemi_thread_id_in_threadgroup<SCOPE>() == 0) nvshmemi_signal_op(sig_addr, signal, sig_op, pe);
+    } else {
+        nvshmemi_memcpy_threadgroup<SCOPE>(nvshmemi_amd_remote(dest, pe), nvshmemi_amd_local(source),
+                                           nelems * sizeof(T));
+        nvshmemi_amd_wait_vm();
+        nvshmemi_threadgroup_sync<SCOPE>();
+        if (nvshmemi_thread_id_in_threadgroup<SCOPE>() == 0)
+            nvshmemi_signal_op_release(sig_addr, signal, sig_op, pe);
+    }
     nvshmemi_threadgroup_sync<SCOPE>();
 }
 
@@ -975,7 +1094,7 @@ NVSHMEMI_DEVICE_INLINE void nvshmemi_amd_ll_store_packet(char *packet, uint64_t 
     v.y = flag;
     v.z = (uint32_t)(w >> 32);
     v.w = flag;
-    asm volatile("global_store_dwordx4 %0, %1, off sc1" : : "v"(packet), "v"(v) : "memory");
+    nvshmemi_amd_store16_agent(packet, v);
 }
 /* Waits until both halves of the packet carry `flag` and returns its 8 payload bytes.  A bounded
  * wait that gives up records the timeout like nvshmemi_wait_until and returns what it last saw. */

@@ -54,6 +54,13 @@ typedef enum {
 /* Signal operators: the values are those of the reference's AMO enumeration. */
 #define NVSHMEM_SIGNAL_SET 9
 #define NVSHMEM_SIGNAL_ADD 10
+/* May be OR-ed into the sig_op of a device-side put-with-signal: the signal is ordered behind the
+ * payload of THIS put only, which is what OpenSHMEM promises for the operation.  Without it the
+ * signal is also ordered behind everything else the calling thread group wrote before the call, as
+ * in the reference (a full fence in front of its signal), which on this GPU costs a write-back of
+ * the XCD's L2 per call.  No counterpart in the reference. */
+#define NVSHMEMX_AMD_SIGNAL_PAYLOAD_ONLY 0x100
+#define NVSHMEMI_AMD_SIGNAL_OP_MASK 0xff
 
 typedef int32_t nvshmem_team_t;
 #define NVSHMEM_TEAM_INVALID (-1)

@@ -243,6 +243,13 @@ typedef struct nvshmemi_device_state {
                             other than WORLD, low-latency counters of all teams */
     char *ll_buffers;    /* [MAX_TEAMS][npes][NVSHMEMI_AMD_LL_BUFFERS][2 * NVSHMEMI_AMD_LL_PAYLOAD_BYTES], then
                             [MAX_TEAMS][npes][NVSHMEMI_AMD_STAGE_BUFFERS][NVSHMEMI_AMD_STAGE_BYTES] */
+    uint64_t *runtime_words; /* one copy for the whole GPU (an address in PE 0's slice, used as it is):
+                                word NVSHMEMI_AMD_TIMEOUT_COUNT_WORD counts the bounded waits that gave up */
 } nvshmemi_device_state_t;
+
+#define NVSHMEMI_AMD_TIMEOUT_COUNT_WORD 0
+/* bytes at the end of every PE's slice that the runtime keeps for itself: barrier arrival row, epoch,
+ * timeout record and runtime words, 512 bytes each */
+#define NVSHMEMI_AMD_INTERNAL_BYTES (4 * 512)
 
 #endif

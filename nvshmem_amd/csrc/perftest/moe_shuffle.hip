@@ -94,7 +94,8 @@ template <bool WARP_SCOPED>
 __global__ void moe_dispatch_rowsignal_kernel(char *recv, const char *send, const int32_t *dest_pe,
                                               const int64_t *dest_row, const uint64_t *expected,
                                               uint64_t *sig, int tokens, int topk,
-                                              size_t row_bytes, size_t recv_cap_rows) {
+                                              size_t row_bytes, size_t recv_cap_rows, int sig_op,
+                                              int sig_stride) {
     const int me = nvshmem_my_pe(), np = nvshmem_n_pes();
     const int32_t *my_dest_pe = (const int32_t *)nvshmem_ptr(dest_pe, me);
     const int64_t *my_dest_row = (const int64_t *)nvshmem_ptr(dest_row, me);
@@ -103,22 +104,27 @@ __global__ void moe_dispatch_rowsignal_kernel(char *recv, const char *send, cons
         const size_t waves_per_block = blockDim.x / NVSHMEMI_WARP_SIZE;
         const size_t wave = blockIdx.x * waves_per_block + wave_in_block();
         const size_t nwaves = (size_t)gridDim.x * waves_per_block;
-        for (size_t r = wave; r < rows; r += nwaves)
-            if (row_ok(my_dest_pe[r], my_dest_row[r], np, recv_cap_rows))
-            nvshmemx_putmem_signal_nbi_warp(recv + (size_t)my_dest_row[r] * row_bytes,
-                                            send + (r / (size_t)topk) * row_bytes, row_bytes,
-                                            sig + me, 1, NVSHMEM_SIGNAL_ADD, my_dest_pe[r]);
+        // a wavefront takes a token and sends its topk copies one behind the other, so that the
+        // copies after the first find the row in this XCD's L2
+        for (size_t t = wave; t < (size_t)tokens; t += nwaves)
+            for (int k = 0; k < topk; ++k) {
+                const size_t r = t * (size_t)topk + (size_t)k;
+                if (row_ok(my_dest_pe[r], my_dest_row[r], np, recv_cap_rows))
+                    nvshmemx_putmem_signal_nbi_warp(recv + (size_t)my_dest_row[r] * row_bytes,
+                                                    send + t * row_bytes, row_bytes,
+                                                    sig + (size_t)me * sig_stride, 1, sig_op, my_dest_pe[r]);
+            }
     } else {
         for (size_t r = blockIdx.x; r < rows; r += gridDim.x)
             if (row_ok(my_dest_pe[r], my_dest_row[r], np, recv_cap_rows))
             nvshmemx_putmem_signal_nbi_block(recv + (size_t)my_dest_row[r] * row_bytes,
                                              send + (r / (size_t)topk) * row_bytes, row_bytes,
-                                             sig + me, 1, NVSHMEM_SIGNAL_ADD, my_dest_pe[r]);
+                                             sig + (size_t)me * sig_stride, 1, sig_op, my_dest_pe[r]);
     }
     if (blockIdx.x == 0) {
         const uint64_t *my_expected = (const uint64_t *)nvshmem_ptr(expected, me);
         for (int src = threadIdx.x; src < np; src += blockDim.x)
-            nvshmem_signal_wait_until(sig + src, NVSHMEM_CMP_GE, my_expected[src]);
+            nvshmem_signal_wait_until(sig + (size_t)src * sig_stride, NVSHMEM_CMP_GE, my_expected[src]);
     }
 }
 
@@ -328,25 +334,30 @@ bool moe_args_ok(const void *table_pe, const void *table_row, int tokens, int to
 extern "C" {
 
 // scope: NVSHMEM_PERFTEST_SCOPE_WARP (row per wavefront) or _BLOCK (row per block);
-// bit 8 set (scope | 256) selects per-row signalling instead of per-block tallies.
-int nvshmem_perftest_moe_dispatch_ex(void *recv, size_t recv_cap_rows, const void *send, const int32_t *dest_pe,
-                                     const int64_t *dest_row, const uint64_t *expected,
-                                     uint64_t *sig, int tokens, int topk, size_t row_bytes,
-                                     int blocks_per_pe, int threads, int scope, void *stream) {
+// bit 8 set (scope | 256) selects per-row signalling instead of per-block tallies, bit 9 (| 512) with
+// it the NVSHMEMX_AMD_SIGNAL_PAYLOAD_ONLY ordering of those signals.  The signal word of source PE s
+// is sig[s * sig_stride] (per-row signalling only; the tallies use stride 1).
+int nvshmem_perftest_moe_dispatch_put_signal(void *recv, size_t recv_cap_rows, const void *send,
+                                             const int32_t *dest_pe, const int64_t *dest_row,
+                                             const uint64_t *expected, uint64_t *sig, int sig_stride,
+                                             int tokens, int topk, size_t row_bytes, int blocks_per_pe,
+                                             int threads, int scope, void *stream) {
     const bool per_row = (scope & 256) != 0;
+    int sig_op = NVSHMEM_SIGNAL_ADD | ((scope & 512) ? NVSHMEMX_AMD_SIGNAL_PAYLOAD_ONLY : 0);
     const bool warp = (scope & 255) == NVSHMEM_PERFTEST_SCOPE_WARP;
     if (!warp && (scope & 255) != NVSHMEM_PERFTEST_SCOPE_BLOCK) return NVSHMEMX_ERROR_INVALID_VALUE;
+    if (sig_stride < 1 || (!per_row && sig_stride != 1)) return NVSHMEMX_ERROR_INVALID_VALUE;
     if (!moe_args_ok(dest_pe, dest_row, tokens, topk, row_bytes, blocks_per_pe, threads, warp))
         return NVSHMEMX_ERROR_INVALID_VALUE;
     const size_t words = sizeof(uint64_t) * (size_t)nvshmem_n_pes();
-    if (!perftest::check_range(expected, words) || !perftest::check_range(sig, words) ||
+    if (!perftest::check_range(expected, words) || !perftest::check_range(sig, words * (size_t)sig_stride) ||
         !perftest::check_range(send, (size_t)tokens * row_bytes) ||
         !perftest::check_range(recv, recv_cap_rows * row_bytes))
         return NVSHMEMX_ERROR_INVALID_VALUE;
     char *r = (char *)recv;
     const char *s = (const char *)send;
     void *args[] = {&r, &s, &dest_pe, &dest_row, &expected, &sig, &tokens, &topk, &row_bytes,
-                    &recv_cap_rows};
+                    &recv_cap_rows, &sig_op, &sig_stride};
     const void *fn;
     if (per_row)
         fn = warp ? (const void *)moe_dispatch_rowsignal_kernel<true>
@@ -355,6 +366,15 @@ int nvshmem_perftest_moe_dispatch_ex(void *recv, size_t recv_cap_rows, const voi
         fn = warp ? (const void *)moe_dispatch_kernel<true> : (const void *)moe_dispatch_kernel<false>;
     return nvshmemx_collective_launch(fn, dim3(blocks_per_pe), dim3(threads), args, 0,
                                       (hipStream_t)stream);
+}
+
+int nvshmem_perftest_moe_dispatch_ex(void *recv, size_t recv_cap_rows, const void *send, const int32_t *dest_pe,
+                                     const int64_t *dest_row, const uint64_t *expected,
+                                     uint64_t *sig, int tokens, int topk, size_t row_bytes,
+                                     int blocks_per_pe, int threads, int scope, void *stream) {
+    return nvshmem_perftest_moe_dispatch_put_signal(recv, recv_cap_rows, send, dest_pe, dest_row, expected, sig,
+                                                    1, tokens, topk, row_bytes, blocks_per_pe, threads, scope,
+                                                    stream);
 }
 
 int nvshmem_perftest_moe_dispatch(void *recv, size_t recv_cap_rows, const void *send, const int32_t *dest_pe,

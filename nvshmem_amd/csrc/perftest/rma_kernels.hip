@@ -7,9 +7,6 @@
 // examples/ring-reduce.cu:88-144.
 #include <hip/hip_runtime.h>
 
-// The kernels of this file move bulk data that is read once: stream the loads too.
-#define NVSHMEMI_AMD_COPY_NT 3
-
 #include "nvshmem_perftest.h"
 #include "nvshmemx.h"
 #include "perftest_common.hpp"
@@ -97,6 +94,54 @@ __global__ void pingpong_kernel(char *data, uint64_t *sig, size_t bytes, int ite
             nvshmemx_putmem_signal_block(data, data, bytes, sig, (uint64_t)i, NVSHMEM_SIGNAL_SET, 0);
         }
     }
+}
+
+// Ordering check for put-with-signal: even PEs stream `iters` messages to their odd neighbours
+// through a ring of `slots` buffers per block.  Message i of block b holds words mix(i, b, j); the
+// receiver waits for the i-th signal, reads the slot at once and counts the words that differ, then
+// returns a credit.  A signal that overtook its payload shows up as a word of an older message.
+__device__ __forceinline__ uint64_t stream_word(uint64_t i, uint64_t b, uint64_t j) {
+    uint64_t x = (i + 1) * 0x9E3779B97F4A7C15ull ^ (b + 1) * 0xC2B2AE3D27D4EB4Full ^ j * 0x165667B19E3779F9ull;
+    x ^= x >> 29;
+    return x * 0xBF58476D1CE4E5B9ull;
+}
+template <int SCOPE>
+__global__ void put_signal_stream_kernel(char *data, char *stage, uint64_t *sig, uint64_t *errors,
+                                         size_t bytes, int slots, int iters, int sig_op) {
+    const int me = nvshmem_my_pe(), peer = me ^ 1;
+    if (peer >= nvshmem_n_pes()) return;
+    const bool sender = (me & 1) == 0;
+    const size_t b = blockIdx.x, words = bytes / 8;
+    char *slot_base = data + b * (size_t)slots * bytes;
+    char *my_stage = stage + b * bytes;
+    uint64_t *data_sig = sig + 2 * b, *credit = sig + 2 * b + 1;
+    unsigned long long bad = 0;
+    for (int i = 0; i < iters; ++i) {
+        char *slot = slot_base + (size_t)(i % slots) * bytes;
+        if (sender) {
+            if (i >= slots) {
+                if (threadIdx.x == 0) nvshmem_signal_wait_until(credit, NVSHMEM_CMP_GE, (uint64_t)(i - slots + 1));
+                __syncthreads();
+            }
+            uint64_t *st = (uint64_t *)nvshmem_ptr(my_stage, me);
+            for (size_t j = threadIdx.x; j < words; j += blockDim.x) st[j] = stream_word(i, b, j);
+            __syncthreads();
+            if (SCOPE == NVSHMEM_PERFTEST_SCOPE_BLOCK)
+                nvshmemx_putmem_signal_nbi_block(slot, my_stage, bytes, data_sig, 1, sig_op, peer);
+            else if (SCOPE == NVSHMEM_PERFTEST_SCOPE_WARP)
+                nvshmemx_putmem_signal_nbi_warp(slot, my_stage, bytes, data_sig, 1, sig_op, peer);
+            else
+                nvshmem_putmem_signal_nbi(slot, my_stage, bytes, data_sig, 1, sig_op, peer);
+        } else {
+            if (threadIdx.x == 0) nvshmem_signal_wait_until(data_sig, NVSHMEM_CMP_GE, (uint64_t)(i + 1));
+            __syncthreads();
+            const uint64_t *got = (const uint64_t *)nvshmem_ptr(slot, me);
+            for (size_t j = threadIdx.x; j < words; j += blockDim.x) bad += got[j] != stream_word(i, b, j);
+            __syncthreads();
+            if (threadIdx.x == 0) nvshmemx_signal_op(credit, 1, NVSHMEM_SIGNAL_ADD, peer);
+        }
+    }
+    if (bad) atomicAdd((unsigned long long *)nvshmem_ptr(errors, me), bad);
 }
 
 // every PE's copy of `words` := value, in one launch (stream ordered, unlike a memset per PE)
@@ -383,6 +428,28 @@ int nvshmem_perftest_put_signal_pingpong(void *data, uint64_t *sig, size_t bytes
     void *args[] = {&d, &sig, &bytes, &iters};
     return nvshmemx_collective_launch((const void *)pingpong_kernel, dim3(1), dim3(threads), args,
                                       0, (hipStream_t)stream);
+}
+
+int nvshmem_perftest_put_signal_stream(void *data, void *stage, uint64_t *sig, uint64_t *errors,
+                                       size_t bytes, int slots, int iters, int blocks, int scope,
+                                       int sig_op, void *stream) {
+    const int threads = scope == NVSHMEM_PERFTEST_SCOPE_BLOCK ? 256 : scope == NVSHMEM_PERFTEST_SCOPE_WARP ? 64 : 1;
+    if (!perftest::ready() || nvshmem_n_pes() < 2 || bytes == 0 || bytes % 8 || slots < 1 || iters < 1 ||
+        scope < NVSHMEM_PERFTEST_SCOPE_THREAD || scope > NVSHMEM_PERFTEST_SCOPE_BLOCK ||
+        !perftest::check_launch(blocks, threads) ||
+        !perftest::check_range(data, (size_t)blocks * (size_t)slots * bytes) ||
+        !perftest::check_range(stage, (size_t)blocks * bytes) ||
+        !perftest::check_range(sig, 2 * sizeof(uint64_t) * (size_t)blocks) ||
+        !perftest::check_range(errors, sizeof(uint64_t)))
+        return NVSHMEMX_ERROR_INVALID_VALUE;
+    const int op = sig_op & NVSHMEMI_AMD_SIGNAL_OP_MASK;
+    if (op != NVSHMEM_SIGNAL_ADD) return NVSHMEMX_ERROR_INVALID_VALUE;
+    char *d = (char *)data, *st = (char *)stage;
+    void *args[] = {&d, &st, &sig, &errors, &bytes, &slots, &iters, &sig_op};
+    const void *fn = scope == NVSHMEM_PERFTEST_SCOPE_BLOCK  ? (const void *)put_signal_stream_kernel<NVSHMEM_PERFTEST_SCOPE_BLOCK>
+                     : scope == NVSHMEM_PERFTEST_SCOPE_WARP ? (const void *)put_signal_stream_kernel<NVSHMEM_PERFTEST_SCOPE_WARP>
+                                                            : (const void *)put_signal_stream_kernel<NVSHMEM_PERFTEST_SCOPE_THREAD>;
+    return nvshmemx_collective_launch(fn, dim3(blocks), dim3(threads), args, 0, (hipStream_t)stream);
 }
 
 int nvshmem_perftest_fill_words(uint64_t *words, uint64_t value, size_t nwords, void *stream) {

@@ -136,7 +136,7 @@ int nvshmemx_amd_init(int npes, size_t symmetric_size) {
     const uint64_t min_slice = 1ull << 16;
     uint64_t want = symmetric_size < min_slice ? min_slice : (uint64_t)symmetric_size;
     // room for the runtime's own symmetric words (barrier row, epoch, timeout record)
-    want += 4 * NVSHMEMI_MALLOC_ALIGNMENT;
+    want += NVSHMEMI_AMD_INTERNAL_BYTES;
     uint32_t shift = 16;
     while ((1ull << shift) < want) {
         if (++shift > 40) {
@@ -172,7 +172,7 @@ int nvshmemx_amd_init(int npes, size_t symmetric_size) {
     // The runtime's own symmetric words (barrier row, epoch, timeout record) live in the last
     // granules of every slice, outside the allocator's space, so that user allocations start at the
     // slice base: large buffers then sit on the 1 KiB boundaries the streaming kernels like.
-    const uint64_t internal_bytes = 4 * NVSHMEMI_MALLOC_ALIGNMENT;
+    const uint64_t internal_bytes = NVSHMEMI_AMD_INTERNAL_BYTES;
     rt.space.reset(new SymmetricSpace((uint64_t)(uintptr_t)rt.base, rt.heap_size - internal_bytes));
     rt.initialized = true;
     const uint64_t internal = (uint64_t)(uintptr_t)rt.base + rt.heap_size - internal_bytes;
@@ -192,6 +192,7 @@ int nvshmemx_amd_init(int npes, size_t symmetric_size) {
     rt.dev.sync_flags = (uint64_t *)(uintptr_t)flags;
     rt.dev.sync_epoch = (uint64_t *)(uintptr_t)epoch;
     rt.dev.timeout_record = (uint64_t *)(uintptr_t)trec;
+    rt.dev.runtime_words = (uint64_t *)(uintptr_t)(trec + NVSHMEMI_MALLOC_ALIGNMENT);
     rt.dev.spin_limit = env_size("NVSHMEM_AMD_SPIN_LIMIT", 1ull << 22);
     rt.plain_collective_launch = env_size("NVSHMEM_AMD_PLAIN_COLLECTIVE_LAUNCH", 0) != 0;
     rt.cacheable_source_bytes = env_size("NVSHMEM_AMD_CACHEABLE_SOURCE_BYTES", (size_t)256 << 20);
@@ -531,6 +532,7 @@ void nvshmemx_signal_op_on_stream(uint64_t *sig_addr, uint64_t signal, int sig_o
     char *target = nullptr;
     if (!rma_target(rt, "nvshmemx_signal_op_on_stream", sig_addr, sizeof(uint64_t), pe, &target))
         return;
+    sig_op &= NVSHMEMI_AMD_SIGNAL_OP_MASK;  // an ordering hint means nothing here: stream order already orders
     if (sig_op != NVSHMEM_SIGNAL_SET && sig_op != NVSHMEM_SIGNAL_ADD) {
         set_error("nvshmemx_signal_op_on_stream: sig_op %d is neither SET (9) nor ADD (10)", sig_op);
         return;

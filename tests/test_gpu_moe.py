@@ -148,3 +148,46 @@ def test_config5_full_size_moe_shuffle():
     need = int(recv_rows.max()) * row + T * K * row + T * row + (64 << 20)
     with runtime(npes, need) as rt:
         _shuffle(rt, npes, T, K, E, row, 64, 256, N.SCOPE_WARP, check_exchange=True)
+
+
+@pytest.mark.parametrize("scope,blocks,threads", [(N.SCOPE_WARP | 256 | 512, 64, 256), (N.SCOPE_BLOCK | 256 | 512, 128, 256),
+                                                   (N.SCOPE_WARP | 256, 64, 256)])
+def test_config5_full_size_dispatch_through_per_row_put_signal(scope, blocks, threads):
+    """Config 5 at full size with one nvshmemx_putmem_signal_nbi per row copy (ADD 1 on the signal word of
+    the source at the destination) and nvshmem_signal_wait_until(GE) on the receiver: every PE's receive
+    buffer bit-exact against the oracle, signal counts exact.  Signal words sit on separate 128-byte
+    lines (stride 16).  Payload-only ordering in both scopes, the reference's ordering once."""
+    npes, T, K, E, row = 8, 8192, 8, 256, 7168 * 2
+    ex = O.moe_routing(npes, T, K, E, 1.1, 8)
+    counts, _, dest_pe, dest_row, recv_rows = O.moe_plan(ex, npes, T, K, E)
+    cap, rows, stride = int(recv_rows.max()), T * K, 16
+    with runtime(npes, cap * row + T * row + (64 << 20)) as rt:
+        perf = rt.perftest()
+        send = rt.malloc(T * row); recv = rt.malloc(cap * row)
+        d_pe = rt.malloc(rows * 4); d_row = rt.malloc(rows * 8)
+        expected = rt.malloc(npes * 8); sig = rt.calloc(npes * stride, 8)
+        payload = np.stack([O.fill("bytes", T * row, 7, pe).reshape(T, row) for pe in range(npes)])
+        rt.upload_all(send, payload); rt.upload_all(d_pe, dest_pe); rt.upload_all(d_row, dest_row)
+        epp = E // npes
+        exp_tab = np.stack([[counts[src, d * epp:(d + 1) * epp].sum() for src in range(npes)]
+                            for d in range(npes)]).astype(np.uint64)
+        rt.upload_all(expected, exp_tab)
+        rt.fill(recv, 0, cap * row)
+        note("moe_dispatch_put_signal full size scope=%#x blocks=%d threads=%d" % (scope, blocks, threads))
+        assert perf.nvshmem_perftest_moe_dispatch_put_signal(recv, cap, send, d_pe, d_row, expected, sig, stride,
+                                                             T, K, row, blocks, threads, scope, None) == 0
+        rt.sync()
+        assert all(rt.read_timeout(pe)[0] == 0 for pe in range(npes)), "a receiver gave up waiting"
+        want_recv = O.moe_dispatch(payload, dest_pe, dest_row, recv_rows, T, K)
+        for pe in range(npes):
+            got = rt.download(recv, pe, (int(recv_rows[pe]), row), np.uint8)
+            assert np.array_equal(got, want_recv[pe]), pe
+        sigs = rt.download_all(sig, (npes * stride,), np.uint64).reshape(npes, npes, stride)
+        assert np.array_equal(sigs[:, :, 0], exp_tab) and (sigs[:, :, 1:] == 0).all()
+        # argument checks
+        assert perf.nvshmem_perftest_moe_dispatch_put_signal(recv, cap, send, d_pe, d_row, expected, sig, 0,
+                                                             T, K, row, blocks, threads, scope, None) != 0
+        assert perf.nvshmem_perftest_moe_dispatch_put_signal(recv, cap, send, d_pe, d_row, expected, sig, 2,
+                                                             T, K, row, 32, 256, N.SCOPE_WARP, None) != 0
+        for p in (send, recv, d_pe, d_row, expected, sig):
+            rt.free(p)

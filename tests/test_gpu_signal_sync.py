@@ -231,6 +231,37 @@ def test_ring_allreduce_from_put_signal_known_answer_and_oracle(rt):
     rt.free(dst); rt.free(src); rt.free(sig)
 
 
+PAYLOAD_ONLY = 0x100      # NVSHMEMX_AMD_SIGNAL_PAYLOAD_ONLY
+SIGNAL_ADD = 10
+
+
+@pytest.mark.parametrize("sig_op", [SIGNAL_ADD, SIGNAL_ADD | PAYLOAD_ONLY])
+def test_put_signal_never_overtakes_its_payload(rt, sig_op):
+    """Receivers read every message inside the kernel, straight after signal_wait_until returns: a
+    signal that arrived ahead of its payload would leave words of an older message in the slot.  Both
+    orderings of put-with-signal (the reference's full release and the payload-only hint), all three
+    scopes, message sizes with and without the long-copy rounds, four PE pairs at once."""
+    perf = rt.perftest()
+    for scope, nbytes, slots, iters, blocks in ((N.SCOPE_BLOCK, 14336, 3, 200, 8), (N.SCOPE_BLOCK, 1 << 20, 2, 12, 4),
+                                                (N.SCOPE_WARP, 14336, 4, 200, 16), (N.SCOPE_WARP, 40, 2, 300, 4),
+                                                (N.SCOPE_WARP, 65536, 2, 40, 8), (N.SCOPE_THREAD, 256, 2, 50, 2)):
+        data = rt.malloc(blocks * slots * nbytes); stage = rt.malloc(blocks * nbytes)
+        sig = rt.calloc(2 * blocks, 8); errors = rt.calloc(1, 8)
+        rt.fill(data, 0xFF, blocks * slots * nbytes)
+        note("put_signal stream scope=%d bytes=%d slots=%d iters=%d blocks=%d sig_op=%#x"
+             % (scope, nbytes, slots, iters, blocks, sig_op))
+        assert perf.nvshmem_perftest_put_signal_stream(data, stage, sig, errors, nbytes, slots, iters, blocks,
+                                                       scope, sig_op, None) == 0
+        rt.sync()
+        assert all(rt.read_timeout(pe)[0] == 0 for pe in range(NPES))
+        assert (_words(rt, errors)[:, 0] == 0).all(), _words(rt, errors)[:, 0]
+        s = _words(rt, sig, 2 * blocks).reshape(NPES, blocks, 2)
+        assert (s[1::2, :, 0] == iters).all() and (s[0::2, :, 1] == iters).all()   # data counts, credits
+        for p in (data, stage, sig, errors):
+            rt.free(p)
+    assert perf.nvshmem_perftest_put_signal_stream(0, 0, 0, 0, 12, 1, 1, 1, N.SCOPE_BLOCK, sig_op, None) != 0
+
+
 def test_collective_launch_refuses_grids_that_cannot_be_co_resident(rt):
     perf = rt.perftest()
     dst = rt.calloc(1 << 20, 4); src = rt.calloc(1 << 20, 4); sig = rt.calloc(65535, 8)
