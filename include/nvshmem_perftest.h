@@ -264,6 +264,17 @@ int nvshmem_perftest_moe_dispatch_pieces(void *recv, size_t recv_cap_rows, const
                                          const int32_t *dest_pe, const int64_t *dest_row,
                                          const uint64_t *expected, uint64_t *sig, int tokens, int topk,
                                          size_t row_bytes, int piece_bytes, int threads, void *stream);
+/* nvshmem_perftest_moe_dispatch_pieces for callers that cannot allocate (code under HIP graph capture,
+ * serving loops, harnesses that forbid hipMalloc).  No counterpart in the reference.  It takes no signal
+ * words from the caller: they live in a static device array of the library (8 KiB per GPU, rows for at
+ * most 32 PEs; more PEs are refused with NVSHMEMX_ERROR_INVALID_VALUE and a message), which a kernel on
+ * `stream` clears before the rows are sent.  It calls no hipMalloc, hipFree or other allocating routine.
+ * All calls on one GPU share that array: calls that overlap in time on one GPU race. */
+int nvshmem_perftest_moe_dispatch_pieces_static(void *recv, size_t recv_cap_rows, const void *send,
+                                                const int32_t *dest_pe, const int64_t *dest_row,
+                                                const uint64_t *expected, int tokens, int topk,
+                                                size_t row_bytes, int piece_bytes, int threads,
+                                                void *stream);
 /* The same with a work item of piece_bytes (1024, 2048 or 4096; wavefront scope) of a row instead of
  * a whole row (0): with 2 KiB items and one wavefront per block every block moves one short piece
  * and exits. */

@@ -18,6 +18,13 @@
 #include "nvshmemx.h"
 #include "perftest_common.hpp"
 
+// Signal words of the dispatch that allocates nothing (nvshmem_perftest_moe_dispatch_pieces_static):
+// kStaticSignalPes rows of kStaticSignalPes words, 8 KiB.  Device memory of this code object: every GPU
+// the library runs on holds its own copy, at its own address, until the process ends.  In host code the
+// name is only a handle for hipGetSymbolAddress; kernels get the address that call returns.
+constexpr int kStaticSignalPes = 32;
+static __device__ __align__(256) uint64_t scratch[kStaticSignalPes * kStaticSignalPes];
+
 namespace {
 
 constexpr int kMaxPes = NVSHMEMI_AMD_MAX_PES;
@@ -206,6 +213,10 @@ __global__ void moe_dispatch_direct_kernel(char *recv, const char *send, const i
 // A few blocks per PE: each counts the rows of its share that this PE sent to every destination and
 // adds the counts to the destinations' signal words; block 0 then waits until every source has
 // announced what this PE expects.
+// SYMMETRIC: `sig` is a symmetric array of npes words per PE, updated with nvshmemx_signal_op.  Otherwise
+// it is an ordinary device array of npes rows of npes words (row p = the signal words of PE p), which
+// the symmetric-address API cannot name, so the words are updated with the same agent-scope add directly.
+template <bool SYMMETRIC>
 __global__ void moe_dispatch_signal_kernel(const int32_t *dest_pe, const int64_t *dest_row,
                                            const uint64_t *expected, uint64_t *sig, int tokens,
                                            int topk, size_t recv_cap_rows) {
@@ -248,11 +259,17 @@ __global__ void moe_dispatch_signal_kernel(const int32_t *dest_pe, const int64_t
     if ((int)lane < np && mine) atomicAdd(&tally[lane], mine);
     __syncthreads();
     for (int pe = threadIdx.x; pe < np; pe += blockDim.x)
-        if (tally[pe]) nvshmemx_signal_op(sig + me, (uint64_t)tally[pe], NVSHMEM_SIGNAL_ADD, pe);
+        if (tally[pe]) {
+            if (SYMMETRIC) nvshmemx_signal_op(sig + me, (uint64_t)tally[pe], NVSHMEM_SIGNAL_ADD, pe);
+            else __hip_atomic_fetch_add(sig + (size_t)pe * np + me, (uint64_t)tally[pe], __ATOMIC_RELAXED,
+                                        __HIP_MEMORY_SCOPE_AGENT);
+        }
     if (blockIdx.x != 0) return;
     const uint64_t *my_expected = (const uint64_t *)nvshmem_ptr(expected, me);
+    // (an address outside the symmetric heap is waited on as it is)
+    uint64_t *my_words = SYMMETRIC ? sig : sig + (size_t)me * np;
     for (int src = threadIdx.x; src < np; src += blockDim.x)
-        nvshmem_signal_wait_until(sig + src, NVSHMEM_CMP_GE, my_expected[src]);
+        nvshmem_signal_wait_until(my_words + src, NVSHMEM_CMP_GE, my_expected[src]);
 }
 
 // PIECE > 0 (wavefront scope): a work item is PIECE bytes of a row instead of a whole row, so that
@@ -313,6 +330,34 @@ __global__ void moe_exchange_offsets_kernel(const int64_t *counts, int64_t *seg_
         }
         if (d == me) ((int64_t *)nvshmem_ptr(recv_rows, me))[0] = run;
     }
+}
+
+__global__ void clear_words_kernel(uint64_t *words, unsigned n) {
+    const unsigned i = blockIdx.x * blockDim.x + threadIdx.x;
+    if (i < n) words[i] = 0;
+}
+
+// Address of this device's copy of `scratch`, looked up once per device.
+constexpr int kMaxDevices = 64;
+uint64_t *scratch_address() {
+    static uint64_t *ptr[kMaxDevices];
+    int dev = -1;
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= kMaxDevices) {
+        (void)hipGetLastError();
+        fprintf(stderr, "nvshmem_perftest: no current device for the static signal words\n");
+        return nullptr;
+    }
+    if (!ptr[dev]) {
+        void *p = nullptr;
+        const hipError_t e = hipGetSymbolAddress(&p, HIP_SYMBOL(scratch));
+        if (e != hipSuccess || !p) {
+            (void)hipGetLastError();
+            fprintf(stderr, "nvshmem_perftest: hipGetSymbolAddress(scratch) failed: %s\n", hipGetErrorString(e));
+            return nullptr;
+        }
+        ptr[dev] = (uint64_t *)p;
+    }
+    return ptr[dev];
 }
 
 bool moe_args_ok(const void *table_pe, const void *table_row, int tokens, int topk,
@@ -390,17 +435,20 @@ int nvshmem_perftest_moe_dispatch(void *recv, size_t recv_cap_rows, const void *
 // 2048 / 4096) of a token's row, pushed to its topk destinations - then one block per PE that
 // publishes the row counts through the signal words and waits for the expected ones.  `threads` (a
 // multiple of 64) sets how many tokens a block takes.
-int nvshmem_perftest_moe_dispatch_pieces(void *recv, size_t recv_cap_rows, const void *send,
-                                         const int32_t *dest_pe, const int64_t *dest_row,
-                                         const uint64_t *expected, uint64_t *sig, int tokens, int topk,
-                                         size_t row_bytes, int piece_bytes, int threads, void *stream) {
+// static_sig: the signal words are this device's `scratch` rows (cleared here, on the stream, by a
+// kernel) instead of the caller's symmetric array.
+static int dispatch_pieces(void *recv, size_t recv_cap_rows, const void *send, const int32_t *dest_pe,
+                           const int64_t *dest_row, const uint64_t *expected, uint64_t *sig,
+                           uint64_t *static_sig, int tokens, int topk, size_t row_bytes, int piece_bytes,
+                           int threads, void *stream) {
     if (piece_bytes != 1024 && piece_bytes != 2048 && piece_bytes != 4096) return NVSHMEMX_ERROR_INVALID_VALUE;
     if (!moe_args_ok(dest_pe, dest_row, tokens, topk, row_bytes, 1, threads, true))
         return NVSHMEMX_ERROR_INVALID_VALUE;
     const size_t words = sizeof(uint64_t) * (size_t)nvshmem_n_pes();
     const size_t pieces = (row_bytes + (size_t)piece_bytes - 1) / (size_t)piece_bytes;
     if (pieces > 0x7fffffffull || !perftest::check_range(expected, words) ||
-        !perftest::check_range(sig, words) || !perftest::check_range(send, (size_t)tokens * row_bytes) ||
+        (!static_sig && !perftest::check_range(sig, words)) ||
+        !perftest::check_range(send, (size_t)tokens * row_bytes) ||
         !perftest::check_range(recv, recv_cap_rows * row_bytes))
         return NVSHMEMX_ERROR_INVALID_VALUE;
     const unsigned waves = (unsigned)threads / NVSHMEMI_WARP_SIZE;
@@ -413,6 +461,12 @@ int nvshmem_perftest_moe_dispatch_pieces(void *recv, size_t recv_cap_rows, const
     unsigned kshift = 0;
     while (((topk + (1 << kshift) - 1) >> kshift) > 4) ++kshift;
     const dim3 dgrid(grid.x << kshift, grid.y, grid.z);
+    if (static_sig) {
+        const unsigned n = (unsigned)(nvshmem_n_pes() * nvshmem_n_pes());
+        hipLaunchKernelGGL(clear_words_kernel, dim3((n + 255) / 256), dim3(256), 0, (hipStream_t)stream, static_sig, n);
+        const int rc0 = perftest::launch_status("clear_words");
+        if (rc0 != 0) return rc0;
+    }
 #define LAUNCH_DIRECT(V)                                                                           \
     hipLaunchKernelGGL((moe_dispatch_direct_kernel<V>), dgrid, dim3(threads), 0, (hipStream_t)stream, \
                        (char *)recv, (const char *)send, dest_pe, dest_row, tokens, topk, row_bytes, \
@@ -436,9 +490,39 @@ int nvshmem_perftest_moe_dispatch_pieces(void *recv, size_t recv_cap_rows, const
     // few blocks per PE - still at most 512 in all, co-resident on this GPU, so an ordinary launch is
     // enough for the waits - the scan is short
     const unsigned sig_blocks = (unsigned)(((size_t)tokens * (size_t)topk + 8191) / 8192 < 8 ? ((size_t)tokens * (size_t)topk + 8191) / 8192 : 8);
-    hipLaunchKernelGGL(moe_dispatch_signal_kernel, dim3(sig_blocks, 1, (unsigned)nvshmem_n_pes()), dim3(1024), 0,
-                       (hipStream_t)stream, dest_pe, dest_row, expected, sig, tokens, topk, recv_cap_rows);
+    if (static_sig)
+        hipLaunchKernelGGL(moe_dispatch_signal_kernel<false>, dim3(sig_blocks, 1, (unsigned)nvshmem_n_pes()), dim3(1024),
+                           0, (hipStream_t)stream, dest_pe, dest_row, expected, static_sig, tokens, topk, recv_cap_rows);
+    else
+        hipLaunchKernelGGL(moe_dispatch_signal_kernel<true>, dim3(sig_blocks, 1, (unsigned)nvshmem_n_pes()), dim3(1024),
+                           0, (hipStream_t)stream, dest_pe, dest_row, expected, sig, tokens, topk, recv_cap_rows);
     return perftest::launch_status("moe_dispatch_signal");
+}
+
+int nvshmem_perftest_moe_dispatch_pieces(void *recv, size_t recv_cap_rows, const void *send,
+                                         const int32_t *dest_pe, const int64_t *dest_row,
+                                         const uint64_t *expected, uint64_t *sig, int tokens, int topk,
+                                         size_t row_bytes, int piece_bytes, int threads, void *stream) {
+    return dispatch_pieces(recv, recv_cap_rows, send, dest_pe, dest_row, expected, sig, nullptr, tokens, topk,
+                           row_bytes, piece_bytes, threads, stream);
+}
+
+int nvshmem_perftest_moe_dispatch_pieces_static(void *recv, size_t recv_cap_rows, const void *send,
+                                                const int32_t *dest_pe, const int64_t *dest_row,
+                                                const uint64_t *expected, int tokens, int topk,
+                                                size_t row_bytes, int piece_bytes, int threads,
+                                                void *stream) {
+    if (!perftest::ready()) return NVSHMEMX_ERROR_INVALID_VALUE;
+    if (nvshmem_n_pes() > kStaticSignalPes) {
+        fprintf(stderr, "nvshmem_perftest_moe_dispatch_pieces_static: %d PEs, the static signal words hold %d; "
+                        "use nvshmem_perftest_moe_dispatch_pieces with signal words of your own\n",
+                nvshmem_n_pes(), kStaticSignalPes);
+        return NVSHMEMX_ERROR_INVALID_VALUE;
+    }
+    uint64_t *words = scratch_address();
+    if (!words) return NVSHMEMX_ERROR_INTERNAL;
+    return dispatch_pieces(recv, recv_cap_rows, send, dest_pe, dest_row, expected, nullptr, words, tokens, topk,
+                           row_bytes, piece_bytes, threads, stream);
 }
 
 // piece_bytes: 0 = a work item is a whole row; 1024 / 2048 / 4096 (wavefront scope only) = a work
