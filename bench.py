@@ -1,20 +1,23 @@
 #!/usr/bin/env python3
 """Benchmark of the NVSHMEM data-movement hot path on one MI355X.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--only name,name]
 
-Prints ONE JSON line.  The headline workload is put_block at the largest size of the put/get
-sweep: every one of 8 logical PEs moves 256 MiB to its right neighbour with
-nvshmemx_putmem_block; a "step" is one such exchange (one kernel launch carrying all PEs).
-`value` is algorithmic bytes (payload read once + written once, all PEs) per second, inputs
-already resident in HBM.  sum_reduce (fp32, 8 PEs x 2^26 elements) and alltoall (fp32, 16 PEs x 2^22
-elements), a 1 GiB alltoall, reducescatter and broadcast are measured the same way and reported under
-"workloads".  The CPU oracle is timed on
-a bounded sample of each workload on this host's cores as a reported baseline.
+Prints ONE JSON line.  The headline workload is put_block on the put/get sweep's own launch shape at
+its largest size: every one of 8 logical PEs moves 256 MiB to its right neighbour with
+nvshmemx_putmem_block from 16 blocks of 1024 threads, block b moving the b-th contiguous slice; a
+"step" is one such exchange (one kernel launch carrying all PEs).  `value` is algorithmic bytes
+(payload read once + written once, all PEs) per second, inputs already resident in HBM.  Every other
+configuration of the sweep - put and get at 64 and 256 MiB from 1 / 4 / 16 blocks, the launch shape
+that fills the GPU, the reductions, fcollect / alltoall, reducescatter, broadcast and the MoE token
+shuffle - is measured the same way and reported under "workloads", each verified against the CPU
+oracle and each with the oracle's own rate on this host (one thread, and all threads OpenMP gives).
 """
 import argparse
+import glob
 import json
 import os
+import re
 import sys
 import time
 
@@ -25,30 +28,19 @@ sys.path.insert(0, os.path.join(ROOT, "tests"))
 HBM_PEAK_GBS = 8000.0   # MI355X published HBM3E peak
 METRIC = "achieved GB/s and % of HBM peak: put_block, sum_reduce, alltoall (1 GPU)"
 
-# HBM bytes per launch measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE (scaled by the plain
-# copy calibration kernel; summaries under profiles/): read + write, equal to the algorithmic bytes.
-MEASURED_TRAFFIC_BYTES = {
-    "put_block": (2048 + 2048) << 20,    # profiles/ring_rma_kernel_put_block_8pe_256MiB.txt
-    "sum_reduce": (2048 + 2048) << 20,   # profiles/reduce_vector_kernel_float_sum_8pe_64Mi.txt
-    "alltoall": (256 + 256) << 20,       # profiles/segment_copy_kernel_alltoall_16pe_4Mi_fp32.txt
-    "alltoall_1GiB": None,              # not profiled
-    "reducescatter": (2048 + 256) << 20,  # profiles/reducescatter_gather_kernel_float_sum_8pe_8Mi.txt
-    "broadcast": (256 + 2048) << 20,      # profiles/segment_copy_kernel_broadcast_8pe_256MiB.txt
-    "fcollect": (256 + 4096) << 20,       # profiles/segment_copy_kernel_fcollect_16pe_4Mi_fp32.txt
-    # fabric traffic: two blocks share a piece and both fetch it (the second from the Infinity Cache)
-    "moe_dispatch": (1840 + 7168) << 20,  # profiles/moe_dispatch_direct_kernel_8pe_8192tok_top8.txt
-    "moe_combine": (7216 + 7168) << 20,   # profiles/moe_combine_kernel_8pe_8192tok_top8.txt
-}
 
-# put_block launch shape: each block is one wavefront that moves a contiguous 1 KiB slice, one
-# 16-byte vector per lane (short-lived blocks keep the set of addresses in flight narrow, which is
-# what HBM serves fastest; two vectors per lane measure 8 % slower)
-PUT_BYTES = 1 << 28
-PUT_BLOCKS_PER_PE = 262144
-PUT_THREADS = 64
+def measured_traffic(name):
+    """HBM bytes per launch of the workload's dominant kernel, from the rocprofv3 FETCH_SIZE / WRITE_SIZE
+    summary committed under profiles/ (None when there is none)."""
+    for path in glob.glob(os.path.join(ROOT, "profiles", "*__%s.txt" % name)):
+        with open(path) as fh:
+            m = re.search(r"^measured_traffic_bytes: (\d+) read \+ (\d+) written", fh.read(), re.M)
+        if m:
+            return int(m.group(1)) + int(m.group(2))
+    return None
 
 
-def _time_steps(fn, steps, warmup, hip):
+def time_steps(fn, steps, warmup, hip):
     """(wall ms per step, event ms per step): K launches bracketed by device synchronisation."""
     for _ in range(warmup):
         fn()
@@ -66,8 +58,7 @@ def _time_steps(fn, steps, warmup, hip):
     return wall, ev
 
 
-def _cpu_time(fn, budget_s, max_passes):
-    """Best wall time of fn over passes that fit the budget."""
+def cpu_time(fn, budget_s, max_passes=20):
     best, spent, passes = None, 0.0, 0
     while passes < max_passes and (spent < budget_s or passes == 0):
         t0 = time.perf_counter()
@@ -79,360 +70,196 @@ def _cpu_time(fn, budget_s, max_passes):
     return best, passes
 
 
-def bench_put_block(N, O, hip, np, steps, warmup, cpu_budget):
-    npes, S = 8, PUT_BYTES
-    with _runtime(N, npes, 2 * S + (64 << 20)) as rt:
-        perf = rt.perftest()
-        src = rt.malloc(S); dst = rt.malloc(S)
-        data = O.fill_all("bytes", npes, S, 2)
-        rt.upload_all(src, data)
-        rt.fill(dst, 0, S)
+class Checker:
+    """Verification against the oracle and the oracle's own rate, per kind of workload."""
 
-        def step():
-            rc = perf.nvshmem_perftest_ring_rma(dst, src, S, PUT_BLOCKS_PER_PE, PUT_THREADS,
-                                                N.SCOPE_BLOCK, 0, 1, None)
-            if rc != 0:
-                raise RuntimeError("ring_rma failed: %d" % rc)
-        wall, ev = _time_steps(step, steps, warmup, hip)
-        # parity spot check on the timed output: PE 3 must hold PE 2's payload
-        got = rt.download(dst, 3, (S,), np.uint8)
-        ok = bool(np.array_equal(got, data[2]))
-        rt.free(src); rt.free(dst)
-    alg = 2 * npes * S
-    # CPU oracle: the same exchange with memcpy on a 64 MiB-per-PE sample, into a destination that
-    # has been touched before, with all the cores this process may use and with one
-    sample = 1 << 26
-    host_src = data[:, :sample].copy()
-    host_dst = np.zeros_like(host_src)
-    cores = min(16, O.lib().oracle_get_threads())
-    O.lib().oracle_set_threads(1)
-    one, _ = _cpu_time(lambda: O.ring_put(host_src, host_dst), cpu_budget / 2, 20)
-    O.lib().oracle_set_threads(cores)
-    best, passes = _cpu_time(lambda: O.ring_put(host_src, host_dst), cpu_budget / 2, 40)
-    cpu = {"value": round(2 * npes * sample / best / 1e9, 2), "unit": "GB/s", "cores": cores,
-           "kind": "port", "sample": "oracle_ring_put, 8 PEs x 64 MiB, best of %d passes" % passes,
-           "single_thread": round(2 * npes * sample / one / 1e9, 2)}
-    return {
-        "name": "put_block", "dtype": "u8", "verified": ok, "algorithmic_bytes": alg,
-        "wall_ms": wall, "kernel_ms": ev,
-        "config": {"workload": "put_block: nvshmemx_putmem_block ring, 8 logical PEs x 256 MiB "
-                               "(largest size of the put/get sweep)",
-                   "npes": npes, "bytes_per_pe": S, "blocks_per_pe": PUT_BLOCKS_PER_PE,
-                   "threads_per_block": PUT_THREADS,
-                   "payload_only_GBs": round(npes * S / ev / 1e6, 1)},
-        "kernel": "ring_rma_kernel<BLOCK, put> (nvshmemi_memcpy_threadgroup)",
-        "cpu_baseline": cpu,
-    }
+    def __init__(self, O, np, cpu_seconds):
+        self.O, self.np, self.budget = O, np, cpu_seconds
+        self.cores = O.lib().oracle_get_threads()      # what OpenMP gives this process on this host
 
+    def baseline(self, fn, bytes_moved, sample):
+        """Two rows: one thread, and all threads."""
+        O = self.O
+        O.lib().oracle_set_threads(1)
+        one, _ = cpu_time(fn, self.budget / 2)
+        O.lib().oracle_set_threads(self.cores)
+        best, passes = cpu_time(fn, self.budget / 2)
+        return {"value": round(bytes_moved / best / 1e9, 2), "unit": "GB/s", "cores": self.cores, "kind": "port",
+                "sample": "%s, best of %d passes" % (sample, passes),
+                "single_thread": round(bytes_moved / one / 1e9, 2)}
 
-def bench_sum_reduce(N, O, hip, np, steps, warmup, cpu_budget):
-    npes, n = 8, 1 << 26
-    with _runtime(N, npes, 2 * n * 4 + (64 << 20)) as rt:
-        src = rt.malloc(n * 4); dst = rt.malloc(n * 4)
-        data = O.fill_all("f32", npes, n, 3)
-        rt.upload_all(src, data)
-        from nvshmem_amd import _lib
-        fn = _lib.typed_coll(rt.lib, "nvshmemx_float_sum_reduce_on_stream", True)
+    # -- put / get ---------------------------------------------------------------------------
+    def rma_prepare(self, g, item):
+        g.rt.fill(g.dst, 0, item.config["bytes_per_pe"])
 
-        def step():
-            rc = fn(N.TEAM_WORLD, dst, src, n, None)
-            if rc != 0:
-                raise RuntimeError("reduce failed: %d %s" % (rc, rt.last_error()))
-        wall, ev = _time_steps(step, steps, warmup, hip)
-        sample = 1 << 22
-        want = O.reduce("f32", "sum", data[:, :sample])
-        got = rt.download(dst, 5, (sample,), np.float32)
-        ok = bool(np.array_equal(got.view(np.uint32), want.view(np.uint32)))
-        rt.free(src); rt.free(dst)
-    alg = 2 * npes * n * 4
-    cores = min(16, O.lib().oracle_get_threads())
-    O.lib().oracle_set_threads(cores)
-    cs = 1 << 24
-    host = np.ascontiguousarray(data[:, :cs])
-    best, passes = _cpu_time(lambda: O.reduce("f32", "sum", host), cpu_budget, 40)
-    # the CPU oracle produces one PE's result; the algorithmic formula counts npes destinations, so
-    # the CPU figure is quoted on what it actually moves: npes reads + 1 write per element
-    cpu = {"value": round((npes + 1) * cs * 4 / best / 1e9, 2), "unit": "GB/s", "cores": cores,
-           "kind": "port",
-           "sample": "oracle_reduce f32 sum, 8 PEs x 2^24 elements (8 reads + 1 write per element), "
-                     "best of %d passes" % passes}
-    return {
-        "name": "sum_reduce", "dtype": "f32", "verified": ok, "algorithmic_bytes": alg,
-        "wall_ms": wall, "kernel_ms": ev,
-        "config": {"workload": "sum_reduce: nvshmemx_float_sum_reduce_on_stream, 8 logical PEs x 2^26 "
-                               "fp32 (256 MiB per PE), fixed PE order", "npes": npes, "nreduce": n},
-        "kernel": "reduce_vector_kernel<float, sum, 8>",
-        "cpu_baseline": cpu,
-    }
+    def rma_verify(self, g, item):
+        np, size, npes = self.np, item.config["bytes_per_pe"], g.npes
+        shift = 1 if item.config["is_get"] else -1
+        return all(bool(np.array_equal(g.rt.download(g.dst, pe, (size,), np.uint8), g.data[(pe + shift) % npes][:size]))
+                   for pe in range(npes))
 
+    def rma_baseline(self, g, item):
+        np, sample = self.np, 32 << 20
+        if not hasattr(g, "_host"):
+            g._host = (np.ascontiguousarray(g.data[:, :sample]), np.zeros((g.npes, sample), np.uint8))
+        src, dst = g._host
+        fn = (lambda: self.O.ring_get(src)) if item.config["is_get"] else (lambda: self.O.ring_put(src, dst))
+        return self.baseline(fn, 2 * g.npes * sample,
+                             "oracle_ring_%s (memcpy), 8 PEs x 32 MiB" % ("get" if item.config["is_get"] else "put"))
 
-def bench_alltoall(N, O, hip, np, steps, warmup, cpu_budget, n=1 << 22, name="alltoall"):
-    npes = 16
-    with _runtime(N, npes, 2 * n * 4 + (16 << 20)) as rt:
-        src = rt.malloc(n * 4); dst = rt.malloc(n * 4)
-        data = O.fill_all("u64", npes, n // 2, 6).view(np.uint8).reshape(npes, -1)
-        rt.upload_all(src, data)
-        from nvshmem_amd import _lib
-        fn = _lib.typed_coll(rt.lib, "nvshmemx_float_alltoall_on_stream", True)
+    # -- allreduce ---------------------------------------------------------------------------
+    def reduce_prepare(self, g, item):
+        item.prepare()
 
-        def step():
-            rc = fn(N.TEAM_WORLD, dst, src, n // npes, None)
-            if rc != 0:
-                raise RuntimeError("alltoall failed: %d %s" % (rc, rt.last_error()))
-        wall, ev = _time_steps(step, steps, warmup, hip)
-        got = rt.download_all(dst, (n * 4,), np.uint8)
-        want = O.alltoall(data)
-        ok = bool(np.array_equal(got, want))
-        rt.free(src); rt.free(dst)
-    alg = 2 * npes * n * 4
-    cores = min(16, O.lib().oracle_get_threads())
-    O.lib().oracle_set_threads(cores)
-    best, passes = _cpu_time(lambda: O.alltoall(data), cpu_budget, 40)
-    cpu = {"value": round(alg / best / 1e9, 2), "unit": "GB/s", "cores": cores, "kind": "port",
-           "sample": "oracle_alltoall, 16 PEs x %d fp32 (the full workload), best of %d passes" % (n, passes)}
-    return {
-        "name": name, "dtype": "u8", "verified": ok, "algorithmic_bytes": alg,
-        "wall_ms": wall, "kernel_ms": ev,
-        "config": {"workload": "alltoall: nvshmemx_float_alltoall_on_stream, 16 logical PEs x %d fp32, "
-                               "block %d elements per destination" % (n, n // npes),
-                   "npes": npes, "nelems": n // npes,
-                   "note": ("the 256 MiB source fits the Infinity Cache, so repeated steps read it from "
-                            "there and the algorithmic rate can exceed the HBM peak"
-                            if npes * n * 4 <= (256 << 20) else
-                            "source larger than the Infinity Cache: HBM-bound")},
-        "kernel": "segment_copy_kernel<alltoall>",
-        "cpu_baseline": cpu,
-    }
+    def reduce_verify(self, g, item):
+        np, O = self.np, self.O
+        data = g.data["array"]
+        n, es = g.n, item.elem_bytes
+        ok = True
+        for lo, cnt in ((0, min(n, 1 << 22)), (max(0, n - (1 << 16)), min(n, 1 << 16))):
+            want = O.reduce(item.oracle_dtype, item.op, data[:, lo:lo + cnt])
+            for pe in (0, 5, g.npes - 1):
+                got = g.rt.download(g.dst, pe, (cnt,), want.dtype, lo * es)
+                ok = ok and bool(np.array_equal(got.view(np.uint8), want.view(np.uint8)))
+        return ok
 
+    def reduce_baseline(self, g, item):
+        np = self.np
+        cs = min(g.n, 1 << 22)
+        host = np.ascontiguousarray(g.data["array"][:, :cs])
+        # the oracle produces one PE's result, so its figure counts what it moves: npes reads + 1 write
+        return self.baseline(lambda: self.O.reduce(item.oracle_dtype, item.op, host), (g.npes + 1) * cs * item.elem_bytes,
+                             "oracle_reduce %s %s, %d PEs x %d elements (%d reads + 1 write per element)"
+                             % (item.oracle_dtype, item.op, g.npes, cs, g.npes))
 
-def bench_reducescatter(N, O, hip, np, steps, warmup, cpu_budget):
-    npes, n = 8, 1 << 23
-    with _runtime(N, npes, 9 * n * 4 + (64 << 20)) as rt:
-        src = rt.malloc(npes * n * 4); dst = rt.malloc(n * 4)
-        data = O.fill_all("f32", npes, npes * n, 9)
-        rt.upload_all(src, data)
-        from nvshmem_amd import _lib
-        fn = _lib.typed_coll(rt.lib, "nvshmemx_float_sum_reducescatter_on_stream", True)
+    # -- fcollect / alltoall -------------------------------------------------------------------
+    def collect_prepare(self, g, item):
+        pass
 
-        def step():
-            rc = fn(N.TEAM_WORLD, dst, src, n, None)
-            if rc != 0:
-                raise RuntimeError("reducescatter failed: %d %s" % (rc, rt.last_error()))
-        wall, ev = _time_steps(step, steps, warmup, hip)
-        sample = 1 << 20
-        pe = 5
-        want = O.reducescatter("f32", "sum", np.ascontiguousarray(
-            data.reshape(npes, npes, n)[:, :, :sample].reshape(npes, npes * sample)))[pe]
-        got = rt.download(dst, pe, (sample,), np.float32)
-        ok = bool(np.array_equal(got.view(np.uint32), want.view(np.uint32)))
-        rt.free(src); rt.free(dst)
-    alg = (npes + 1) * npes * n * 4
-    cores = min(16, O.lib().oracle_get_threads())
-    O.lib().oracle_set_threads(cores)
-    cs = 1 << 20
-    host = np.ascontiguousarray(data[:, :npes * cs])
-    best, passes = _cpu_time(lambda: O.reducescatter("f32", "sum", host), cpu_budget, 20)
-    cpu = {"value": round((npes + 1) * npes * cs * 4 / best / 1e9, 2), "unit": "GB/s", "cores": cores,
-           "kind": "port", "sample": "oracle_reducescatter f32 sum, 8 PEs x 8 x 2^20 elements, best of %d "
-                                     "passes" % passes}
-    return {
-        "name": "reducescatter", "dtype": "f32", "verified": ok, "algorithmic_bytes": alg,
-        "wall_ms": wall, "kernel_ms": ev,
-        "config": {"workload": "reducescatter: nvshmemx_float_sum_reducescatter_on_stream, 8 logical PEs, "
-                               "source 8 x 2^23 fp32 (256 MiB) per PE, result 2^23 fp32 per PE",
-                   "npes": npes, "nreduce": n},
-        "kernel": "reducescatter_gather_kernel<float, sum, 8>",
-        "cpu_baseline": cpu,
-    }
+    def collect_verify(self, g, item):
+        np, npes = self.np, g.npes
+        nbytes = g.n * g.es
+        if item.what == "alltoall":
+            want = self.O.alltoall(g.data)
+            return all(bool(np.array_equal(g.rt.download(g.a2a_dst, pe, (nbytes,), np.uint8), want[pe]))
+                       for pe in range(npes))
+        want = g.data.reshape(-1)                      # every PE: the sources in PE order
+        return all(bool(np.array_equal(g.rt.download(g.fc_dst, pe, (npes * nbytes,), np.uint8), want))
+                   for pe in (0, 9, 15))
 
+    def collect_baseline(self, g, item):
+        np, npes = self.np, g.npes
+        seg = (1 << 20) if item.what == "alltoall" else (1 << 18)     # bytes per (source, destination) / per source
+        if item.what == "alltoall":
+            host = np.ascontiguousarray(g.data[:, :npes * seg])
+            return self.baseline(lambda: self.O.alltoall(host), 2 * npes * npes * seg,
+                                 "oracle_alltoall, 16 PEs x 16 MiB")
+        host = np.ascontiguousarray(g.data[:, :seg * 16])
+        return self.baseline(lambda: self.O.fcollect(host), (npes + 1) * npes * seg * 16,
+                             "oracle_fcollect, 16 PEs x 4 MiB")
 
-def bench_broadcast(N, O, hip, np, steps, warmup, cpu_budget):
-    npes, nbytes, root = 8, 1 << 28, 3
-    with _runtime(N, npes, 2 * nbytes + (64 << 20)) as rt:
-        src = rt.malloc(nbytes); dst = rt.malloc(nbytes)
-        rows = [O.fill("bytes", nbytes, 12, pe) if pe == root else np.zeros(1, np.uint8) for pe in range(npes)]
-        rt.upload(src, root, rows[root])
+    # -- reducescatter / broadcast ---------------------------------------------------------------
+    def reducescatter_prepare(self, g, item):
+        pass
 
-        def step():
-            rc = rt.lib.nvshmemx_broadcastmem_on_stream(N.TEAM_WORLD, dst, src, nbytes, root, None)
-            if rc != 0:
-                raise RuntimeError("broadcast failed: %d %s" % (rc, rt.last_error()))
-        wall, ev = _time_steps(step, steps, warmup, hip)
-        ok = all(bool(np.array_equal(rt.download(dst, pe, (nbytes,), np.uint8), rows[root])) for pe in (0, 3, 7))
-        rt.free(src); rt.free(dst)
-    alg = (npes + 1) * nbytes
-    sample = 1 << 26
-    host = np.ascontiguousarray(np.broadcast_to(rows[root][:sample], (npes, sample)))
-    best, passes = _cpu_time(lambda: O.broadcast(host, root), cpu_budget, 20)
-    cpu = {"value": round((npes + 1) * sample / best / 1e9, 2), "unit": "GB/s", "cores": 1, "kind": "port",
-           "sample": "oracle_broadcast (memcpy per PE), 8 PEs x 64 MiB, best of %d passes" % passes}
-    return {
-        "name": "broadcast", "dtype": "u8", "verified": ok, "algorithmic_bytes": alg,
-        "wall_ms": wall, "kernel_ms": ev,
-        "config": {"workload": "broadcast: nvshmemx_broadcastmem_on_stream, 8 logical PEs, 256 MiB from PE 3",
-                   "npes": npes, "bytes": nbytes, "root": root,
-                   "note": "the 256 MiB source fits the Infinity Cache and is re-read from it on repeated "
-                           "steps; a 512 MiB source measures 6.5 TB/s"},
-        "kernel": "segment_copy_kernel<broadcast>",
-        "cpu_baseline": cpu,
-    }
+    def reducescatter_verify(self, g, item):
+        np, npes, n, sample = self.np, g.npes, g.n, 1 << 20
+        want = self.O.reducescatter("f32", "sum", np.ascontiguousarray(
+            g.data.reshape(npes, npes, n)[:, :, :sample].reshape(npes, npes * sample)))
+        return all(bool(np.array_equal(g.rt.download(g.dst, pe, (sample,), np.float32).view(np.uint32),
+                                       want[pe].view(np.uint32))) for pe in (0, 5))
 
+    def reducescatter_baseline(self, g, item):
+        np, npes, cs = self.np, g.npes, 1 << 19
+        host = np.ascontiguousarray(g.data[:, :npes * cs])
+        return self.baseline(lambda: self.O.reducescatter("f32", "sum", host), (npes + 1) * npes * cs * 4,
+                             "oracle_reducescatter f32 sum, 8 PEs x 8 x 2^19 elements")
 
-def bench_fcollect(N, O, hip, np, steps, warmup, cpu_budget):
-    """Config 4, fp32: 16 PEs x 2^22 elements, every PE ends with all 16 contributions."""
-    npes, n = 16, 1 << 22
-    with _runtime(N, npes, 17 * n * 4 + (16 << 20)) as rt:
-        src = rt.malloc(n * 4); dst = rt.malloc(npes * n * 4)
-        data = O.fill_all("u64", npes, n // 2, 6).view(np.uint8).reshape(npes, -1)
-        rt.upload_all(src, data)
-        from nvshmem_amd import _lib
-        fn = _lib.typed_coll(rt.lib, "nvshmemx_float_fcollect_on_stream", True)
+    def broadcast_prepare(self, g, item):
+        pass
 
-        def step():
-            rc = fn(N.TEAM_WORLD, dst, src, n, None)
-            if rc != 0:
-                raise RuntimeError("fcollect failed: %d %s" % (rc, rt.last_error()))
-        wall, ev = _time_steps(step, steps, warmup, hip)
-        want = data.reshape(-1)                       # every PE: the sources in PE order
-        ok = all(bool(np.array_equal(rt.download(dst, pe, (npes * n * 4,), np.uint8), want)) for pe in (0, 9, 15))
-        rt.free(src); rt.free(dst)
-    alg = (npes + 1) * npes * n * 4
-    cores = min(16, O.lib().oracle_get_threads())
-    O.lib().oracle_set_threads(cores)
-    best, passes = _cpu_time(lambda: O.fcollect(data), cpu_budget, 10)
-    cpu = {"value": round(alg / best / 1e9, 2), "unit": "GB/s", "cores": cores, "kind": "port",
-           "sample": "oracle_fcollect, 16 PEs x %d fp32 (the full workload), best of %d passes" % (n, passes)}
-    return {
-        "name": "fcollect", "dtype": "u8", "verified": ok, "algorithmic_bytes": alg,
-        "wall_ms": wall, "kernel_ms": ev,
-        "config": {"workload": "fcollect: nvshmemx_float_fcollect_on_stream, 16 logical PEs x %d fp32" % n,
-                   "npes": npes, "nelems": n,
-                   "note": "the 256 MiB of sources fit the Infinity Cache and are re-read from it on repeated steps"},
-        "kernel": "segment_copy_kernel<fcollect>",
-        "cpu_baseline": cpu,
-    }
+    def broadcast_verify(self, g, item):
+        np = self.np
+        return all(bool(np.array_equal(g.rt.download(g.dst, pe, (g.nbytes,), np.uint8), g.row)) for pe in (0, 3, 7))
 
+    def broadcast_baseline(self, g, item):
+        np, sample = self.np, 32 << 20
+        host = np.ascontiguousarray(np.broadcast_to(g.row[:sample], (g.npes, sample)))
+        return self.baseline(lambda: self.O.broadcast(host, g.root), (g.npes + 1) * sample,
+                             "oracle_broadcast (memcpy per PE), 8 PEs x 32 MiB")
 
-def bench_moe(N, O, hip, np, steps, warmup, cpu_budget):
-    """Config 5: 8 PEs x 8192 tokens x 7168 bf16, top-8 of 256 experts, Zipf(1.1).  Returns the
-    dispatch and the combine as two workloads; a step of each is one full pass over all rows."""
-    npes, T, K, E, row = 8, 8192, 8, 256, 7168 * 2
-    ex = O.moe_routing(npes, T, K, E, 1.1, 8)
-    counts, seg_base, dest_pe, dest_row, recv_rows = O.moe_plan(ex, npes, T, K, E)
-    cap, rows = int(recv_rows.max()), T * K
-    steps, warmup = max(1, steps // 5), max(1, warmup // 5)      # a step moves 8 / 14 GiB
-    with _runtime(N, npes, cap * row + rows * row + T * row + (64 << 20)) as rt:
-        perf = rt.perftest()
-        send = rt.malloc(T * row); recv = rt.malloc(cap * row); out = rt.malloc(rows * row)
-        d_pe = rt.malloc(rows * 4); d_row = rt.malloc(rows * 8)
-        expected = rt.malloc(npes * 8); sig = rt.calloc(npes, 8)
-        rt.upload_all(d_pe, dest_pe); rt.upload_all(d_row, dest_row)
-        epp = E // npes
-        exp_tab = np.stack([[counts[s, d * epp:(d + 1) * epp].sum() for s in range(npes)]
-                            for d in range(npes)]).astype(np.uint64)
-        rt.upload_all(expected, exp_tab)
-        payload = O.fill_all("u64", npes, T * row // 8, 7).view(np.uint8).reshape(npes, T, row)
-        rt.upload_all(send, payload)
+    # -- MoE -----------------------------------------------------------------------------------
+    def moe_prepare(self, g, item):
+        if item.what != "combine":
+            g.rt.fill(g.recv, 0, g.cap * g.row)
 
-        def dispatch():
-            perf.nvshmem_perftest_fill_words(sig, 0, npes, None)
-            rc = perf.nvshmem_perftest_moe_dispatch_pieces(recv, cap, send, d_pe, d_row, expected, sig, T, K, row,
-                                                           1024, 256, None)
-            if rc != 0:
-                raise RuntimeError("moe dispatch failed: %d" % rc)
-
-        def combine():
-            rc = perf.nvshmem_perftest_moe_combine_pieces(out, recv, cap, d_pe, d_row, T, K, row, 2048, 262144, 64,
-                                                          N.SCOPE_WARP, None)
-            if rc != 0:
-                raise RuntimeError("moe combine failed: %d" % rc)
-        d_wall, d_ev = _time_steps(dispatch, steps, warmup, hip)
-        c_wall, c_ev = _time_steps(combine, steps, warmup, hip)
-        # parity on samples: signals count the rows exactly, sampled copies sit where the plan says,
-        # and the round trip returns every sampled row
-        ok = bool(np.array_equal(rt.download_all(sig, (npes,), np.uint64), exp_tab))
-        ok = ok and all(rt.read_timeout(pe)[0] == 0 for pe in range(npes))
+    def moe_verify(self, g, item):
+        np, rt = self.np, g.rt
+        npes, K, row, rows = g.npes, g.K, g.row, g.rows
+        ok = all(rt.read_timeout(pe)[0] == 0 for pe in range(npes))
+        if item.what == "put_signal":
+            sig = rt.download_all(g.sig, (npes * g.SIG_STRIDE,), np.uint64)[:, ::g.SIG_STRIDE]
+            ok = ok and bool(np.array_equal(sig, g.expected))
+        elif item.what == "plain_store":
+            ok = ok and bool(np.array_equal(rt.download_all(g.sig, (npes,), np.uint64), g.expected))
         rng = np.random.default_rng(0)
         for src_pe in range(npes):
-            for r in rng.integers(0, rows, 64):
-                got = rt.download(recv, int(dest_pe[src_pe, r]), (row,), np.uint8, int(dest_row[src_pe, r]) * row)
-                back = rt.download(out, src_pe, (row,), np.uint8, int(r) * row)
-                ok = ok and bool(np.array_equal(got, payload[src_pe, r // K])) and bool(np.array_equal(back, got))
-        for p in (send, recv, out, d_pe, d_row, expected, sig):
-            rt.free(p)
-    moved = npes * rows * row
-    # CPU oracle on a bounded sample: the same shuffle with 1024 tokens per PE
-    Ts = 1024
-    exs = O.moe_routing(npes, Ts, K, E, 1.1, 8)
-    _, _, s_pe, s_row, s_recv = O.moe_plan(exs, npes, Ts, K, E)
-    small = np.ascontiguousarray(payload[:, :Ts])
-    cores = min(16, O.lib().oracle_get_threads())
-    O.lib().oracle_set_threads(cores)
-    held = {}
+            for r in rng.integers(0, rows, 128):
+                got = rt.download(g.recv, int(g.dest_pe[src_pe, r]), (row,), np.uint8, int(g.dest_row[src_pe, r]) * row)
+                ok = ok and bool(np.array_equal(got, g.payload[src_pe, r // K]))
+                if item.what == "combine":
+                    back = rt.download(g.out, src_pe, (row,), np.uint8, int(r) * row)
+                    ok = ok and bool(np.array_equal(back, got))
+        return ok
 
-    def cpu_dispatch():
-        held["recv"] = O.moe_dispatch(small, s_pe, s_row, s_recv, Ts, K)
-    best_d, passes_d = _cpu_time(cpu_dispatch, cpu_budget, 5)
-    best_c, passes_c = _cpu_time(lambda: O.moe_combine(held["recv"], s_pe, s_row, Ts, K, row), cpu_budget, 5)
-    small_moved = npes * Ts * K * row
-    shape = "8 logical PEs x 8192 tokens x 7168 bf16, top-8 of 256 experts, Zipf(1.1)"
-    common = {"npes": npes, "tokens": T, "topk": K, "experts": E, "row_bytes": row}
-    disp = {
-        "name": "moe_dispatch", "dtype": "u8", "verified": ok, "algorithmic_bytes": moved + moved // K,
-        "wall_ms": d_wall, "kernel_ms": d_ev,
-        "config": dict(common, workload="moe_dispatch: 1 KiB work items stored through nvshmem_ptr, ADD signals, "
-                       "signal_wait_until(GE); " + shape,
-                       note="algorithmic bytes = every source row read once and written top-k times "
-                            "(7.875 GiB); the timed step includes clearing the signal words"),
-        "kernel": "moe_dispatch_direct_kernel<1> + moe_dispatch_signal_kernel",
-        "cpu_baseline": {"value": round((small_moved + small_moved // K) / best_d / 1e9, 2), "unit": "GB/s",
-                         "cores": cores, "kind": "port",
-                         "sample": "oracle_moe_dispatch, 1024 tokens per PE, best of %d passes" % passes_d},
-    }
-    comb = {
-        "name": "moe_combine", "dtype": "u8", "verified": ok, "algorithmic_bytes": 2 * moved,
-        "wall_ms": c_wall, "kernel_ms": c_ev,
-        "config": dict(common, workload="moe_combine: nvshmemx_getmem_nbi_warp per 2 KiB of a row; " + shape),
-        "kernel": "moe_combine_kernel<warp, 2048>",
-        "cpu_baseline": {"value": round(2 * small_moved / best_c / 1e9, 2), "unit": "GB/s", "cores": cores,
-                         "kind": "port",
-                         "sample": "oracle_moe_combine, 1024 tokens per PE, best of %d passes" % passes_c},
-    }
-    return disp, comb
+    def moe_baseline(self, g, item):
+        np, O = self.np, self.O
+        npes, K, E, row, Ts = g.npes, g.K, g.E, g.row, 512
+        if not hasattr(g, "_small"):
+            exs = O.moe_routing(npes, Ts, K, E, 1.1, 8)
+            _, _, s_pe, s_row, s_recv = O.moe_plan(exs, npes, Ts, K, E)
+            small = np.ascontiguousarray(g.payload[:, :Ts])
+            g._small = (small, s_pe, s_row, s_recv, O.moe_dispatch(small, s_pe, s_row, s_recv, Ts, K))
+        small, s_pe, s_row, s_recv, held = g._small
+        moved = npes * Ts * K * row
+        if item.what == "combine":
+            return self.baseline(lambda: O.moe_combine(held, s_pe, s_row, Ts, K, row), 2 * moved,
+                                 "oracle_moe_combine, 512 tokens per PE")
+        return self.baseline(lambda: O.moe_dispatch(small, s_pe, s_row, s_recv, Ts, K), moved + moved // K,
+                             "oracle_moe_dispatch, 512 tokens per PE")
 
 
-class _runtime:
-    def __init__(self, N, npes, size):
-        self.N, self.npes, self.size = N, npes, size
-
-    def __enter__(self):
-        self.rt = self.N.Runtime(npes=self.npes, symmetric_size=self.size)
-        return self.rt
-
-    def __exit__(self, *exc):
-        self.rt.finalize()
+def oracle_moe_plan(O, np, npes, T, K, E):
+    ex = O.moe_routing(npes, T, K, E, 1.1, 8)
+    counts, _, dest_pe, dest_row, recv_rows = O.moe_plan(ex, npes, T, K, E)
+    epp = E // npes
+    expected = np.stack([[counts[s, d * epp:(d + 1) * epp].sum() for s in range(npes)]
+                         for d in range(npes)]).astype(np.uint64)
+    return dest_pe, dest_row, expected, recv_rows
 
 
-def _summarise(r):
-    gbs = r["algorithmic_bytes"] / r["wall_ms"] / 1e6
-    kernel_gbs = r["algorithmic_bytes"] / r["kernel_ms"] / 1e6
+def summarise(item, wall, ev, ok, cpu):
+    gbs = item.algorithmic_bytes / wall / 1e6
+    kernel_gbs = item.algorithmic_bytes / ev / 1e6
+    cfg = dict(item.config, workload=item.workload)
+    if "bytes_per_pe" in item.config:
+        cfg["payload_only_GBs"] = round(item.config["npes"] * item.config["bytes_per_pe"] / ev / 1e6, 1)
     return {
         "GBs": round(gbs, 1), "frac_of_hbm_peak": round(gbs / HBM_PEAK_GBS, 4),
-        "ms_per_step": round(r["wall_ms"], 5), "kernel_ms": round(r["kernel_ms"], 5),
-        "kernel_GBs": round(kernel_gbs, 1), "algorithmic_bytes": r["algorithmic_bytes"],
-        "traffic": MEASURED_TRAFFIC_BYTES[r["name"]],
-        "dtype": r["dtype"], "verified": r["verified"], "config": r["config"], "kernel": r["kernel"],
-        "cpu_baseline": r["cpu_baseline"],
+        "ms_per_step": round(wall, 5), "kernel_ms": round(ev, 5), "kernel_GBs": round(kernel_gbs, 1),
+        "kernel_frac_of_hbm_peak": round(kernel_gbs / HBM_PEAK_GBS, 4),
+        "algorithmic_bytes": item.algorithmic_bytes, "traffic": measured_traffic(item.name),
+        "dtype": item.dtype, "verified": ok, "config": cfg, "kernel": item.kernel, "cpu_baseline": cpu,
     }
 
 
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
-    ap.add_argument("--steps", type=int, default=50)
-    ap.add_argument("--warmup", type=int, default=10)
-    ap.add_argument("--cpu-seconds", type=float, default=6.0,
-                    help="CPU oracle timing budget per workload")
+    ap.add_argument("--steps", type=int, default=30)
+    ap.add_argument("--warmup", type=int, default=5)
+    ap.add_argument("--cpu-seconds", type=float, default=1.5, help="CPU oracle timing budget per workload")
+    ap.add_argument("--only", default="", help="comma-separated workload names (the headline always runs)")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this build runs all logical PEs on ONE GPU; --gpus %d is not supported "
@@ -441,51 +268,58 @@ def main():
 
     import numpy as np
     import nvshmem_amd as N          # raises if the HIP libraries are not built
-    from nvshmem_amd import hip
+    from nvshmem_amd import hip, workloads
     import oracle_lib as O           # the checker / CPU baseline only
 
     if hip.device_count() < 1:
         print("bench.py: no GPU visible", file=sys.stderr)
         return 3
 
-    put = bench_put_block(N, O, hip, np, args.steps, args.warmup, args.cpu_seconds)
-    red = bench_sum_reduce(N, O, hip, np, args.steps, args.warmup, args.cpu_seconds)
-    a2a = bench_alltoall(N, O, hip, np, args.steps, args.warmup, args.cpu_seconds)
-    a2a_big = bench_alltoall(N, O, hip, np, args.steps, args.warmup, 1.0, n=1 << 24,
-                             name="alltoall_1GiB")
-    rsc = bench_reducescatter(N, O, hip, np, args.steps, args.warmup, 1.0)
-    bca = bench_broadcast(N, O, hip, np, args.steps, args.warmup, 1.0)
-    fco = bench_fcollect(N, O, hip, np, args.steps, args.warmup, 1.0)
-    moe_d, moe_c = bench_moe(N, O, hip, np, args.steps, args.warmup, 1.0)
+    only = set(x for x in args.only.split(",") if x)
+    if only:
+        only.add(workloads.HEADLINE)
+    check = Checker(O, np, args.cpu_seconds)
+    results = {}
+    groups = workloads.all_groups(oracle_moe_plan(O, np, 8, 8192, 8, 256))
+    for g in groups:
+        if only and not any(n in only for n in g.names()):
+            continue
+        rt = N.Runtime(npes=g.npes, symmetric_size=g.heap_bytes)
+        try:
+            for item in g.setup(rt, O.fill_all):
+                if only and item.name not in only:
+                    continue
+                getattr(check, g.kind + "_prepare")(g, item)
+                steps, warmup = max(1, args.steps // item.scale), max(1, args.warmup // item.scale)
+                wall, ev = time_steps(item.step, steps, warmup, hip)
+                ok = getattr(check, g.kind + "_verify")(g, item)
+                cpu = getattr(check, g.kind + "_baseline")(g, item)
+                results[item.name] = summarise(item, wall, ev, ok, cpu)
+                results[item.name]["steps"] = steps
+        finally:
+            rt.finalize()
 
-    head = put
-    value = head["algorithmic_bytes"] / head["wall_ms"] / 1e6
-    achieved = head["algorithmic_bytes"] / head["kernel_ms"] / 1e6
+    head = results[workloads.HEADLINE]
     line = {
         "metric": METRIC,
-        "value": round(value, 1),
+        "value": head["GBs"],
         "unit": "GB/s",
         "n_gpus": 1,
-        "steps": args.steps,
+        "steps": head["steps"],
         "warmup": args.warmup,
-        "ms_per_step": round(head["wall_ms"], 5),
+        "ms_per_step": head["ms_per_step"],
         "higher_is_better": True,
         "scaling": "weak",
         "vs_baseline": None,
         "dtype": head["dtype"],
         "data": "synthetic",
         "config": head["config"],
-        "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS,
-                     "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBS, 4),
-                     "traffic": MEASURED_TRAFFIC_BYTES[head["name"]], "kernel": head["kernel"]},
+        "roofline": {"bound": "hbm", "achieved": head["kernel_GBs"], "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                     "frac": round(head["kernel_GBs"] / HBM_PEAK_GBS, 4), "traffic": head["traffic"],
+                     "kernel": head["kernel"]},
         "cpu_baseline": head["cpu_baseline"],
-        "verified": bool(put["verified"] and red["verified"] and a2a["verified"] and a2a_big["verified"]
-                         and rsc["verified"] and bca["verified"] and fco["verified"] and moe_d["verified"]),
-        "workloads": {"put_block": _summarise(put), "sum_reduce": _summarise(red),
-                      "alltoall": _summarise(a2a), "alltoall_1GiB": _summarise(a2a_big),
-                      "reducescatter": _summarise(rsc), "broadcast": _summarise(bca),
-                      "fcollect": _summarise(fco), "moe_dispatch": _summarise(moe_d),
-                      "moe_combine": _summarise(moe_c)},
+        "verified": all(r["verified"] for r in results.values()),
+        "workloads": results,
     }
     print(json.dumps(line))
     return 0 if line["verified"] else 1

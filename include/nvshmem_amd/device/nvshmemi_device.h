@@ -157,11 +157,14 @@ typedef nvshmemi_v4u __attribute__((aligned(1))) nvshmemi_v4u_unaligned;
 #define NVSHMEMI_AMD_COPY_UNROLL 4
 #endif
 /* Long copies - a lane owns at least NVSHMEMI_AMD_COPY_DEEP_MIN vectors - run rounds of
- * NVSHMEMI_AMD_COPY_DEEP_UNROLL vectors per lane first (0 switches the deep rounds off).  A thread group
- * that streams a long slice on its own compute unit is bound by the bytes it keeps in flight: 1024
- * threads x 4 vectors are 64 KiB, which at the loaded memory latency is about 33 GB/s. */
+ * NVSHMEMI_AMD_COPY_DEEP_UNROLL vectors per lane first (0 switches them off).  Eight is what fits the
+ * registers the rest of the engine needs anyway.  Sixteen measured 6 % more for 16 blocks of 1024
+ * threads that each stream a 16 MiB slice, but its 28 extra vector registers lower the occupancy of
+ * every kernel that inlines the engine, and kernels of one-wavefront blocks that move 1-2 KiB each -
+ * the fastest shapes on this GPU - lost 9-13 %.  (A block that streams a long slice alone on its
+ * compute unit moves about 31 GB/s of payload whatever the depth: see the counter profiles.) */
 #ifndef NVSHMEMI_AMD_COPY_DEEP_UNROLL
-#define NVSHMEMI_AMD_COPY_DEEP_UNROLL 16
+#define NVSHMEMI_AMD_COPY_DEEP_UNROLL 8
 #endif
 #ifndef NVSHMEMI_AMD_COPY_DEEP_MIN
 #define NVSHMEMI_AMD_COPY_DEEP_MIN 32
@@ -173,7 +176,7 @@ typedef nvshmemi_v4u __attribute__((aligned(1))) nvshmemi_v4u_unaligned;
  * too (measured +5 % on a 256 MiB put).  NVSHMEMI_AMD_COPY_NT overrides the choice for a translation
  * unit: bit 0 set = always non-temporal loads, 0 = never; bit 1 = non-temporal stores. */
 #ifndef NVSHMEMI_AMD_COPY_NT_BYTES
-#define NVSHMEMI_AMD_COPY_NT_BYTES (1u << 20)
+#define NVSHMEMI_AMD_COPY_NT_BYTES (32u << 20)
 #endif
 
 /* A 16-byte store at agent scope (written through the L2).  The compiler has no such store, so it is

@@ -42,6 +42,10 @@ int nvshmem_perftest_ring_rma(void *dest, const void *src, size_t bytes, int blo
  * `bytes` each. */
 int nvshmem_perftest_plain_copy(void *dst, const void *src, size_t bytes, void *stream);
 
+/* One launch of an empty kernel named profile_marker_kernel: a boundary that a script reading a profiler's
+ * kernel trace can recognise (nvshmem_amd/profile_workloads.py brackets every workload with two). */
+int nvshmem_perftest_profile_marker(void *stream);
+
 /* PE p writes value_base + p into word [p] of PE (p+1)%npes's `words` with nvshmem_uint64_p, then
  * (after a barrier) reads word [q] of every PE q's `words`... with nvshmem_uint64_g into
  * out[q] of its own `out`.  words and out hold npes uint64 each. */

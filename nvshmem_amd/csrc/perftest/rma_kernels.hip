@@ -250,6 +250,9 @@ __global__ void ring_reduce_kernel(int32_t *dst, const int32_t *src, size_t nred
     if (threadIdx.x == 0) *(uint64_t *)nvshmem_ptr(signal, me) = 0;  // ready for the next run
 }
 
+// Boundary between workloads in a profiler trace: does nothing, has a name of its own.
+__global__ void profile_marker_kernel() {}
+
 // Calibration kernel for hardware counters: a plain copy of a known size that uses nothing of the
 // NVSHMEM API (one 16-byte vector per thread).
 __global__ void plain_copy_kernel(nvshmemi_v4u *dst, const nvshmemi_v4u *src, size_t nvec) {
@@ -386,6 +389,11 @@ int nvshmem_perftest_plain_copy(void *dst, const void *src, size_t bytes, void *
     hipLaunchKernelGGL(plain_copy_kernel, dim3((unsigned)((nvec + 255) / 256)), dim3(256), 0,
                        (hipStream_t)stream, (nvshmemi_v4u *)dst, (const nvshmemi_v4u *)src, nvec);
     return perftest::launch_status("plain_copy");
+}
+
+int nvshmem_perftest_profile_marker(void *stream) {
+    hipLaunchKernelGGL(profile_marker_kernel, dim3(1), dim3(1), 0, (hipStream_t)stream);
+    return perftest::launch_status("profile_marker");
 }
 
 int nvshmem_perftest_p_g(uint64_t *words, uint64_t *out, uint64_t value_base, void *stream) {

@@ -1,25 +1,44 @@
-"""Turns rocprofv3 result databases (rocpd / sqlite) into the short text summary kept under
-profiles/.
+"""Turns rocprofv3 result databases (rocpd / sqlite) of nvshmem_amd/profile_workloads.py runs into the
+short text summaries kept under profiles/, one per workload.
 
-    python3 nvshmem_amd/profile_summary.py --stats <dir> [--fetch <dir>] [--write <dir>]
+    python3 nvshmem_amd/profile_summary.py --manifest <json> --stats <dir> [--pmc <dir> ...]
+                                           [--profiles-dir profiles] [--only name,name]
 
-Each <dir> is a rocprofv3 `-d` output directory.  Per kernel: calls and average duration from the
-kernel trace; average FETCH_SIZE / WRITE_SIZE (KiB per dispatch) from the counter runs, and the
-same scaled by what the counter reads for the plain copy calibration kernel, whose traffic is known
-(1 GiB read, 1 GiB written).
+Each <dir> is a rocprofv3 `-d` output directory: --stats from a `--kernel-trace --stats` run, every
+--pmc from one `--pmc <counters>` run.  profile_workloads.py brackets each workload with two launches
+of profile_marker_kernel and records the order in the manifest, so dispatches are assigned to workloads
+by counting markers.  Per workload and kernel: calls and average / min / max duration; per counter the
+average per dispatch; FETCH_SIZE / WRITE_SIZE (KiB per dispatch) also scaled by what the same counter
+reads for the calibration workload, a plain copy kernel of known traffic (1 GiB read, 1 GiB written).
 """
 import argparse
 import glob
+import json
 import os
+import re
 import sqlite3
 
-CALIBRATION = "plain_copy_kernel"
+MARKER = "profile_marker_kernel"
+CALIBRATION = "calibration"
 CALIBRATION_KIB = float(1 << 20)   # 1 GiB in KiB, read and written
+HBM_PEAK_GBS = 8000.0
+
+
+COMMANDS = """Commands (on the GPU box, from the repository root; every file they run is committed):
+  export OUT=<a scratch directory>; cd /tmp; export TMPDIR=/tmp
+  rocprofv3 --kernel-trace --stats -d $OUT/stats -- python3 $REPO/nvshmem_amd/profile_workloads.py --iters 4 --manifest $OUT/manifest.json
+  rocprofv3 --pmc FETCH_SIZE -d $OUT/p1 -- python3 $REPO/nvshmem_amd/profile_workloads.py --iters 4 --manifest $OUT/manifest.json
+  rocprofv3 --pmc WRITE_SIZE -d $OUT/p2 -- python3 $REPO/nvshmem_amd/profile_workloads.py --iters 4 --manifest $OUT/manifest.json
+  rocprofv3 --pmc TCP_TCC_READ_REQ_sum TCP_TCC_READ_REQ_LATENCY_sum TCP_PENDING_STALL_CYCLES_sum TCP_TCR_TCP_STALL_CYCLES_sum -d $OUT/p3 -- (the same)
+  rocprofv3 --pmc SQ_WAVES SQ_BUSY_CYCLES SQ_WAIT_INST_ANY SQ_INSTS_VMEM_RD SQ_INSTS_VMEM_WR SQ_INST_LEVEL_VMEM GRBM_GUI_ACTIVE -d $OUT/p4 -- (the same)
+  rocprofv3 --pmc TCC_HIT_sum TCC_MISS_sum TCC_TAG_STALL_sum TCC_EA0_WRREQ_STALL_sum -d $OUT/p5 -- (the same)
+  cd $REPO; python3 nvshmem_amd/profile_summary.py --manifest $OUT/manifest.json --stats $OUT/stats --pmc $OUT/p1 ... --pmc $OUT/p5 --profiles-dir profiles
+(a summary lists the counters of the passes that were run for it.)  Hardware: one MI355X (gfx950), ROCm 7.2.
+Durations are per dispatch from the kernel trace."""
 
 
 def _db(directory):
-    hits = sorted(glob.glob(os.path.join(directory, "**", "*_results.db"), recursive=True),
-                  key=os.path.getmtime)
+    hits = sorted(glob.glob(os.path.join(directory, "**", "*_results.db"), recursive=True), key=os.path.getmtime)
     if not hits:
         raise SystemExit("no *_results.db under %s" % directory)
     return sqlite3.connect(hits[-1])
@@ -31,141 +50,150 @@ def _short(name):
     return name.split("(")[0]
 
 
-def kernel_stats(directory):
-    cur = _db(directory).cursor()
-    rows = cur.execute("select name, count(*), avg(duration), min(duration), max(duration) "
-                       "from kernels group by name order by sum(duration) desc").fetchall()
-    return [(_short(n), c, a / 1e3, lo / 1e3, hi / 1e3) for n, c, a, lo, hi in rows]
-
-
-def counter_avg(directory, counter):
-    cur = _db(directory).cursor()
-    rows = cur.execute("select kernel_name, avg(value), count(*) from counters_collection "
-                       "where counter_name = ? group by kernel_name", (counter,)).fetchall()
-    return {_short(n): (v, c) for n, v, c in rows}
-
-
-# workloads of nvshmem_amd/profile_workloads.py:
-# leading part of the kernel name as the trace prints it -> (file name, description, algorithmic bytes)
-WORKLOADS = {
-    "ring_rma_kernel<2, false>": (
-        "ring_rma_kernel_put_block_8pe_256MiB.txt",
-        "put_block: nvshmemx_putmem_block ring, 8 logical PEs x 256 MiB, 262144 blocks x 64 threads per PE (1 KiB per block).\n"
-        "Algorithmic bytes per launch: 8 x 256 MiB read + 8 x 256 MiB written = 4 GiB.", 4 << 30),
-    "reduce_vector_kernel<float, 5, 8, true,": (
-        "reduce_vector_kernel_float_sum_8pe_64Mi.txt",
-        "sum_reduce: nvshmemx_float_sum_reduce_on_stream, 8 logical PEs x 2^26 fp32.\n"
-        "Algorithmic bytes per launch: 8 sources read once + 8 destinations written once = 4 GiB.", 4 << 30),
-    "segment_copy_kernel<1, 1, false>": (
-        "segment_copy_kernel_alltoall_16pe_4Mi_fp32.txt",
-        "alltoall: nvshmemx_float_alltoall_on_stream, 16 logical PEs x 2^22 fp32 (block 2^18 elements).\n"
-        "Algorithmic bytes per launch: 256 MiB read + 256 MiB written = 512 MiB.  The 256 MiB source fits the\n"
-        "Infinity Cache and the profiled loop re-sends it; FETCH_SIZE counts between L2 and the fabric and\n"
-        "cannot tell a cache hit from an HBM read, but a rate above the HBM peak shows that part of the\n"
-        "reads are served by the cache.", 512 << 20),
-    "segment_copy_kernel<0, 1, false>": (
-        "segment_copy_kernel_fcollect_16pe_4Mi_fp32.txt",
-        "fcollect: nvshmemx_float_fcollect_on_stream, 16 logical PEs x 2^22 fp32.\n"
-        "Algorithmic bytes per launch: 256 MiB read + 16 x 256 MiB written = 4.25 GiB.", (17 * 256) << 20),
-    "reducescatter_gather_kernel<float, 5, 8, true>": (
-        "reducescatter_gather_kernel_float_sum_8pe_8Mi.txt",
-        "reducescatter: nvshmemx_float_sum_reducescatter_on_stream, 8 logical PEs, source 8 x 2^23 fp32\n"
-        "(256 MiB) per PE, result 2^23 fp32 (32 MiB) per PE.\n"
-        "Algorithmic bytes per launch: 8 sources of 256 MiB read once + 8 results of 32 MiB written = 2.25 GiB.",
-        (9 * 256) << 20),
-    "segment_copy_kernel<2, 1, false>": (
-        "segment_copy_kernel_broadcast_8pe_256MiB.txt",
-        "broadcast: nvshmemx_broadcastmem_on_stream, 8 logical PEs, 256 MiB from PE 3.\n"
-        "Algorithmic bytes per launch: 256 MiB read + 8 x 256 MiB written = 2.25 GiB.", (9 * 256) << 20),
-    "moe_dispatch_direct_kernel<1>": (
-        "moe_dispatch_direct_kernel_8pe_8192tok_top8.txt",
-        "MoE dispatch (config 5): 8 logical PEs x 8192 tokens x 7168 bf16, top-8 of 256 experts, Zipf(1.1);\n"
-        "1 KiB work items, at most four copies per wavefront: two neighbouring blocks share a piece.  They run on\n"
-        "different XCDs, so both fetch it through the fabric (FETCH_SIZE counts it twice); the second fetch is\n"
-        "served by the Infinity Cache, not by HBM.  The signalling kernel that follows\n"
-        "(moe_dispatch_signal_kernel) is not part of this figure.\n"
-        "Algorithmic bytes per launch: every row read once (896 MiB) + written 8 times (7 GiB) = 7.875 GiB.",
-        (896 + 7168) << 20),
-    "moe_combine_kernel<true, 2048>": (
-        "moe_combine_kernel_8pe_8192tok_top8.txt",
-        "MoE combine (config 5): every one of the 8 x 65536 row copies fetched back with nvshmemx_getmem_nbi_warp,\n"
-        "2 KiB per single-wavefront block.\n"
-        "Algorithmic bytes per launch: 7 GiB read + 7 GiB written = 14 GiB.", 14 << 30),
-    "plain_copy_kernel": (
-        "plain_copy_kernel_calibration_1GiB.txt",
-        "Counter calibration: plain one-vector-per-thread copy, 1 GiB read + 1 GiB written.", 2 << 30),
-}
-
-COMMANDS = """Commands (from the repository root on the GPU box; every file they run is committed):
-  cd /tmp && export TMPDIR=/tmp OUT=<a scratch directory>
-  rocprofv3 --kernel-trace --stats -d $OUT/prof_stats -- python3 $REPO/nvshmem_amd/profile_workloads.py
-  rocprofv3 --pmc FETCH_SIZE -d $OUT/prof_fetch -- python3 $REPO/nvshmem_amd/profile_workloads.py --iters 5
-  rocprofv3 --pmc WRITE_SIZE -d $OUT/prof_write -- python3 $REPO/nvshmem_amd/profile_workloads.py --iters 5
-  python3 nvshmem_amd/profile_summary.py --stats $OUT/prof_stats --fetch $OUT/prof_fetch \\
-          --write $OUT/prof_write --profiles-dir profiles
-Hardware: one MI355X (gfx950), ROCm 7.2.  Durations are per dispatch from the kernel trace."""
-
-
-def write_profiles(directory, stats, fetch, write, fscale, wscale):
-    os.makedirs(directory, exist_ok=True)
-    def find(table, prefix):
-        hits = [k for k in table if k.startswith(prefix)]
-        return hits[0] if len(hits) == 1 else None
-
-    by_name = {s[0]: s for s in stats}
-    for prefix, (fname, desc, alg) in WORKLOADS.items():
-        kernel = find(by_name, prefix)
-        if kernel is None:
+def _windows(rows, manifest):
+    """rows: (start, kernel name, payload...) of every dispatch -> {workload: [rows between its markers]}."""
+    rows = sorted(rows, key=lambda r: r[0])
+    out, index, inside = {}, -1, False
+    for r in rows:
+        if MARKER in r[1]:
+            if not inside:
+                index += 1
+            inside = not inside
             continue
-        name, calls, avg, lo, hi = by_name[kernel]
-        lines = [desc, "", COMMANDS, "",
-                 "%-46s %6s %12s %12s %12s" % ("kernel", "calls", "avg us", "min us", "max us"),
-                 "%-46s %6d %12.2f %12.2f %12.2f" % (name[:46], calls, avg, lo, hi), "",
-                 "full kernel name: " + name, ""]
-        if fscale and wscale and kernel in fetch and kernel in write:
-            f, w = fetch[kernel][0], write[kernel][0]
-            lines += ["counters (KiB per dispatch): FETCH_SIZE %.1f  WRITE_SIZE %.1f" % (f, w),
-                      "scale factors from plain_copy_kernel (1 GiB read + 1 GiB written): "
-                      "FETCH_SIZE x%.4f, WRITE_SIZE x%.4f" % (fscale, wscale),
-                      "HBM traffic per dispatch (scaled): read %.1f MiB + written %.1f MiB = %.1f MiB; "
-                      "algorithmic bytes %.1f MiB" % (f * fscale / 1024, w * wscale / 1024,
-                                                      (f * fscale + w * wscale) / 1024, alg / 2**20), ""]
-        lines.append("achieved = algorithmic bytes / average duration = %.0f GB/s = %.1f %% of the "
-                     "8000 GB/s HBM peak" % (alg / avg / 1e3, alg / avg / 1e3 / 80.0))
-        with open(os.path.join(directory, fname), "w") as fh:
-            fh.write("\n".join(lines) + "\n")
+        if inside and 0 <= index < len(manifest):
+            out.setdefault(manifest[index]["name"], []).append(r)
+    return out
+
+
+def kernel_windows(directory, manifest):
+    cur = _db(directory).cursor()
+    rows = cur.execute("select start, name, duration, grid_x, grid_y, grid_z, workgroup_x, vgpr_count from kernels").fetchall()
+    return _windows([(s, _short(n), d, gx, gy, gz, wx, v) for s, n, d, gx, gy, gz, wx, v in rows], manifest)
+
+
+def counter_windows(directory, manifest):
+    cur = _db(directory).cursor()
+    rows = cur.execute("select start, kernel_name, counter_name, value, dispatch_id from counters_collection").fetchall()
+    # one row per (dispatch, counter); markers must be counted once per dispatch
+    seen, flat = set(), []
+    for s, n, c, v, d in rows:
+        if MARKER in n:
+            if d in seen:
+                continue
+            seen.add(d)
+        flat.append((s, _short(n), c, v))
+    return _windows(flat, manifest)
+
+
+def stats_of(rows):
+    """[(start, kernel, duration, grid...)] -> {kernel: (calls, avg us, min us, max us, launch shape, vgprs)}"""
+    out = {}
+    for _, k, d, gx, gy, gz, wx, v in rows:
+        out.setdefault(k, []).append((d, (gx, gy, gz, wx), v))
+    return {k: (len(v), sum(x[0] for x in v) / len(v) / 1e3, min(x[0] for x in v) / 1e3, max(x[0] for x in v) / 1e3,
+                v[0][1], v[0][2]) for k, v in out.items()}
+
+
+def counters_of(rows):
+    """[(start, kernel, counter, value)] -> {kernel: {counter: average per dispatch}}"""
+    acc = {}
+    for _, k, c, v in rows:
+        acc.setdefault(k, {}).setdefault(c, []).append(v)
+    return {k: {c: sum(v) / len(v) for c, v in cs.items()} for k, cs in acc.items()}
 
 
 def main():
     ap = argparse.ArgumentParser()
+    ap.add_argument("--manifest", required=True)
     ap.add_argument("--stats", required=True)
-    ap.add_argument("--fetch")
-    ap.add_argument("--write")
-    ap.add_argument("--profiles-dir", help="also write one summary file per workload there")
+    ap.add_argument("--pmc", action="append", default=[])
+    ap.add_argument("--profiles-dir")
+    ap.add_argument("--only", default="")
     args = ap.parse_args()
-    stats = kernel_stats(args.stats)
-    fetch = counter_avg(args.fetch, "FETCH_SIZE") if args.fetch else {}
-    write = counter_avg(args.write, "WRITE_SIZE") if args.write else {}
-    fscale = CALIBRATION_KIB / fetch[CALIBRATION][0] if CALIBRATION in fetch else None
-    wscale = CALIBRATION_KIB / write[CALIBRATION][0] if CALIBRATION in write else None
-    print("%-46s %6s %12s %12s %12s" % ("kernel", "calls", "avg us", "min us", "max us"))
-    for name, calls, avg, lo, hi in stats:
-        print("%-46s %6d %12.2f %12.2f %12.2f" % (name[:46], calls, avg, lo, hi))
-    if fetch or write:
-        print()
-        print("counter scale factors from %s (known 1 GiB read + 1 GiB written): FETCH_SIZE x%s, "
-              "WRITE_SIZE x%s" % (CALIBRATION, "%.4f" % fscale if fscale else "n/a",
-                                  "%.4f" % wscale if wscale else "n/a"))
-        print("%-46s %14s %14s %14s %14s" % ("kernel", "FETCH KiB", "WRITE KiB", "read MiB (scaled)",
-                                             "write MiB (scaled)"))
-        for name in sorted(set(fetch) | set(write)):
-            f = fetch.get(name, (float("nan"), 0))[0]
-            w = write.get(name, (float("nan"), 0))[0]
-            fs = f * fscale / 1024 if fscale else float("nan")
-            ws = w * wscale / 1024 if wscale else float("nan")
-            print("%-46s %14.1f %14.1f %14.1f %14.1f" % (name[:46], f, w, fs, ws))
-    if args.profiles_dir:
-        write_profiles(args.profiles_dir, stats, fetch, write, fscale, wscale)
+    manifest = json.load(open(args.manifest))
+    only = set(x for x in args.only.split(",") if x)
+    commands = COMMANDS
+    kwin = kernel_windows(args.stats, manifest)
+    cwins = [counter_windows(d, manifest) for d in args.pmc]
+    # calibration factors
+    scale = {}
+    for cw in cwins:
+        cal = counters_of(cw.get(CALIBRATION, []))
+        for k, cs in cal.items():
+            for c in ("FETCH_SIZE", "WRITE_SIZE"):
+                if c in cs and cs[c] > 0:
+                    scale[c] = CALIBRATION_KIB / cs[c]
+    for entry in manifest:
+        name = entry["name"]
+        if only and name not in only:
+            continue
+        st = stats_of(kwin.get(name, []))
+        if not st:
+            continue
+        dominant = max(st, key=lambda k: st[k][0] * st[k][1])
+        counters = {}
+        for cw in cwins:
+            for k, cs in counters_of(cw.get(name, [])).items():
+                counters.setdefault(k, {}).update(cs)
+        alg = entry.get("algorithmic_bytes", 2 << 30)
+        lines = [entry.get("workload", "Counter calibration: plain one-vector-per-thread copy, 1 GiB read + 1 GiB written."),
+                 "Algorithmic bytes per step: %d (%.1f MiB)." % (alg, alg / 2**20), ""]
+        if commands:
+            lines += [commands, ""]
+        lines += ["%-58s %6s %11s %11s %11s  %s" % ("kernel", "calls", "avg us", "min us", "max us", "grid (threads) / block, VGPRs")]
+        for k in sorted(st, key=lambda k: -st[k][0] * st[k][1]):
+            calls, avg, lo, hi, shape, vg = st[k]
+            lines.append("%-58s %6d %11.2f %11.2f %11.2f  %dx%dx%d / %d, %s" % (k[:58], calls, avg, lo, hi, shape[0], shape[1],
+                                                                            shape[2], shape[3], vg))
+        lines += ["", "dominant kernel: " + dominant]
+        calls, avg = st[dominant][0], st[dominant][1]
+        step_us = sum(st[k][0] * st[k][1] for k in st) / max(1, entry["launches"])
+        lines.append("kernel time per step (all kernels of the step): %.2f us; dominant kernel alone: %.2f us per launch"
+                     % (step_us, avg))
+        lines.append("achieved = algorithmic bytes / dominant kernel's average duration = %.0f GB/s = %.1f %% of the %.0f GB/s "
+                     "HBM peak" % (alg / avg / 1e3, alg / avg / 1e3 / HBM_PEAK_GBS * 100, HBM_PEAK_GBS))
+        cs = counters.get(dominant, {})
+        if cs:
+            lines += ["", "counters of the dominant kernel (average per dispatch):"]
+            for c in sorted(cs):
+                lines.append("  %-40s %18.1f" % (c, cs[c]))
+            if "TCP_TCC_READ_REQ_LATENCY_sum" in cs and cs.get("TCP_TCC_READ_REQ_sum"):
+                lines.append("  -> average L1-to-L2 read latency: %.0f cycles per request"
+                             % (cs["TCP_TCC_READ_REQ_LATENCY_sum"] / cs["TCP_TCC_READ_REQ_sum"]))
+            if "TCP_TCC_WRITE_REQ_LATENCY_sum" in cs and cs.get("TCP_TCC_WRITE_REQ_sum"):
+                lines.append("  -> average L1-to-L2 write latency: %.0f cycles per request"
+                             % (cs["TCP_TCC_WRITE_REQ_LATENCY_sum"] / cs["TCP_TCC_WRITE_REQ_sum"]))
+            if ("TCP_TCC_READ_REQ_LATENCY_sum" in cs and cs.get("TCP_TCC_READ_REQ_sum") and cs.get("GRBM_GUI_ACTIVE")):
+                # Little's law per compute unit: requests in flight = requests x latency / elapsed cycles;
+                # GRBM_GUI_ACTIVE sums the busy cycles of the 8 XCDs
+                shape = st[dominant][4]
+                groups = shape[0] * shape[1] * shape[2] // max(1, shape[3])
+                cus = min(groups, 256)
+                cycles = cs["GRBM_GUI_ACTIVE"] / 8.0
+                lines.append("  -> %d work-groups on at most %d compute units, %.0f cycles: %.1f L1 read requests (128 bytes) "
+                             "in flight per compute unit on average"
+                             % (groups, cus, cycles, cs["TCP_TCC_READ_REQ_LATENCY_sum"] / cycles / cus))
+            if "TCC_EA0_RDREQ_LEVEL_sum" in cs and cs.get("TCC_EA0_RDREQ_sum"):
+                lines.append("  -> average L2-to-fabric read latency: %.0f cycles per request"
+                             % (cs["TCC_EA0_RDREQ_LEVEL_sum"] / cs["TCC_EA0_RDREQ_sum"]))
+            if "TCC_HIT_sum" in cs and "TCC_MISS_sum" in cs and cs["TCC_HIT_sum"] + cs["TCC_MISS_sum"] > 0:
+                lines.append("  -> L2 hit rate: %.1f %%" % (100 * cs["TCC_HIT_sum"] / (cs["TCC_HIT_sum"] + cs["TCC_MISS_sum"])))
+            if "FETCH_SIZE" in cs and "WRITE_SIZE" in cs and "FETCH_SIZE" in scale and "WRITE_SIZE" in scale:
+                f, w = cs["FETCH_SIZE"] * scale["FETCH_SIZE"] * 1024, cs["WRITE_SIZE"] * scale["WRITE_SIZE"] * 1024
+                lines += ["", "scale factors from the calibration copy (1 GiB read + 1 GiB written): FETCH_SIZE x%.4f, WRITE_SIZE x%.4f"
+                          % (scale["FETCH_SIZE"], scale["WRITE_SIZE"]),
+                          "measured_traffic_bytes: %d read + %d written = %.1f MiB per launch of the dominant kernel "
+                          "(algorithmic %.1f MiB)" % (f, w, (f + w) / 2**20, alg / 2**20)]
+        text = "\n".join(lines) + "\n"
+        tag = re.split(r"[<(]", dominant)[0].strip().split("::")[-1]
+        print("== %s (%s)" % (name, tag))
+        print(text)
+        if args.profiles_dir:
+            os.makedirs(args.profiles_dir, exist_ok=True)
+            for old in glob.glob(os.path.join(args.profiles_dir, "*__%s.txt" % name)):
+                os.remove(old)
+            with open(os.path.join(args.profiles_dir, "%s__%s.txt" % (tag, name)), "w") as fh:
+                fh.write(text)
 
 
 if __name__ == "__main__":

@@ -1,16 +1,18 @@
-"""Runs the benchmark's kernels a few times each, for use under rocprofv3:
+"""Runs the benchmark's workloads a few times each, for use under rocprofv3:
 
     rocprofv3 --kernel-trace --stats -d <out> -- python3 nvshmem_amd/profile_workloads.py
-    rocprofv3 --pmc FETCH_SIZE -d <out> -- python3 nvshmem_amd/profile_workloads.py
-    rocprofv3 --pmc WRITE_SIZE -d <out> -- python3 nvshmem_amd/profile_workloads.py
+    rocprofv3 --pmc FETCH_SIZE -d <out> -- python3 nvshmem_amd/profile_workloads.py --iters 3
+    rocprofv3 --pmc WRITE_SIZE -d <out> -- python3 nvshmem_amd/profile_workloads.py --iters 3
+    (any other counter set the same way, one rocprofv3 run per set)
 
-Workloads (same shapes as bench.py): plain_copy calibration (1 GiB read + 1 GiB written),
-put_block (8 PEs x 256 MiB), float sum reduce (8 PEs x 2^26), float sum reducescatter (8 PEs, 256 MiB
-source per PE), broadcast (8 PEs x 256 MiB), then with 16 PEs alltoall and fcollect (2^22 fp32 per
-PE).  The large sources hold random data, as in bench.py: HBM moves all-zero buffers a few per
-cent faster, and the durations here are meant to agree with the benchmark's.
+The workloads are the objects of nvshmem_amd/workloads.py, the ones bench.py times, with numpy noise as
+input (the oracle is not involved).  Every workload is bracketed by two launches of the empty kernel
+profile_marker_kernel, and the order of the workloads is written to --manifest, so that
+nvshmem_amd/profile_summary.py can cut the trace into workloads by counting markers.  The first
+workload is the counter calibration: a plain copy kernel that reads 1 GiB and writes 1 GiB.
 """
 import argparse
+import json
 import os
 import sys
 
@@ -18,7 +20,7 @@ ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
 sys.path.insert(0, ROOT)
 
 
-def moe_plan(np, rng, npes, tokens, topk, experts, zipf_s):
+def noise_plan(np, rng, npes, tokens, topk, experts, zipf_s):
     """Routing and receive layout of the MoE shuffle: top-k distinct experts per token with
     P(expert k) ~ (k + 1)^-s (drawn without replacement through Gumbel keys), rows grouped on the
     destination PE by (expert, source PE, token order).  -> dest_pe, dest_row [npes, tokens * topk],
@@ -30,7 +32,6 @@ def moe_plan(np, rng, npes, tokens, topk, experts, zipf_s):
         keys = logp[None, :] + rng.gumbel(size=(tokens, experts))
         picks[pe] = np.argsort(-keys, axis=1)[:, :topk]
     counts = np.stack([np.bincount(picks[pe].reshape(-1), minlength=experts) for pe in range(npes)])  # [src, expert]
-    # segment (expert, src) starts after all segments in front of it on the expert's PE
     seg = np.zeros((experts, npes), np.int64)
     recv_rows = np.zeros(npes, np.int64)
     for d in range(npes):
@@ -54,129 +55,81 @@ def moe_plan(np, rng, npes, tokens, topk, experts, zipf_s):
     return dest_pe, dest_row, expected, recv_rows
 
 
-def moe_shuffle(N, hip, np, rng, noise, iters):
-    """Config 5: 8 PEs x 8192 tokens x 7168 bf16, top-8 of 256 experts, Zipf(1.1): dispatch, then combine."""
-    npes, T, K, E, row = 8, 8192, 8, 256, 7168 * 2
-    dest_pe, dest_row, expected, recv_rows = moe_plan(np, rng, npes, T, K, E, 1.1)
-    cap, rows = int(recv_rows.max()), T * K
-    rt = N.Runtime(npes=npes, symmetric_size=cap * row + rows * row + T * row + (64 << 20))
-    perf = rt.perftest()
-    send = rt.malloc(T * row); recv = rt.malloc(cap * row); out = rt.malloc(rows * row)
-    d_pe = rt.malloc(rows * 4); d_row = rt.malloc(rows * 8)
-    d_expected = rt.malloc(npes * 8); sig = rt.calloc(npes, 8)
-    for pe in range(npes):
-        rt.upload(send, pe, np.roll(noise[:T * row], 4096 * (pe + 1)))
-    rt.upload_all(d_pe, dest_pe); rt.upload_all(d_row, dest_row); rt.upload_all(d_expected, expected)
-    for _ in range(iters):
-        assert perf.nvshmem_perftest_fill_words(sig, 0, npes, None) == 0
-        assert perf.nvshmem_perftest_moe_dispatch_pieces(recv, cap, send, d_pe, d_row, d_expected, sig, T, K, row,
-                                                         1024, 256, None) == 0
-        assert perf.nvshmem_perftest_moe_combine_pieces(out, recv, cap, d_pe, d_row, T, K, row, 2048, 262144, 64,
-                                                        N.SCOPE_WARP, None) == 0
-    hip.synchronize()
-    assert all(rt.read_timeout(pe)[0] == 0 for pe in range(npes)), "a receiver gave up waiting"
-    # the round trip gives every row back: spot check
-    for pe in (0, npes - 1):
-        got = rt.download(out, pe, (64, row), np.uint8)
-        want = np.repeat(np.roll(noise[:T * row], 4096 * (pe + 1)).reshape(T, row)[:8], K, axis=0)
-        assert np.array_equal(got, want), "combine(dispatch(x)) != x"
-    rt.finalize()
-
-
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--iters", type=int, default=10)
+    ap.add_argument("--only", default="", help="comma-separated workload names")
+    ap.add_argument("--manifest", default=os.path.join(ROOT, "gpurun_out", "profile_manifest.json"))
     args = ap.parse_args()
     import numpy as np
     import nvshmem_amd as N
-    from nvshmem_amd import _lib, hip
+    from nvshmem_amd import hip, workloads
 
     rng = np.random.default_rng(1)
-    noise = rng.integers(0, 256, 1 << 28, dtype=np.uint8)     # 256 MiB, rotated per PE
+    noise = rng.integers(0, 256, 1 << 28, dtype=np.uint8)     # 256 MiB, rotated per PE and tiled when short
 
-    def randomize(rt, ptr, nbytes, as_float=False):
-        for pe in range(rt.npes):
-            block = np.roll(noise[:nbytes], 4096 * (pe + 1))
-            if as_float:   # keep exponents small: random bit patterns would be NaN / inf heavy
-                block = (block.view(np.uint32) & np.uint32(0x007FFFFF)) | np.uint32(0x3F800000)
-                block = block.view(np.uint8)
-            rt.upload(ptr, pe, block)
+    def gen(kind, npes, n, seed):
+        """Noise of the right shape; floating-point kinds get bounded exponents (random bit patterns
+        would be mostly NaN and infinity)."""
+        dtype, es = {"bytes": (np.uint8, 1), "u64": (np.uint64, 8), "i32": (np.int32, 4), "f32": (np.float32, 4),
+                     "bf16": (np.uint16, 2)}[kind]
+        out = np.empty((npes, n * es), np.uint8)
+        for pe in range(npes):
+            row = np.roll(noise, 4096 * (pe + 1) + 64 * seed)
+            reps = -(-n * es // row.size)
+            out[pe] = np.tile(row, reps)[:n * es] if reps > 1 else row[:n * es]
+        if kind == "f32":
+            v = out.view(np.uint32)
+            v &= np.uint32(0x807FFFFF); v |= np.uint32(0x3F800000)
+        elif kind == "bf16":
+            v = out.view(np.uint16)
+            v &= np.uint16(0x807F); v |= np.uint16(0x3F80)
+        return out.view(dtype)
 
-    # calibration copy: 1 GiB read, 1 GiB written
+    only = set(x for x in args.only.split(",") if x)
+    manifest = []
+
+    def bracket(perf, name, fn, iters):
+        assert perf.nvshmem_perftest_profile_marker(None) == 0
+        for _ in range(iters):
+            fn()
+        assert perf.nvshmem_perftest_profile_marker(None) == 0
+        hip.synchronize()
+        manifest.append({"name": name, "launches": iters})
+
+    # counter calibration: 1 GiB read, 1 GiB written
     rt = N.Runtime(npes=2, symmetric_size=(2 << 30) + (64 << 20))
     perf = rt.perftest()
     cal_a = rt.calloc(1 << 30, 1)
     cal_b = rt.calloc(1 << 30, 1)
-    for _ in range(args.iters):
+
+    def calibrate():
         assert perf.nvshmem_perftest_plain_copy(cal_b, cal_a, 1 << 30, None) == 0
-    hip.synchronize()
+    bracket(perf, "calibration", calibrate, args.iters)
     rt.finalize()
 
-    # put_block: heap and buffer layout exactly as bench.py's bench_put_block
-    S = 1 << 28
-    rt = N.Runtime(npes=8, symmetric_size=2 * S + (64 << 20))
-    src = rt.calloc(S, 1)
-    dst = rt.calloc(S, 1)
-    randomize(rt, src, S)
-    for _ in range(args.iters):
-        assert perf.nvshmem_perftest_ring_rma(dst, src, S, 262144, 64, N.SCOPE_BLOCK, 0, 1, None) == 0
-    hip.synchronize()
-    rt.finalize()
-
-    # sum_reduce: as bench_sum_reduce
-    n = 1 << 26
-    rt = N.Runtime(npes=8, symmetric_size=2 * n * 4 + (64 << 20))
-    src = rt.calloc(n, 4)
-    dst = rt.calloc(n, 4)
-    randomize(rt, src, n * 4, as_float=True)
-    red = _lib.typed_coll(rt.lib, "nvshmemx_float_sum_reduce_on_stream", True)
-    for _ in range(args.iters):
-        assert red(N.TEAM_WORLD, dst, src, n, None) == 0
-    hip.synchronize()
-    rt.finalize()
-
-    # reducescatter (source 8 blocks of 2^23 fp32 per PE) and broadcast (256 MiB from PE 3)
-    n = 1 << 23
-    rt = N.Runtime(npes=8, symmetric_size=9 * n * 4 + (64 << 20))
-    src = rt.calloc(8 * n, 4)
-    dst = rt.calloc(n, 4)
-    randomize(rt, src, 8 * n * 4, as_float=True)
-    for _ in range(args.iters):
-        rt.reducescatter("float", "sum", dst, src, n, stream=None)
-    hip.synchronize()
-    rt.free(dst)
-    dst = None
-    rt.finalize()
-    S = 1 << 28
-    rt = N.Runtime(npes=8, symmetric_size=2 * S + (64 << 20))
-    src = rt.calloc(S, 1)
-    dst = rt.calloc(S, 1)
-    randomize(rt, src, S)
-    for _ in range(args.iters):
-        rt.broadcastmem(dst, src, S, 3)
-    hip.synchronize()
-    rt.finalize()
-
-    # alltoall as bench_alltoall, then fcollect of the same source into a 16x larger destination
-    n = 1 << 22
-    rt = N.Runtime(npes=16, symmetric_size=2 * n * 4 + (16 << 20))
-    src = rt.calloc(n, 4)
-    dst = rt.calloc(n, 4)
-    randomize(rt, src, n * 4)
-    for _ in range(args.iters):
-        rt.alltoall("float", dst, src, n // 16, stream=None)
-    hip.synchronize()
-    rt.finalize()
-    rt = N.Runtime(npes=16, symmetric_size=(512 << 20))
-    src = rt.calloc(n, 4)
-    dst = rt.calloc(16 * n, 4)
-    randomize(rt, src, n * 4)
-    for _ in range(args.iters):
-        rt.fcollect("float", dst, src, n, stream=None)
-    hip.synchronize()
-    rt.finalize()
-    moe_shuffle(N, hip, np, rng, noise, max(2, args.iters // 2))
-    print("profile_workloads: done (%d iterations each)" % args.iters)
+    plan = noise_plan(np, rng, 8, 8192, 8, 256, 1.1)
+    for g in workloads.all_groups(plan):
+        if only and not any(n in only for n in g.names()):
+            continue
+        rt = N.Runtime(npes=g.npes, symmetric_size=g.heap_bytes)
+        try:
+            for item in g.setup(rt, gen):
+                if only and item.name not in only:
+                    continue
+                if hasattr(item, "prepare"):
+                    item.prepare()
+                iters = max(2, args.iters // item.scale)
+                item.step()                    # one untimed pass (first touch of the destination)
+                hip.synchronize()
+                bracket(rt.perftest(), item.name, item.step, iters)
+                manifest[-1].update(algorithmic_bytes=item.algorithmic_bytes, workload=item.workload)
+        finally:
+            rt.finalize()
+    os.makedirs(os.path.dirname(args.manifest), exist_ok=True)
+    with open(args.manifest, "w") as fh:
+        json.dump(manifest, fh, indent=1)
+    print("profile_workloads: %d workloads, manifest %s" % (len(manifest), args.manifest))
 
 
 if __name__ == "__main__":
