@@ -114,12 +114,17 @@ NVSHMEMI_DEVICE_INLINE int nvshmemi_amd_my_pe() {
 }
 NVSHMEMI_DEVICE_INLINE int nvshmemi_amd_n_pes() { return nvshmemi_device_state_d.npes; }
 
+/* Offset inside its slice of an address anywhere in the heap.  Symmetric addresses are nearly always
+ * canonical (PE 0's slice), where the offset is the distance from the heap base; the division only
+ * runs for an address that names another PE's copy. */
+NVSHMEMI_DEVICE_INLINE uint64_t nvshmemi_amd_slice_offset(const void *sym) {
+    const uint64_t d = (uint64_t)((const char *)sym - nvshmemi_device_state_d.heap_base);
+    return d < nvshmemi_device_state_d.heap_size ? d : d % nvshmemi_device_state_d.heap_size;
+}
 /* Address of PE `pe`'s copy of the symmetric object at `sym` (an address in any PE's slice). */
 NVSHMEMI_DEVICE_INLINE char *nvshmemi_amd_remote(const void *sym, int pe) {
-    const uint64_t off = (uint64_t)((const char *)sym - nvshmemi_device_state_d.heap_base) &
-                         (nvshmemi_device_state_d.heap_size - 1);
-    return nvshmemi_device_state_d.heap_base +
-           ((uint64_t)(unsigned)pe << nvshmemi_device_state_d.heap_shift) + off;
+    return nvshmemi_device_state_d.heap_base + (uint64_t)(unsigned)pe * nvshmemi_device_state_d.heap_size +
+           nvshmemi_amd_slice_offset(sym);
 }
 
 /* Local operand: a canonical address means "my copy"; anything else is taken literally. */
@@ -127,14 +132,14 @@ NVSHMEMI_DEVICE_INLINE char *nvshmemi_amd_local(const void *p) {
     const uint64_t off = (uint64_t)((const char *)p - nvshmemi_device_state_d.heap_base);
     if (off < nvshmemi_device_state_d.heap_size)
         return nvshmemi_device_state_d.heap_base +
-               ((uint64_t)(unsigned)nvshmemi_amd_my_pe() << nvshmemi_device_state_d.heap_shift) + off;
+               (uint64_t)(unsigned)nvshmemi_amd_my_pe() * nvshmemi_device_state_d.heap_size + off;
     return (char *)p;
 }
 
 NVSHMEMI_DEVICE_INLINE void *nvshmemi_ptr(const void *ptr, int pe) {
     const uint64_t off = (uint64_t)((const char *)ptr - nvshmemi_device_state_d.heap_base);
     if (pe >= 0 && pe < nvshmemi_device_state_d.npes &&
-        off < ((uint64_t)(unsigned)nvshmemi_device_state_d.npes << nvshmemi_device_state_d.heap_shift))
+        off < (uint64_t)(unsigned)nvshmemi_device_state_d.npes * nvshmemi_device_state_d.heap_size)
         return nvshmemi_amd_remote(ptr, pe);
     return nullptr;
 }
@@ -538,6 +543,9 @@ NVSHMEMI_DEVICE_INLINE void nvshmemi_amd_record_timeout(const void *addr, uint64
     rec[2] = found;
     rec[3] = expected;
     __hip_atomic_store(rec, (uint64_t)1, __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_AGENT);
+    /* the count the host checks at its synchronisation points */
+    __hip_atomic_fetch_add(nvshmemi_device_state_d.runtime_words + NVSHMEMI_AMD_TIMEOUT_COUNT_WORD, (uint64_t)1,
+                           __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 }
 
 /* Spin until `*ivar cmp value`; `ivar` is a local operand.  Returns the value that ended the wait.

@@ -383,6 +383,13 @@ NVSHMEMI_HOST_ONLY int nvshmemx_amd_module_init(void);
 NVSHMEMI_HOST_ONLY void nvshmemx_amd_set_spin_limit(uint64_t polls);
 /* Copies PE `pe`'s timeout record (4 words) to `out` and clears it; returns the flag word. */
 NVSHMEMI_HOST_ONLY uint64_t nvshmemx_amd_read_timeout(int pe, uint64_t out[4]);
+/* A wait that gives up does not stay silent.  The device counts every one; the host calls that wait
+ * for the device - nvshmem_quiet, nvshmem_fence, nvshmem_barrier_all / nvshmem_sync_all, nvshmem_barrier /
+ * nvshmem_team_sync (which then return non-zero), nvshmem_free, nvshmem_finalize - compare the count
+ * with what they reported before, and for new timeouts print a message (how many, the spin limit, one
+ * PE's record) to stderr and leave it in nvshmemx_amd_last_error().  This call returns the count since
+ * nvshmem_init without reporting or clearing anything. */
+NVSHMEMI_HOST_ONLY uint64_t nvshmemx_amd_timeout_count(void);
 
 /* Last error text of the calling thread ("" if none); argument errors are reported here and as a
  * non-zero return instead of terminating the process. */

@@ -58,6 +58,7 @@ def load():
         "nvshmem_quiet": (None, []),
         "nvshmem_fence": (None, []),
         "nvshmem_barrier_all": (None, []),
+        "nvshmemx_amd_timeout_count": (u64, []),
         "nvshmem_barrier": (i32, [i32]),
         "nvshmem_sync_all": (None, []),
         "nvshmemx_barrier_all_on_stream": (None, [vp]),

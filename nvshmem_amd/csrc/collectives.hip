@@ -110,7 +110,7 @@ __device__ __forceinline__ void copy_tile(char *__restrict__ dst, const char *__
 }
 
 template <int MODE, int kCopyUnroll, bool NTL>
-__global__ __launch_bounds__(kCopyThreads) void segment_copy_kernel(char *base, uint32_t shift,
+__global__ __launch_bounds__(kCopyThreads) void segment_copy_kernel(char *base, uint64_t slice_bytes,
                                                                 const nvshmemi_amd_team_view_t *groups,
                                                                 int max_size, uint64_t dst_off,
                                                                 uint64_t src_off, uint64_t seg_bytes,
@@ -118,8 +118,8 @@ __global__ __launch_bounds__(kCopyThreads) void segment_copy_kernel(char *base, 
     // this block's team: members are the PEs start + i*stride, i < size
     const nvshmemi_amd_team_view_t g = groups[blockIdx.z];
     const unsigned npes = (unsigned)g.size;
-    base += (uint64_t)g.start << shift;
-    const uint64_t rep_stride = (uint64_t)g.stride << shift;  // from one member to the next
+    base += (uint64_t)g.start * slice_bytes;
+    const uint64_t rep_stride = (uint64_t)g.stride * slice_bytes;  // from one member to the next
     const unsigned seg = blockIdx.y;
     const char *src;
     char *dst;
@@ -199,7 +199,7 @@ __device__ __forceinline__ T fold_next(int p, T acc, T x) {
 }
 
 template <typename T, int OP, int NPES, bool NTL, int VPT = NVSHMEM_AMD_REDUCE_VPT>
-__global__ __launch_bounds__(NPES ? NPES * 64 : 1024) void reduce_vector_kernel(char *base, uint32_t shift,
+__global__ __launch_bounds__(NPES ? NPES * 64 : 1024) void reduce_vector_kernel(char *base, uint64_t slice_bytes,
                                                              const nvshmemi_amd_team_view_t *groups,
                                                              uint32_t lane_shift_arg, uint64_t dst_off,
                                                              uint64_t src_off, uint64_t nelems) {
@@ -208,7 +208,7 @@ __global__ __launch_bounds__(NPES ? NPES * 64 : 1024) void reduce_vector_kernel(
     // this block's team; with NPES > 0 the host has checked that every team has NPES members
     const nvshmemi_amd_team_view_t g = groups[blockIdx.z];
     const int npes = NPES ? NPES : g.size;
-    base += (uint64_t)g.start << shift;
+    base += (uint64_t)g.start * slice_bytes;
     const uint32_t lane_shift = NPES ? 6u : lane_shift_arg;
     const unsigned lanes = 1u << lane_shift;
     const unsigned pe = threadIdx.x >> lane_shift, i = threadIdx.x & (lanes - 1);
@@ -216,7 +216,7 @@ __global__ __launch_bounds__(NPES ? NPES * 64 : 1024) void reduce_vector_kernel(
     // tiles are cut on absolute (16 * lanes)-byte boundaries of the destination, so a wavefront's
     // access is one aligned 1 KiB piece whatever the buffer's own alignment: `lead` vector slots of
     // the first tile lie in front of the buffer
-    const uint64_t pe_stride = (uint64_t)g.stride << shift;  // from one member to the next
+    const uint64_t pe_stride = (uint64_t)g.stride * slice_bytes;  // from one member to the next
     const bool member = NPES ? true : (int)pe < npes;        // the block is sized for the largest team
     const uint64_t lead = ((uint64_t)(uintptr_t)(base + dst_off) >> 4) & (lanes - 1);
     // a tile is VPT pieces of `lanes` vectors per PE: thread (pe, i) loads vector i of each piece
@@ -272,26 +272,29 @@ __global__ __launch_bounds__(NPES ? NPES * 64 : 1024) void reduce_vector_kernel(
 // of 1024 threads leaves 32 or 16 lanes per member, i.e. 512 or 256 byte accesses): a block is ONE
 // wavefront, lane i loads vector i of a 1 KiB piece from every member, eight loads in flight at a time,
 // folds in member order and stores the result to every member.
-template <typename T, int OP, bool NTL>
-__global__ __launch_bounds__(64) void reduce_gather_kernel(char *base, uint32_t shift,
+// NPES > 0 fixes the team size at compile time (loads, fold and stores fully unrolled).
+template <typename T, int OP, int NPES, bool NTL>
+__global__ __launch_bounds__(64) void reduce_gather_kernel(char *base, uint64_t slice_bytes,
                                                            const nvshmemi_amd_team_view_t *groups,
                                                            uint64_t dst_off, uint64_t src_off, uint64_t nelems) {
     constexpr int VEC = 16 / sizeof(T);
     constexpr int kBatch = 8;
+    constexpr int kBatches = NPES ? (NPES + kBatch - 1) / kBatch : 1, kStores = NPES ? NPES : 1;  // unroll counts
     union pack_t {
         nvshmemi_v4u v;
         T e[VEC];
     };
     const nvshmemi_amd_team_view_t g = groups[blockIdx.z];
-    const int npes = g.size;
-    base += (uint64_t)g.start << shift;
-    const uint64_t pe_stride = (uint64_t)g.stride << shift;
+    const int npes = NPES ? NPES : g.size;
+    base += (uint64_t)g.start * slice_bytes;
+    const uint64_t pe_stride = (uint64_t)g.stride * slice_bytes;
     const uint64_t nvec = nelems / VEC;
     const uint64_t lead = ((uint64_t)(uintptr_t)(base + dst_off) >> 4) & 63;
     const uint64_t v = (uint64_t)blockIdx.x * 64 + threadIdx.x - lead;
     if (v < nvec) {
         const char *src = base + src_off + 16 * v;
         pack_t acc;
+#pragma unroll kBatches
         for (int p0 = 0; p0 < npes; p0 += kBatch) {
             pack_t x[kBatch];
 #pragma unroll
@@ -310,6 +313,7 @@ __global__ __launch_bounds__(64) void reduce_gather_kernel(char *base, uint32_t 
                 }
         }
         char *dst = base + dst_off + 16 * v;
+#pragma unroll kStores
         for (int p = 0; p < npes; ++p) stream_store(dst + (uint64_t)p * pe_stride, acc.v);
     }
     // elements behind the last full vector
@@ -333,7 +337,7 @@ __global__ __launch_bounds__(64) void reduce_gather_kernel(char *base, uint32_t 
 // 8 members with 256 MiB of source each, 5.9 against 3.7 TB/s for 16 members.  NPES > 0 fixes the team
 // size at compile time; NPES == 0 reads it from the team.
 template <typename T, int OP, int NPES, bool NTL>
-__global__ __launch_bounds__(64) void reducescatter_gather_kernel(char *base, uint32_t shift,
+__global__ __launch_bounds__(64) void reducescatter_gather_kernel(char *base, uint64_t slice_bytes,
                                                                   const nvshmemi_amd_team_view_t *groups,
                                                                   uint64_t dst_off, uint64_t src_off,
                                                                   uint64_t nelems) {
@@ -346,8 +350,8 @@ __global__ __launch_bounds__(64) void reducescatter_gather_kernel(char *base, ui
     const nvshmemi_amd_team_view_t g = groups[blockIdx.z];
     const int npes = NPES ? NPES : g.size;
     if ((int)blockIdx.y >= npes) return;
-    base += (uint64_t)g.start << shift;
-    const uint64_t pe_stride = (uint64_t)g.stride << shift;
+    base += (uint64_t)g.start * slice_bytes;
+    const uint64_t pe_stride = (uint64_t)g.stride * slice_bytes;
     const uint64_t nvec = nelems / VEC;
     src_off += (uint64_t)blockIdx.y * nelems * sizeof(T);
     // pieces are cut on absolute 1 KiB boundaries of the source: `lead` slots of piece 0 lie in front
@@ -377,16 +381,16 @@ __global__ __launch_bounds__(64) void reducescatter_gather_kernel(char *base, ui
 
 // Element-at-a-time variant for buffers that are not 16-byte aligned.
 template <typename T, int OP, bool SCATTER = false>
-__global__ __launch_bounds__(kThreads) void reduce_scalar_kernel(char *base, uint32_t shift,
+__global__ __launch_bounds__(kThreads) void reduce_scalar_kernel(char *base, uint64_t slice_bytes,
                                                                  const nvshmemi_amd_team_view_t *groups,
                                                                  uint64_t dst_off, uint64_t src_off,
                                                                  uint64_t nelems) {
     const nvshmemi_amd_team_view_t g = groups[blockIdx.z];
     const int npes = g.size;
     if (SCATTER && (int)blockIdx.y >= npes) return;
-    base += (uint64_t)g.start << shift;
+    base += (uint64_t)g.start * slice_bytes;
     const uint64_t gsz = (uint64_t)gridDim.x * kThreads;
-    const uint64_t es = ((uint64_t)g.stride << shift) / sizeof(T);
+    const uint64_t es = ((uint64_t)g.stride * slice_bytes) / sizeof(T);
     const T *s = reinterpret_cast<const T *>(base + src_off) + (SCATTER ? (uint64_t)blockIdx.y * nelems : 0);
     T *d = reinterpret_cast<T *>(base + dst_off) + (SCATTER ? (uint64_t)blockIdx.y * es : 0);
     for (uint64_t i = (uint64_t)blockIdx.x * kThreads + threadIdx.x; i < nelems; i += gsz) {
@@ -450,11 +454,11 @@ void launch_reduce(Runtime &rt, const TeamLaunch &tl, uint64_t dst_off, uint64_t
     do {                                                                                          \
         if (stream_source)                                                                        \
             hipLaunchKernelGGL((reduce_vector_kernel<T, OP, N, true>), grid, dim3(threads), lds,  \
-                               stream, rt.base, rt.heap_shift, tl.groups, lane_shift, dst_off,    \
+                               stream, rt.base, rt.heap_size, tl.groups, lane_shift, dst_off,    \
                                src_off, nelems);                                                  \
         else                                                                                      \
             hipLaunchKernelGGL((reduce_vector_kernel<T, OP, N, false>), grid, dim3(threads), lds, \
-                               stream, rt.base, rt.heap_shift, tl.groups, lane_shift, dst_off,    \
+                               stream, rt.base, rt.heap_size, tl.groups, lane_shift, dst_off,    \
                                src_off, nelems);                                                  \
     } while (0)
         if (fixed_size == 8) NVSHMEM_AMD_LAUNCH_REDUCE(8);
@@ -468,18 +472,26 @@ void launch_reduce(Runtime &rt, const TeamLaunch &tl, uint64_t dst_off, uint64_t
             return;
         }
         const dim3 grid((unsigned)blocks, 1, ngroups);
-        if (stream_source)
-            hipLaunchKernelGGL((reduce_gather_kernel<T, OP, true>), grid, dim3(64), 0, stream, rt.base,
-                               rt.heap_shift, tl.groups, dst_off, src_off, nelems);
-        else
-            hipLaunchKernelGGL((reduce_gather_kernel<T, OP, false>), grid, dim3(64), 0, stream, rt.base,
-                               rt.heap_shift, tl.groups, dst_off, src_off, nelems);
+#define NVSHMEM_AMD_LAUNCH_GATHER_REDUCE(N)                                                            \
+    do {                                                                                               \
+        if (stream_source)                                                                             \
+            hipLaunchKernelGGL((reduce_gather_kernel<T, OP, N, true>), grid, dim3(64), 0, stream, rt.base, \
+                               rt.heap_size, tl.groups, dst_off, src_off, nelems);                    \
+        else                                                                                           \
+            hipLaunchKernelGGL((reduce_gather_kernel<T, OP, N, false>), grid, dim3(64), 0, stream, rt.base, \
+                               rt.heap_size, tl.groups, dst_off, src_off, nelems);                    \
+    } while (0)
+        // (sixteen members unrolled measured slower than the loop: 5.2 against 5.4 TB/s)
+        if (fixed_size == 4) NVSHMEM_AMD_LAUNCH_GATHER_REDUCE(4);
+        else if (fixed_size == 8) NVSHMEM_AMD_LAUNCH_GATHER_REDUCE(8);
+        else NVSHMEM_AMD_LAUNCH_GATHER_REDUCE(0);
+#undef NVSHMEM_AMD_LAUNCH_GATHER_REDUCE
     } else {
         uint64_t blocks = (nelems + kThreads - 1) / kThreads;
         const uint64_t cap = (uint64_t)rt.num_cus * 64 / ngroups + 1;
         if (blocks > cap) blocks = cap;
         hipLaunchKernelGGL((reduce_scalar_kernel<T, OP>), dim3((unsigned)blocks, 1, ngroups),
-                           dim3(kThreads), 0, stream, rt.base, rt.heap_shift, tl.groups, dst_off,
+                           dim3(kThreads), 0, stream, rt.base, rt.heap_size, tl.groups, dst_off,
                            src_off, nelems);
     }
 }
@@ -502,7 +514,7 @@ void launch_reducescatter(Runtime &rt, const TeamLaunch &tl, uint64_t dst_off, u
             total_members(tl) * tl.max_size * nelems * sizeof(T) > rt.cacheable_source_bytes;
 #define NVSHMEM_AMD_LAUNCH_GATHER(N, NTL)                                                         \
     hipLaunchKernelGGL((reducescatter_gather_kernel<T, OP, N, NTL>), grid, dim3(64), 0, stream,   \
-                       rt.base, rt.heap_shift, tl.groups, dst_off, src_off, nelems)
+                       rt.base, rt.heap_size, tl.groups, dst_off, src_off, nelems)
         if (tl.min_size == 8 && tl.max_size == 8) {
             if (stream_source) NVSHMEM_AMD_LAUNCH_GATHER(8, true);
             else NVSHMEM_AMD_LAUNCH_GATHER(8, false);
@@ -517,7 +529,7 @@ void launch_reducescatter(Runtime &rt, const TeamLaunch &tl, uint64_t dst_off, u
         if (blocks > cap) blocks = cap;
         hipLaunchKernelGGL((reduce_scalar_kernel<T, OP, true>),
                            dim3((unsigned)blocks, (unsigned)tl.max_size, ngroups), dim3(kThreads), 0,
-                           stream, rt.base, rt.heap_shift, tl.groups, dst_off, src_off, nelems);
+                           stream, rt.base, rt.heap_size, tl.groups, dst_off, src_off, nelems);
     }
 }
 
@@ -682,11 +694,11 @@ int broadcast_on_stream(nvshmem_team_t team, void *dest, const void *src, size_t
     // blocks that share a piece re-read it from the cache, so the loads stay cacheable then
     if (part_shift == 0 && big_source)
         hipLaunchKernelGGL((segment_copy_kernel<kModeBroadcast, 1, true>), grid, block, 0, stream,
-                           rt.base, rt.heap_shift, tl.groups, tl.max_size, doff, soff,
+                           rt.base, rt.heap_size, tl.groups, tl.max_size, doff, soff,
                            (uint64_t)bytes, root, part_shift);
     else
         hipLaunchKernelGGL((segment_copy_kernel<kModeBroadcast, 1, false>), grid, block, 0, stream,
-                           rt.base, rt.heap_shift, tl.groups, tl.max_size, doff, soff,
+                           rt.base, rt.heap_size, tl.groups, tl.max_size, doff, soff,
                            (uint64_t)bytes, root, part_shift);
     hipError_t e = hipGetLastError();
     if (e != hipSuccess) {
@@ -732,7 +744,7 @@ static int segment_collective(int mode, const char *what, nvshmem_team_t team, v
     const dim3 grid((unsigned)tiles, segs, (unsigned)tl.ngroups), block(kCopyThreads);
 #define NVSHMEM_AMD_LAUNCH_SEGCOPY(MODE, U, NTL)                                                   \
     hipLaunchKernelGGL((segment_copy_kernel<MODE, U, NTL>), grid, block, 0, stream, rt.base,       \
-                       rt.heap_shift, tl.groups, tl.max_size, doff, soff, (uint64_t)seg_bytes, 0,  \
+                       rt.heap_size, tl.groups, tl.max_size, doff, soff, (uint64_t)seg_bytes, 0,  \
                        part_shift)
     if (mode == kModeFcollect) {
         if (stream_source) NVSHMEM_AMD_LAUNCH_SEGCOPY(kModeFcollect, NVSHMEM_AMD_FCOLLECT_UNROLL, true);

@@ -50,12 +50,41 @@ bool check_symmetric_range(Runtime &rt, const char *what, const void *p, uint64_
         set_error("%s: %p is not a symmetric address", what, p);
         return false;
     }
-    if (bytes > rt.heap_size || *off + bytes > rt.heap_size) {
+    // the runtime's own words (barrier rows, epoch, timeout record) end every slice and are not the
+    // caller's to address
+    const uint64_t usable = rt.heap_size - NVSHMEMI_AMD_INTERNAL_BYTES;
+    if (bytes > usable || *off + bytes > usable) {
         set_error("%s: range [%p, +%llu) leaves the PE's heap slice (%llu bytes per PE)", what, p,
-                  (unsigned long long)bytes, (unsigned long long)rt.heap_size);
+                  (unsigned long long)bytes, (unsigned long long)usable);
         return false;
     }
     return true;
+}
+
+uint64_t report_timeouts(Runtime &rt, const char *where) {
+    if (!rt.initialized || !rt.dev.runtime_words) return 0;
+    uint64_t count = 0;
+    if (hipMemcpy(&count, rt.dev.runtime_words + NVSHMEMI_AMD_TIMEOUT_COUNT_WORD, sizeof count,
+                  hipMemcpyDeviceToHost) != hipSuccess) {
+        (void)hipGetLastError();
+        return 0;
+    }
+    if (count <= rt.timeouts_seen) return 0;
+    const uint64_t fresh = count - rt.timeouts_seen;
+    rt.timeouts_seen = count;
+    // the most recent record of the first PE that has one says where
+    uint64_t rec[4] = {0, 0, 0, 0};
+    int pe_hit = -1;
+    uint64_t off = 0;
+    rt.offset_of(rt.dev.timeout_record, &off);
+    for (int pe = 0; pe < rt.npes && pe_hit < 0; ++pe)
+        if (hipMemcpy(rec, rt.slice(pe) + off, sizeof rec, hipMemcpyDeviceToHost) == hipSuccess && rec[0]) pe_hit = pe;
+    set_error("%s: %llu device-side wait%s gave up after the spin limit of %llu polls (NVSHMEM_AMD_SPIN_LIMIT; 0 waits "
+              "forever) and the kernel went on as if satisfied - results may be incomplete; e.g. PE %d waited at %p "
+              "for %llu and last saw %llu",
+              where, (unsigned long long)fresh, fresh == 1 ? "" : "s", (unsigned long long)rt.dev.spin_limit, pe_hit,
+              (void *)(uintptr_t)rec[1], (unsigned long long)rec[3], (unsigned long long)rec[2]);
+    return fresh;
 }
 
 namespace {
@@ -137,13 +166,14 @@ int nvshmemx_amd_init(int npes, size_t symmetric_size) {
     uint64_t want = symmetric_size < min_slice ? min_slice : (uint64_t)symmetric_size;
     // room for the runtime's own symmetric words (barrier row, epoch, timeout record)
     want += NVSHMEMI_AMD_INTERNAL_BYTES;
-    uint32_t shift = 16;
-    while ((1ull << shift) < want) {
-        if (++shift > 40) {
-            set_error("nvshmemx_amd_init: symmetric size %zu too large", symmetric_size);
-            return NVSHMEMX_ERROR_INVALID_VALUE;
-        }
+    // slices start on 2 MiB boundaries (the granule of the GPU's large page fragments) and are no
+    // larger than asked for beyond that: the distance between them need not be a power of two
+    const uint64_t granule = 2ull << 20;
+    if (want > (1ull << 40)) {
+        set_error("nvshmemx_amd_init: symmetric size %zu too large", symmetric_size);
+        return NVSHMEMX_ERROR_INVALID_VALUE;
     }
+    const uint64_t slice_bytes = (want + granule - 1) / granule * granule;
     int dev = 0;
     if (hipGetDevice(&dev) != hipSuccess) {
         set_error("nvshmemx_amd_init: no HIP device available");
@@ -154,20 +184,19 @@ int nvshmemx_amd_init(int npes, size_t symmetric_size) {
         set_error("nvshmemx_amd_init: hipGetDeviceProperties failed");
         return NVSHMEMX_ERROR_INTERNAL;
     }
-    const uint64_t total = (uint64_t)npes << shift;
+    const uint64_t total = (uint64_t)npes * slice_bytes;
     void *mem = nullptr;
     hipError_t e = hipMalloc(&mem, total);
     if (e != hipSuccess || !mem) {
         (void)hipGetLastError();
         set_error("nvshmemx_amd_init: hipMalloc of %llu bytes (%d PEs x %llu) failed: %s",
-                  (unsigned long long)total, npes, 1ull << shift, hipGetErrorString(e));
+                  (unsigned long long)total, npes, (unsigned long long)slice_bytes, hipGetErrorString(e));
         return NVSHMEMX_ERROR_OUT_OF_MEMORY;
     }
     rt.device = dev;
     rt.num_cus = prop.multiProcessorCount;
     rt.npes = npes;
-    rt.heap_shift = shift;
-    rt.heap_size = 1ull << shift;
+    rt.heap_size = slice_bytes;
     rt.base = (char *)mem;
     // The runtime's own symmetric words (barrier row, epoch, timeout record) live in the last
     // granules of every slice, outside the allocator's space, so that user allocations start at the
@@ -186,7 +215,6 @@ int nvshmemx_amd_init(int npes, size_t symmetric_size) {
     rt.dev.version = (1u << 16) + (uint32_t)sizeof(nvshmemi_device_state_t);
     rt.dev.mype = 0;
     rt.dev.npes = npes;
-    rt.dev.heap_shift = shift;
     rt.dev.heap_base = rt.base;
     rt.dev.heap_size = rt.heap_size;
     rt.dev.sync_flags = (uint64_t *)(uintptr_t)flags;
@@ -230,6 +258,8 @@ void nvshmem_finalize(void) {
     std::lock_guard<std::recursive_mutex> lock(rt.mu);
     if (!rt.initialized) return;
     (void)hipDeviceSynchronize();
+    (void)report_timeouts(rt, "nvshmem_finalize");
+    rt.timeouts_seen = 0;
     teams_finalize(rt);
     (void)hipFree(rt.base);
     rt.space.reset();
@@ -367,6 +397,7 @@ void nvshmem_free(void *ptr) {
     if (!ptr || !require_init(rt, "nvshmem_free")) return;
     // barrier before release, as in the reference: no PE may still be using the block
     NVSHMEM_AMD_HIP_CHECK(hipDeviceSynchronize());
+    (void)report_timeouts(rt, "nvshmem_free");
     uint64_t off = 0;
     if (!rt.offset_of(ptr, &off) ||
         !rt.space->deallocate((uint64_t)(uintptr_t)rt.base + off)) {
@@ -386,13 +417,24 @@ void *nvshmem_ptr(const void *ptr, int pe) {
  * Ordering.  Every logical PE's work is stream work of this one process, so completion of all PEs
  * is completion of the device's streams.
  * ------------------------------------------------------------------------------------------- */
-void nvshmem_quiet(void) { NVSHMEM_AMD_HIP_CHECK(hipDeviceSynchronize()); }
-void nvshmem_fence(void) { NVSHMEM_AMD_HIP_CHECK(hipDeviceSynchronize()); }
-void nvshmem_barrier_all(void) {
+static uint64_t device_wait(const char *where) {
     Runtime &rt = Runtime::get();
     std::lock_guard<std::recursive_mutex> lock(rt.mu);
     refresh_symbols(rt, false);
     NVSHMEM_AMD_HIP_CHECK(hipDeviceSynchronize());
+    return report_timeouts(rt, where);
+}
+void nvshmem_quiet(void) { (void)device_wait("nvshmem_quiet"); }
+void nvshmem_fence(void) { (void)device_wait("nvshmem_fence"); }
+void nvshmem_barrier_all(void) { (void)device_wait("nvshmem_barrier_all"); }
+uint64_t nvshmemx_amd_timeout_count(void) {
+    Runtime &rt = Runtime::get();
+    std::lock_guard<std::recursive_mutex> lock(rt.mu);
+    uint64_t count = 0;
+    if (rt.initialized && rt.dev.runtime_words)
+        NVSHMEM_AMD_HIP_CHECK(hipMemcpy(&count, rt.dev.runtime_words + NVSHMEMI_AMD_TIMEOUT_COUNT_WORD, sizeof count,
+                                        hipMemcpyDeviceToHost));
+    return count;
 }
 /* The host thread stands for every PE of any team, so a team barrier is the device-wide wait too. */
 static int known_team(const char *what, nvshmem_team_t team) {
@@ -402,8 +444,7 @@ static int known_team(const char *what, nvshmem_team_t team) {
 int nvshmem_barrier(nvshmem_team_t team) {
     std::lock_guard<std::recursive_mutex> lock(Runtime::get().mu);
     if (known_team("nvshmem_barrier", team)) return NVSHMEMX_ERROR_INVALID_VALUE;
-    nvshmem_barrier_all();
-    return 0;
+    return device_wait("nvshmem_barrier") ? NVSHMEMX_ERROR_INTERNAL : 0;
 }
 void nvshmem_sync_all(void) { nvshmem_barrier_all(); }
 int nvshmem_team_sync(nvshmem_team_t team) { return nvshmem_barrier(team); }

@@ -50,8 +50,7 @@ struct Runtime {
     int device = 0;
     int npes = 0;
     int num_cus = 0;
-    uint32_t heap_shift = 0;
-    uint64_t heap_size = 0;  // bytes per PE, power of two
+    uint64_t heap_size = 0;  // bytes from one PE's slice to the next, a multiple of 2 MiB
     char *base = nullptr;    // start of PE 0's slice
     std::unique_ptr<SymmetricSpace> space;
     nvshmemi_device_state_t dev{};
@@ -66,24 +65,28 @@ struct Runtime {
     // all PEs together hold more than this many bytes' worth of 4-byte elements:
     // NVSHMEM_AMD_LDS_REDUCE_BYTES, read at init
     uint64_t lds_reduce_bytes = (uint64_t)1 << 30;
+    uint64_t timeouts_seen = 0;  // bounded waits that gave up, as far as the host has reported them
 
     static Runtime &get();
 
     // Offset of a symmetric address inside its PE slice; false when p is outside the heap.
     bool offset_of(const void *p, uint64_t *off) const {
         const uint64_t d = (uint64_t)((const char *)p - base);
-        if (!initialized || p == nullptr || (const char *)p < base ||
-            d >= ((uint64_t)npes << heap_shift))
+        if (!initialized || p == nullptr || (const char *)p < base || d >= (uint64_t)npes * heap_size)
             return false;
-        *off = d & (heap_size - 1);
+        *off = d % heap_size;
         return true;
     }
-    char *slice(int pe) const { return base + ((uint64_t)pe << heap_shift); }
+    char *slice(int pe) const { return base + (uint64_t)pe * heap_size; }
 };
 
 // Records a message for nvshmemx_amd_last_error() and prints it to stderr.
 void set_error(const char *fmt, ...) __attribute__((format(printf, 1, 2)));
 void clear_error();
+
+// After the device has been synchronised: reports bounded device-side waits that gave up since the last
+// check (stderr, nvshmemx_amd_last_error) and returns how many there were.
+uint64_t report_timeouts(Runtime &rt, const char *where);
 
 // Pushes the state block to every registered translation unit when it changed.
 void refresh_symbols(Runtime &rt, bool force);

@@ -47,7 +47,8 @@ def test_malloc_ptr_translation_matches_closed_form(rt):
     b = rt.malloc(1)
     assert a % 512 == 0 and b == a + 1024          # 512-byte granules, first fit
     heap_size = rt.ptr(a, 1) - rt.ptr(a, 0)
-    assert heap_size >= (1 << 30) and heap_size & (heap_size - 1) == 0
+    # slices are 2 MiB-aligned and no larger than asked for beyond that (no rounding to a power of two)
+    assert (1 << 30) <= heap_size <= (1 << 30) + (2 << 20) and heap_size % (2 << 20) == 0
     assert rt.ptr(a, 0) == a                       # canonical address is PE 0's copy
     L = O.lib()
     for pe in range(NPES):
@@ -168,20 +169,64 @@ def test_ring_put_get_256MiB_16_blocks(rt, is_get):
     rt.free(src); rt.free(dst)
 
 
-def test_ring_put_get_8MiB_to_128MiB_and_the_gpu_filling_shape(rt):
-    # the upper half of the sweep (config 2: 8 B ... 256 MiB), block counts 1 / 4 / 16 in turn, and
-    # the launch shape the benchmark uses (one wavefront per KiB) at 256 MiB
+def _sampled_equal(rt, dst, pe, want, size, size_max):
+    """Compares windows of the destination instead of all of it: both ends, every slice boundary of a
+    16-block launch, and the bytes behind the message, which must still be zero."""
+    edges = sorted(set([0, size] + [size // 16 * b for b in range(1, 16)] + [size // 4 * b for b in range(1, 4)]))
+    for e in edges:
+        lo, hi = max(0, e - (1 << 16)), min(size, e + (1 << 16))
+        if hi > lo:
+            got = rt.download(dst, pe, (hi - lo,), np.uint8, lo)
+            if not np.array_equal(got, want[lo:hi]):
+                return False
+    tail = min(4096, size_max - size)
+    return tail == 0 or bool((rt.download(dst, pe, (tail,), np.uint8, size) == 0).all())
+
+
+def test_ring_put_get_upper_half_of_the_sweep_every_block_count_and_direction(rt):
+    # config 2's sizes from 8 MiB to 256 MiB, each at 1 / 4 / 16 blocks of 1024 threads, put and get:
+    # one PE compared in full (it changes from case to case), the others on sampled windows
     perf = rt.perftest()
     size_max = 1 << 28
     src = rt.malloc(size_max); dst = rt.malloc(size_max)
     data = O.fill_all("bytes", NPES, size_max, 3)
     rt.upload_all(src, data)
-    cases = [(1 << p, (1, 4, 16)[p % 3], 1024, p % 2) for p in range(23, 28)]
-    cases += [(size_max, size_max >> 10, 64, 0), (size_max, size_max >> 10, 64, 1), ((1 << 27) + 12345, 1 << 17, 64, 0)]
-    for size, blocks, threads, is_get in cases:
+    case = 0
+    for p in range(23, 29):
+        for blocks in (1, 4, 16):
+            for is_get in (0, 1):
+                size = 1 << p
+                rt.fill(dst, 0, size_max)
+                note("ring_rma size=%d blocks=%d get=%d" % (size, blocks, is_get))
+                assert perf.nvshmem_perftest_ring_rma(dst, src, size, blocks, 1024, N.SCOPE_BLOCK, is_get, 1, None) == 0
+                rt.sync()
+                full = case % NPES
+                case += 1
+                for pe in range(NPES):
+                    want = data[(pe + 1) % NPES] if is_get else data[(pe - 1) % NPES]
+                    if pe == full:
+                        got = rt.download(dst, pe, (size,), np.uint8)
+                        assert np.array_equal(got, want[:size]), (size, blocks, is_get, pe)
+                    assert _sampled_equal(rt, dst, pe, want, size, size_max), (size, blocks, is_get, pe)
+    rt.free(src); rt.free(dst)
+
+
+def test_ring_put_get_large_messages_other_scopes_and_the_gpu_filling_shape(rt):
+    # warp and thread scope at 64 MiB and more, a ragged 128 MiB + 12345, and the launch shape with one
+    # wavefront per KiB at 256 MiB
+    perf = rt.perftest()
+    size_max = 1 << 28
+    src = rt.malloc(size_max); dst = rt.malloc(size_max)
+    data = O.fill_all("bytes", NPES, size_max, 4)
+    rt.upload_all(src, data)
+    cases = [(1 << 26, 16, 256, N.SCOPE_WARP, 0), (1 << 27, 64, 512, N.SCOPE_WARP, 1),
+             ((1 << 26) + 77, 256, 256, N.SCOPE_THREAD, 0), (1 << 26, 1024, 64, N.SCOPE_THREAD, 1),
+             (size_max, size_max >> 10, 64, N.SCOPE_BLOCK, 0), (size_max, size_max >> 10, 64, N.SCOPE_BLOCK, 1),
+             ((1 << 27) + 12345, 1 << 17, 64, N.SCOPE_BLOCK, 0), ((1 << 27) + 12345, 4, 1024, N.SCOPE_BLOCK, 1)]
+    for size, blocks, threads, scope, is_get in cases:
         rt.fill(dst, 0, size_max)
-        note("ring_rma size=%d blocks=%d threads=%d get=%d" % (size, blocks, threads, is_get))
-        assert perf.nvshmem_perftest_ring_rma(dst, src, size, blocks, threads, N.SCOPE_BLOCK, is_get, 1, None) == 0
+        note("ring_rma size=%d blocks=%d threads=%d scope=%d get=%d" % (size, blocks, threads, scope, is_get))
+        assert perf.nvshmem_perftest_ring_rma(dst, src, size, blocks, threads, scope, is_get, 1, None) == 0
         rt.sync()
         for pe in (0, 3, NPES - 1):
             got = rt.download(dst, pe, (min(size + 4096, size_max),), np.uint8)

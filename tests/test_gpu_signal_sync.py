@@ -98,8 +98,18 @@ def test_bounded_wait_gives_up_and_records_the_timeout(rt):
     rt.lib.nvshmemx_amd_set_spin_limit(200)
     try:
         note("bounded wait: spin limit 200, condition never true")
+        before = rt.lib.nvshmemx_amd_timeout_count()
         assert perf.nvshmem_perftest_signal_wait(sig, N.CMP["GE"], 5, out, None) == 0
         rt.sync()
+        # the host call that waited for the device reports the waits that gave up ...
+        assert rt.lib.nvshmemx_amd_timeout_count() == before + NPES
+        msg = rt.last_error()
+        assert "%d device-side waits gave up" % NPES in msg and "spin limit of 200 polls" in msg
+        # ... once: a second synchronisation has nothing new to say, a team barrier returns 0 again
+        assert rt.lib.nvshmem_barrier(N.TEAM_WORLD) == 0
+        assert perf.nvshmem_perftest_signal_wait(sig, N.CMP["GE"], 5, out, None) == 0
+        assert rt.lib.nvshmem_barrier(N.TEAM_WORLD) != 0       # new timeouts: the barrier says so
+        assert rt.lib.nvshmemx_amd_timeout_count() == before + 2 * NPES
         for pe in range(NPES):
             flag, rec = rt.read_timeout(pe)
             assert flag == 1
