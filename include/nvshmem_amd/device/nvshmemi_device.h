@@ -278,9 +278,23 @@ NVSHMEMI_DEVICE_INLINE size_t nvshmemi_amd_copy_deep_rounds(char *__restrict__ d
     const size_t rounds = nvec / per_round;
     const size_t wave = (size_t)__builtin_amdgcn_readfirstlane(tid >> 6);
     const unsigned lane_off = (tid & 63u) * 16u;
-    const char *s = src + wave * (size_t)(U * 1024);
-    char *d = dst + wave * (size_t)(U * 1024);
-    for (size_t r = 0; r < rounds; ++r, s += 16 * per_round, d += 16 * per_round) {
+    const char *s0 = src + wave * (size_t)(U * 1024);
+    char *d0 = dst + wave * (size_t)(U * 1024);
+    /* The rounds are walked from a start that differs from block to block, wrapping at the end.  Blocks
+     * that each stream a slice of one large message otherwise march in step, at equal offsets in slices
+     * that lie a power of two (or the PE distance) apart, and keep meeting on the same memory channels. */
+#ifndef NVSHMEMI_AMD_COPY_ROTATE
+#define NVSHMEMI_AMD_COPY_ROTATE 1
+#endif
+    size_t r = 0;
+    if (NVSHMEMI_AMD_COPY_ROTATE && rounds >= 8 && rounds <= 0xffffffffu) {
+        const unsigned h = (blockIdx.x * 0x9E3779B1u) ^ (blockIdx.y * 0x85EBCA77u) ^ (blockIdx.z * 0xC2B2AE3Du);
+        r = (size_t)(((uint64_t)h * (uint64_t)(rounds & 0xffffffffu)) >> 32);  /* in [0, rounds) */
+    }
+    for (size_t k = 0; k < rounds; ++k) {
+        const char *s = s0 + r * (16 * per_round);
+        char *d = d0 + r * (16 * per_round);
+        if (++r == rounds) r = 0;
         nvshmemi_v4u v[U];
 #pragma unroll
         for (int u = 0; u < U; ++u) v[u] = nvshmemi_amd_stream_load16<true, NT_LOAD>(s + u * 1024 + lane_off);

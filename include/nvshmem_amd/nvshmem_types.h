@@ -233,7 +233,7 @@ typedef struct nvshmemi_device_state {
     int32_t npes;
     uint32_t reserved;
     char *heap_base;      /* start of PE 0's slice */
-    uint64_t heap_size;   /* bytes from one PE's slice to the next (a multiple of 2 MiB) */
+    uint64_t heap_size;   /* bytes from one PE's slice to the next (a multiple of 2 MiB, of 16 MiB for large heaps) */
     uint64_t *sync_flags; /* canonical address: NVSHMEMI_AMD_MAX_PES arrival words per PE */
     uint64_t *sync_epoch; /* canonical address: that PE's barrier epoch */
     uint64_t spin_limit;  /* 0 = wait forever; else a bounded wait gives up after this many polls */

@@ -166,13 +166,15 @@ int nvshmemx_amd_init(int npes, size_t symmetric_size) {
     uint64_t want = symmetric_size < min_slice ? min_slice : (uint64_t)symmetric_size;
     // room for the runtime's own symmetric words (barrier row, epoch, timeout record)
     want += NVSHMEMI_AMD_INTERNAL_BYTES;
-    // slices start on 2 MiB boundaries (the granule of the GPU's large page fragments) and are no
-    // larger than asked for beyond that: the distance between them need not be a power of two
-    const uint64_t granule = 2ull << 20;
+    // The distance between slices is the size asked for rounded up to 16 MiB (2 MiB for small heaps),
+    // not to a power of two.  16 MiB multiples measured best for kernels that store one piece into
+    // many slices at equal offsets (fcollect of 16 x 16 MiB: 6.0-6.2 TB/s against 5.2-5.6 at distances
+    // that are odd multiples of 2 MiB); the copy engine and the reductions do not care.
     if (want > (1ull << 40)) {
         set_error("nvshmemx_amd_init: symmetric size %zu too large", symmetric_size);
         return NVSHMEMX_ERROR_INVALID_VALUE;
     }
+    const uint64_t granule = want > (16ull << 20) ? (16ull << 20) : (2ull << 20);
     const uint64_t slice_bytes = (want + granule - 1) / granule * granule;
     int dev = 0;
     if (hipGetDevice(&dev) != hipSuccess) {

@@ -50,7 +50,7 @@ struct Runtime {
     int device = 0;
     int npes = 0;
     int num_cus = 0;
-    uint64_t heap_size = 0;  // bytes from one PE's slice to the next, a multiple of 2 MiB
+    uint64_t heap_size = 0;  // bytes from one PE's slice to the next, a multiple of 2 MiB (16 MiB for large heaps)
     char *base = nullptr;    // start of PE 0's slice
     std::unique_ptr<SymmetricSpace> space;
     nvshmemi_device_state_t dev{};

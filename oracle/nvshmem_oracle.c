@@ -560,6 +560,51 @@ int oracle_space_free(oracle_space_t *s, uint64_t addr) {
     return -1;
 }
 
+/* reallocate (custom_malloc.cpp:198-229): the size is rounded like a request; the same rounded size
+ * returns the block; a smaller one keeps the front and frees the tail (:202-206); a larger one grows
+ * in place when the chunk right behind the block is free and the two together suffice (:208-219),
+ * else takes a fresh block by first fit and frees the old one (:221-226; the copy of the contents is
+ * the caller's business here, *moved_from names the old block).  NULL (0) when there is no room: the
+ * old block stays.
+ * One deviation is pinned on purpose.  In the in-place branch the reference returns
+ * `size - current_size` bytes at `ptr + size` to the free list (:216-217), not the real remainder
+ * `current_size + chunk_size - size`, so the rest of the consumed chunk is lost and the free chunk it
+ * creates can cover memory that is no chunk's at all.  The model (and the library) return the real
+ * remainder; tests/golden/allocator_traces.json holds a trace whose later steps tell the two apart.
+ * An address that is not a live block returns 0 (the reference would create a zero-size entry). */
+uint64_t oracle_space_realloc(oracle_space_t *s, uint64_t addr, uint64_t bytes, uint64_t *moved_from) {
+    if (moved_from) *moved_from = 0;
+    size_t i = 0;
+    while (i < s->n && !(s->b[i].addr == addr && s->b[i].used)) ++i;
+    if (i == s->n) return 0;
+    bytes = (bytes + 511) & ~(uint64_t)511;
+    const uint64_t cur = s->b[i].size;
+    if (bytes == cur || bytes == 0) return addr;
+    if (bytes < cur) {
+        s->b[i].size = bytes;
+        oracle_block_t tail = {addr + bytes, cur - bytes, 0};
+        space_insert(s, i + 1, tail);
+        space_merge_around(s, i + 1);
+        return addr;
+    }
+    if (i + 1 < s->n && !s->b[i + 1].used && s->b[i + 1].addr == addr + cur && cur + s->b[i + 1].size >= bytes) {
+        const uint64_t rest = cur + s->b[i + 1].size - bytes;
+        s->b[i].size = bytes;
+        if (rest) {
+            s->b[i + 1].addr = addr + bytes;
+            s->b[i + 1].size = rest;
+        } else {
+            space_remove(s, i + 1);
+        }
+        return addr;
+    }
+    const uint64_t fresh = oracle_space_alloc(s, bytes);
+    if (!fresh) return 0;
+    oracle_space_free(s, addr);
+    if (moved_from) *moved_from = addr;
+    return fresh;
+}
+
 uint64_t oracle_space_free_bytes(const oracle_space_t *s) {
     uint64_t t = 0;
     for (size_t i = 0; i < s->n; ++i) if (!s->b[i].used) t += s->b[i].size;

@@ -123,6 +123,7 @@ void oracle_space_destroy(oracle_space_t *s);
 uint64_t oracle_space_alloc(oracle_space_t *s, uint64_t bytes);
 uint64_t oracle_space_align(oracle_space_t *s, uint64_t alignment, uint64_t bytes);
 int oracle_space_free(oracle_space_t *s, uint64_t addr);
+uint64_t oracle_space_realloc(oracle_space_t *s, uint64_t addr, uint64_t bytes, uint64_t *moved_from);
 uint64_t oracle_space_free_bytes(const oracle_space_t *s);
 uint64_t oracle_space_free_chunks(const oracle_space_t *s);
 

@@ -64,6 +64,7 @@ def lib():
         "oracle_space_alloc": (u64, [vp, u64]),
         "oracle_space_align": (u64, [vp, u64, u64]),
         "oracle_space_free": (i32, [vp, u64]),
+        "oracle_space_realloc": (u64, [vp, u64, u64, vp]),
         "oracle_space_free_bytes": (u64, [vp]),
         "oracle_space_free_chunks": (u64, [vp]),
         "oracle_moe_routing": (None, [vp, i32, i32, i32, C.c_double, u64, u64]),

@@ -60,6 +60,11 @@ class Model:
     def free(self, addr):
         return self.L.oracle_space_free(self.h, addr)
 
+    def realloc(self, addr, n):
+        moved = C.c_uint64(0)
+        r = self.L.oracle_space_realloc(self.h, addr, n, C.byref(moved))
+        return r, moved.value
+
     def free_bytes(self):
         return self.L.oracle_space_free_bytes(self.h)
 
@@ -81,6 +86,10 @@ def _replay(impl_cls, trace):
             elif st["op"] == "align":
                 got = impl.align(st["alignment"], st["bytes"])
                 got = got - base if got else -1
+            elif st["op"] == "realloc":
+                got, moved = impl.realloc(base + st["addr"], st["bytes"])
+                got = got - base if got else -1
+                assert (moved - base if moved else -1) == st["moved"], "%s step %d %r moved %d" % (trace["name"], i, st, moved)
             else:
                 got = impl.free(base + st["addr"])
             assert got == st["expect"], "%s step %d %r -> %d" % (trace["name"], i, st, got)
@@ -116,6 +125,13 @@ def test_differential_random_traces(seed):
                 if pa:
                     assert pa % 512 == 0 or pa % 8 == 0
                     live.append(pa)
+            elif r < 0.65:
+                k = int(rng.integers(0, len(live)))
+                n = int(rng.choice([1, 300, 512, 2000, 4096, 50000, 200000]))
+                (pa, ma), (pb, mb) = a.realloc(live[k], n), b.realloc(live[k], n)
+                assert (pa, ma) == (pb, mb), (step, n)
+                if pa:
+                    live[k] = pa
             else:
                 addr = live.pop(int(rng.integers(0, len(live))))
                 assert a.free(addr) == 0 and b.free(addr) == 0

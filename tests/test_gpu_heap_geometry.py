@@ -1,5 +1,5 @@
-"""Heap geometry: the distance between PE slices is the requested size rounded up to 2 MiB, not to a
-power of two (a2: PE -> address translation on such a heap)."""
+"""Heap geometry: the distance between PE slices is the requested size rounded up to 16 MiB (2 MiB for
+small heaps), not to a power of two (a2: PE -> address translation on such a heap)."""
 import numpy as np
 import pytest
 
@@ -11,14 +11,14 @@ pytestmark = pytest.mark.gpu
 
 
 def test_heap_whose_size_is_no_power_of_two():
-    """NVSHMEM_SYMMETRIC_SIZE = 96 MiB + 12345 bytes on 5 PEs: the slices are 98 MiB apart (no rounding to
+    """NVSHMEM_SYMMETRIC_SIZE = 96 MiB + 12345 bytes on 5 PEs: the slices are 112 MiB apart (no rounding to
     128 MiB), translation, ring put / get and an allreduce work as on any other heap."""
     npes, want_size = 5, (96 << 20) + 12345
     with runtime(npes, want_size) as r:
         perf = r.perftest()
         a = r.malloc(1 << 20)
         stride = r.ptr(a, 1) - r.ptr(a, 0)
-        assert stride == 98 << 20
+        assert stride == 112 << 20
         assert r.ptr(r.ptr(a, 4) + 5, 2) == a + 5 + 2 * stride        # any PE's copy names the object
         assert r.ptr(a + npes * stride, 0) is None
         r.free(a)

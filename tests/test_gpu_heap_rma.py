@@ -47,8 +47,8 @@ def test_malloc_ptr_translation_matches_closed_form(rt):
     b = rt.malloc(1)
     assert a % 512 == 0 and b == a + 1024          # 512-byte granules, first fit
     heap_size = rt.ptr(a, 1) - rt.ptr(a, 0)
-    # slices are 2 MiB-aligned and no larger than asked for beyond that (no rounding to a power of two)
-    assert (1 << 30) <= heap_size <= (1 << 30) + (2 << 20) and heap_size % (2 << 20) == 0
+    # slices are 16 MiB-aligned and no larger than asked for beyond that (no rounding to a power of two)
+    assert (1 << 30) <= heap_size <= (1 << 30) + (16 << 20) and heap_size % (16 << 20) == 0
     assert rt.ptr(a, 0) == a                       # canonical address is PE 0's copy
     L = O.lib()
     for pe in range(NPES):
