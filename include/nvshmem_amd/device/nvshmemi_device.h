@@ -1291,6 +1291,163 @@ NVSHMEMI_DEVICE_INLINE unsigned nvshmemi_amd_ll_reduce_group(size_t nbytes, int 
 }
 
 /* ------------------------------------------------------------------------------------------------
+ * Line packets: the reference's LL128 (128-byte lines with one flag word,
+ * non_abi/device/common/nvshmemi_common_device.cuh:699-920, used by coll/fcollect.cuh:157-314)
+ * re-derived for this GPU.
+ *
+ * The unit is HALF a cache line: 64 bytes = 56 bytes of payload and an 8-byte flag word, written by
+ * four adjacent lanes with one 16-byte agent-scope store each - lane k of the four carries payload
+ * bytes [16 k, 16 k + 16), the last lane 8 bytes and the flag.  The compute unit sends a wavefront's
+ * stores to the L2 as 64-byte requests and the L2 writes them through as 64-byte requests, so a unit
+ * travels as one write and a receiver that finds the flag finds the payload (the protocol assumes
+ * that such a write is not torn; tests stream changing data through it and check every unit).  A
+ * 128-byte line with ONE flag would need the two requests of a line to arrive together, which nothing
+ * promises here.  56 bytes are a whole number of elements of every type, so a lane folds whole
+ * elements.  Efficiency 7/8 against the 1/2 of the 16-byte packets, and a block of 256 threads covers
+ * 3.5 KiB per member with one unit-lane per thread.
+ *
+ * Allreduce / reducescatter in one hop, no barrier: thread (u, k) - unit u, lane k - sends its 16
+ * bytes of the PE's contribution to every other member's buffer (slot `me`), then fetches the same
+ * position of every member's slot in its own buffer, all loads issued before the first check; the
+ * wavefront repeats the batch until every unit it covers carries the call's flag, and the lane folds
+ * its elements in member order and stores them.  Flags, buffer rotation and the `done` word are those
+ * of the 16-byte packets above (the two formats share the buffers: a stale word of the other format
+ * cannot equal a later call's flag word).
+ * ---------------------------------------------------------------------------------------------- */
+#define NVSHMEMI_AMD_UNIT_BYTES 64
+#define NVSHMEMI_AMD_UNIT_PAYLOAD 56
+NVSHMEMI_DEVICE_INLINE unsigned nvshmemi_amd_units(size_t nbytes) {
+    return (unsigned)((nbytes + NVSHMEMI_AMD_UNIT_PAYLOAD - 1) / NVSHMEMI_AMD_UNIT_PAYLOAD);
+}
+/* one unit-lane per thread, all members' slots in one buffer, buffers at hand */
+template <int SCOPE>
+NVSHMEMI_DEVICE_INLINE bool nvshmemi_amd_units_fit(size_t nbytes, int npes) {
+    const size_t units = (nbytes + NVSHMEMI_AMD_UNIT_PAYLOAD - 1) / NVSHMEMI_AMD_UNIT_PAYLOAD;
+    const size_t nthr = (size_t)nvshmemi_threadgroup_size<SCOPE>();
+    return SCOPE != NVSHMEMI_THREADGROUP_THREAD && nbytes > 0 && nvshmemi_amd_ll_available() && (nthr & 3) == 0 &&
+           4 * units <= nthr && (size_t)npes * units * NVSHMEMI_AMD_UNIT_BYTES <= 2 * (size_t)NVSHMEMI_AMD_LL_PAYLOAD_BYTES;
+}
+/* the 16 bytes lane k of unit u carries: payload from src (zeros behind its end), for k == 3 the flag word on top */
+NVSHMEMI_DEVICE_INLINE nvshmemi_v4u nvshmemi_amd_unit_pack(const char *src, size_t nbytes, unsigned u, unsigned k,
+                                                           uint32_t flag) {
+    const size_t at = (size_t)u * NVSHMEMI_AMD_UNIT_PAYLOAD + 16 * k;
+    const size_t want = k == 3 ? 8 : 16;
+    nvshmemi_v4u x = {0, 0, 0, 0};
+    if (at + want <= nbytes) {
+        if (k == 3) {
+            uint64_t w;
+            __builtin_memcpy(&w, src + at, 8);
+            x.x = (uint32_t)w;
+            x.y = (uint32_t)(w >> 32);
+        } else {
+            x = nvshmemi_amd_load16<false>(src + at);
+        }
+    } else if (at < nbytes) {
+        unsigned char b[16] = {0};
+        for (size_t i = 0; at + i < nbytes && i < want; ++i) b[i] = (unsigned char)src[at + i];
+        __builtin_memcpy(&x, b, 16);
+    }
+    if (k == 3) {
+        x.z = flag;
+        x.w = flag;
+    }
+    return x;
+}
+template <typename T, int OP, int SCOPE, bool SCATTER>
+NVSHMEMI_DEVICE_INLINE void nvshmemi_amd_unit_reduce(nvshmem_team_t team, const nvshmemi_amd_team_view_t &tv, T *dest,
+                                                     const T *source, size_t nreduce) {
+    constexpr size_t VEC = 16 / sizeof(T);
+    union pack_t {
+        nvshmemi_v4u v;
+        T e[VEC];
+    };
+    const int me = tv.my_pe, npes = tv.size;
+    const unsigned tid = (unsigned)nvshmemi_thread_id_in_threadgroup<SCOPE>();
+    const size_t nbytes = nreduce * sizeof(T);
+    const unsigned units = nvshmemi_amd_units(nbytes);
+    const unsigned u = tid >> 2, k = tid & 3;
+    const bool active = u < units;
+    const uint32_t flag = nvshmemi_amd_ll_next_flag<SCOPE>(team);
+    const char *src_all = nvshmemi_amd_local(source);
+    /* SCATTER: member idx is sent block idx of the source and folds the blocks `me` it receives */
+    const size_t slot_off = ((size_t)me * units + u) * NVSHMEMI_AMD_UNIT_BYTES + 16 * k;
+    if (active) {
+        const nvshmemi_v4u same = SCATTER ? nvshmemi_v4u{0, 0, 0, 0} : nvshmemi_amd_unit_pack(src_all, nbytes, u, k, flag);
+        for (int off = 1; off < npes; ++off) {
+            const int idx = me + off < npes ? me + off : me + off - npes;
+            const nvshmemi_v4u x = SCATTER ? nvshmemi_amd_unit_pack(src_all + (size_t)idx * nbytes, nbytes, u, k, flag) : same;
+            nvshmemi_amd_store16_agent(nvshmemi_amd_ll_buffer(team, nvshmemi_amd_team_pe(tv, idx), flag) + slot_off, x);
+        }
+    }
+    /* (dest may be source: a lane stores only the bytes whose source it has read itself) */
+    const char *mine = nvshmemi_amd_ll_buffer(team, nvshmemi_amd_my_pe(), flag);
+    const size_t at = (size_t)u * NVSHMEMI_AMD_UNIT_PAYLOAD + 16 * k;
+    const uint64_t limit = nvshmemi_device_state_d.spin_limit;
+    pack_t acc;
+    acc.v = nvshmemi_v4u{0, 0, 0, 0};
+    for (int p0 = 0; p0 < npes; p0 += 8) {
+        pack_t x[8];
+#pragma unroll
+        for (int q = 0; q < 8; ++q) x[q].v = nvshmemi_v4u{0, 0, 0, 0};
+        uint64_t polls = 0;
+        for (;;) {
+            bool missing = false;
+#pragma unroll
+            for (int q = 0; q < 8; ++q) {
+                const int p = p0 + q;
+                if (active && p < npes && p != me) {
+                    const char *from = mine + ((size_t)p * units + u) * NVSHMEMI_AMD_UNIT_BYTES + 16 * k;
+                    asm volatile("global_load_dwordx4 %0, %1, off sc1" : "=v"(x[q].v) : "v"(from) : "memory");
+                }
+            }
+            /* the registers are operands so that no use of them moves in front of the wait */
+            asm volatile("s_waitcnt vmcnt(0)"
+                         : "+v"(x[0].v), "+v"(x[1].v), "+v"(x[2].v), "+v"(x[3].v), "+v"(x[4].v), "+v"(x[5].v),
+                           "+v"(x[6].v), "+v"(x[7].v)
+                         :
+                         : "memory");
+#pragma unroll
+            for (int q = 0; q < 8; ++q) {
+                const int p = p0 + q;
+                if (active && k == 3 && p < npes && p != me) missing |= x[q].v.z != flag || x[q].v.w != flag;
+            }
+            if (!__builtin_amdgcn_ballot_w64(missing)) break;
+            if (limit && ++polls > limit) {
+                if (missing) nvshmemi_amd_record_timeout(mine, 0, flag);
+                break;
+            }
+            __builtin_amdgcn_s_sleep(1);
+        }
+        if (active) {
+#pragma unroll
+            for (int q = 0; q < 8; ++q) {
+                const int p = p0 + q;
+                if (p >= npes) break;
+                if (p == me) x[q].v = nvshmemi_amd_unit_pack(src_all + (SCATTER ? (size_t)me * nbytes : 0), nbytes, u, k, flag);
+                if (p == 0) {
+                    acc = x[q];
+                } else {
+#pragma unroll
+                    for (size_t e = 0; e < VEC; ++e)
+                        acc.e[e] = SCATTER ? nvshmemi_amd_reduce_op<T, OP>(acc.e[e], x[q].e[e])
+                                           : nvshmemi_amd_fold_step<T, OP>(p, acc.e[e], x[q].e[e]);
+                }
+            }
+        }
+    }
+    if (active && at < nbytes) {
+        char *dst = nvshmemi_amd_local(dest) + at;
+        const size_t room = (k == 3 ? 8 : 16), left = nbytes - at < room ? nbytes - at : room;
+        if (left == 16 && (((uintptr_t)dst) & 15) == 0) {
+            *reinterpret_cast<nvshmemi_v4u *>(dst) = acc.v;
+        } else {
+            for (size_t e = 0; e * sizeof(T) < left; ++e) reinterpret_cast<T *>(dst)[e] = acc.e[e];
+        }
+    }
+    nvshmemi_amd_ll_publish_done<SCOPE>(team, flag);
+}
+
+/* ------------------------------------------------------------------------------------------------
  * Collectives called from inside a user kernel, one thread group per PE
  * (reference coll/reduce.cuh:1158-1196 get-based reduce, coll/fcollect.cuh:331-344,
  * coll/alltoall.cuh:122-143).  Calls small enough for the packets above return when the caller's
@@ -1498,6 +1655,11 @@ NVSHMEMI_DEVICE_INLINE int nvshmemi_reduce_threadgroup(nvshmem_team_t team, T *d
     const size_t nthr = (size_t)nvshmemi_threadgroup_size<SCOPE>();
     if (const unsigned group = nvshmemi_amd_ll_reduce_group<SCOPE>(nreduce * sizeof(T), npes)) {
         nvshmemi_amd_ll_reduce<T, OP, SCOPE>(team, tv, dest, source, nreduce, group);
+        return 0;
+    }
+    if ((nvshmemi_device_state_d.options & NVSHMEMI_AMD_OPTION_UNIT_PACKETS) &&
+        nvshmemi_amd_units_fit<SCOPE>(nreduce * sizeof(T), npes)) {
+        nvshmemi_amd_unit_reduce<T, OP, SCOPE, false>(team, tv, dest, source, nreduce);
         return 0;
     }
     if (nvshmemi_amd_staged_fits<SCOPE, false>(dest, source, nreduce * sizeof(T), npes)) {
@@ -1777,6 +1939,11 @@ NVSHMEMI_DEVICE_INLINE int nvshmemi_reducescatter_threadgroup(nvshmem_team_t tea
     const size_t nthr = (size_t)nvshmemi_threadgroup_size<SCOPE>();
     if (const unsigned group = nvshmemi_amd_ll_reduce_group<SCOPE>(nreduce * sizeof(T), npes)) {
         nvshmemi_amd_ll_reduce<T, OP, SCOPE, true>(team, tv, dest, source, nreduce, group);
+        return 0;
+    }
+    if ((nvshmemi_device_state_d.options & NVSHMEMI_AMD_OPTION_UNIT_PACKETS) &&
+        nvshmemi_amd_units_fit<SCOPE>(nreduce * sizeof(T), npes)) {
+        nvshmemi_amd_unit_reduce<T, OP, SCOPE, true>(team, tv, dest, source, nreduce);
         return 0;
     }
     if (nvshmemi_amd_staged_fits<SCOPE, true>(dest, source, nreduce * sizeof(T), npes)) {
