@@ -260,6 +260,10 @@ def main():
     ap.add_argument("--warmup", type=int, default=5)
     ap.add_argument("--cpu-seconds", type=float, default=1.5, help="CPU oracle timing budget per workload")
     ap.add_argument("--only", default="", help="comma-separated workload names (the headline always runs)")
+    ap.add_argument("--trace-manifest", default="",
+                    help="for runs under rocprofv3: bracket every workload's launches with the empty "
+                         "profile_marker_kernel and write the order of the workloads to this file, so that "
+                         "nvshmem_amd/profile_summary.py can cut the kernel trace into workloads")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this build runs all logical PEs on ONE GPU; --gpus %d is not supported "
@@ -279,7 +283,7 @@ def main():
     if only:
         only.add(workloads.HEADLINE)
     check = Checker(O, np, args.cpu_seconds)
-    results = {}
+    results, manifest = {}, []
     groups = workloads.all_groups(oracle_moe_plan(O, np, 8, 8192, 8, 256))
     for g in groups:
         if only and not any(n in only for n in g.names()):
@@ -291,7 +295,14 @@ def main():
                     continue
                 getattr(check, g.kind + "_prepare")(g, item)
                 steps, warmup = max(1, args.steps // item.scale), max(1, args.warmup // item.scale)
+                if args.trace_manifest:
+                    rt.perftest().nvshmem_perftest_profile_marker(None)
                 wall, ev = time_steps(item.step, steps, warmup, hip)
+                if args.trace_manifest:
+                    rt.perftest().nvshmem_perftest_profile_marker(None)
+                    hip.synchronize()
+                    manifest.append({"name": item.name, "launches": steps + warmup, "workload": item.workload,
+                                     "algorithmic_bytes": item.algorithmic_bytes})
                 ok = getattr(check, g.kind + "_verify")(g, item)
                 cpu = getattr(check, g.kind + "_baseline")(g, item)
                 results[item.name] = summarise(item, wall, ev, ok, cpu)
@@ -299,6 +310,9 @@ def main():
         finally:
             rt.finalize()
 
+    if args.trace_manifest:
+        with open(args.trace_manifest, "w") as fh:
+            json.dump(manifest, fh, indent=1)
     head = results[workloads.HEADLINE]
     line = {
         "metric": METRIC,

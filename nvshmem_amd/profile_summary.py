@@ -109,6 +109,8 @@ def main():
     ap.add_argument("--pmc", action="append", default=[])
     ap.add_argument("--profiles-dir")
     ap.add_argument("--only", default="")
+    ap.add_argument("--table", default="", help="also write a one-line-per-workload table of the kernel trace there")
+    ap.add_argument("--table-title", default="", help="first lines of that table")
     args = ap.parse_args()
     manifest = json.load(open(args.manifest))
     only = set(x for x in args.only.split(",") if x)
@@ -123,6 +125,20 @@ def main():
             for c in ("FETCH_SIZE", "WRITE_SIZE"):
                 if c in cs and cs[c] > 0:
                     scale[c] = CALIBRATION_KIB / cs[c]
+    if args.table:
+        rows = [args.table_title.replace("\\n", "\n"), "",
+                "%-28s %-48s %6s %11s %11s %11s %9s" % ("workload", "dominant kernel", "calls", "avg us", "min us", "max us",
+                                                       "GB/s")]
+        for entry in manifest:
+            st = stats_of(kwin.get(entry["name"], []))
+            if not st:
+                continue
+            k = max(st, key=lambda k: st[k][0] * st[k][1])
+            calls, avg, lo, hi = st[k][:4]
+            rows.append("%-28s %-48s %6d %11.2f %11.2f %11.2f %9.0f" % (entry["name"], k[:48], calls, avg, lo, hi,
+                                                                      entry.get("algorithmic_bytes", 0) / avg / 1e3))
+        with open(args.table, "w") as fh:
+            fh.write("\n".join(rows) + "\n")
     for entry in manifest:
         name = entry["name"]
         if only and name not in only:
