@@ -190,10 +190,7 @@ typedef nvshmemi_v4u __attribute__((aligned(1))) nvshmemi_v4u_unaligned;
  * and a write to the registers that hold the store's data, so the s_nop supplies it (without it a
  * following address computation that reused the data registers corrupted the stored value). */
 NVSHMEMI_DEVICE_INLINE void nvshmemi_amd_store16_agent(char *p, nvshmemi_v4u v) {
-#ifndef NVSHMEMI_AMD_AGENT_STORE_MODS
-#define NVSHMEMI_AMD_AGENT_STORE_MODS "sc1"
-#endif
-    asm volatile("global_store_dwordx4 %0, %1, off " NVSHMEMI_AMD_AGENT_STORE_MODS "\n\ts_nop 1" : : "v"(p), "v"(v) : "memory");
+    asm volatile("global_store_dwordx4 %0, %1, off sc1\n\ts_nop 1" : : "v"(p), "v"(v) : "memory");
 }
 
 template <bool SRC_ALIGNED>

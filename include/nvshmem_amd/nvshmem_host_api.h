@@ -90,8 +90,9 @@ NVSHMEMI_HOST_ONLY void nvshmemx_vendor_get_version_info(int *major, int *minor,
 
 /*
  * Logical-PE bring-up (stands where the reference's nvshmemx_init_attr + bootstrap sit,
- * src/include/host/nvshmemx_api.h:52-66): npes PEs with symmetric_size bytes each (rounded up to a
- * power of two).  nvshmem_init() calls it with NVSHMEM_AMD_NPES (default 8) and
+ * src/include/host/nvshmemx_api.h:52-66): npes PEs with symmetric_size bytes each (the distance
+ * between two PEs' slices is that size plus 2 KiB of runtime words, rounded up to 16 MiB, or to 2 MiB for
+ * heaps of at most 16 MiB).  nvshmem_init() calls it with NVSHMEM_AMD_NPES (default 8) and
  * NVSHMEM_SYMMETRIC_SIZE (default 1 GiB; reference src/include/host/env/env_defs.h).
  * Returns an nvshmemx_status.
  */

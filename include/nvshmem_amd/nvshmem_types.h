@@ -186,8 +186,9 @@ typedef enum {
 /*
  * State block read by device code (counterpart of the reference's nvshmemi_device_host_state_t,
  * src/include/device_host/nvshmem_types.h:452-509).  All logical PEs live in one allocation:
- * PE p owns [heap_base + p*heap_size, heap_base + (p+1)*heap_size), heap_size is a power of two,
- * so the reference's peer_heap_base_p2p[] table collapses to a shift.  Symmetric addresses handed
+ * PE p owns [heap_base + p*heap_size, heap_base + (p+1)*heap_size), heap_size being the distance
+ * between slices (a multiple of 2 MiB, of 16 MiB for large heaps; no power of two), so the
+ * reference's peer_heap_base_p2p[] table collapses to a multiplication.  Symmetric addresses handed
  * to users are addresses inside PE 0's slice ("canonical" addresses).
  */
 /* Team `t` as PE `p` sees it: entry [t * NVSHMEMI_AMD_MAX_PES + p] of the team table.  The

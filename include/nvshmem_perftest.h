@@ -51,6 +51,13 @@ int nvshmem_perftest_profile_marker(void *stream);
  * out[q] of its own `out`.  words and out hold npes uint64 each. */
 int nvshmem_perftest_p_g(uint64_t *words, uint64_t *out, uint64_t value_base, void *stream);
 
+/* The PE identity rule of the device API (the reference's nvshmem_my_pe reads the per-process
+ * nvshmemi_device_state_d.mype, src/include/device/nvshmem_defines.h:55-57):
+ * a launch of grid (1, 1, grid_z) with one thread per block writes nvshmem_my_pe() of block z to out[z]
+ * and nvshmem_n_pes() to out[64 + z].  `out` is any device memory of 128 ints.  A grid whose z extent
+ * equals the PE count is a PE grid (block z acts as PE z); any other z extent acts as PE 0. */
+int nvshmem_perftest_pe_identity(int *out, int grid_z, void *stream);
+
 /* Each of `threads` threads of one block per PE applies nvshmemx_signal_op(sig, value, sig_op,
  * (p+1)%npes) `reps` times. */
 int nvshmem_perftest_signal_op(uint64_t *sig, uint64_t value, int sig_op, int threads, int reps,

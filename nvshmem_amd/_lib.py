@@ -132,6 +132,7 @@ def load_perftest():
         "nvshmem_perftest_plain_copy": [vp, vp, sz, vp],
         "nvshmem_perftest_profile_marker": [vp],
         "nvshmem_perftest_p_g": [vp, vp, u64, vp],
+        "nvshmem_perftest_pe_identity": [vp, i32, vp],
         "nvshmem_perftest_api_matrix": [vp, vp, vp, vp, vp, i32, vp],
         "nvshmem_perftest_signal_op": [vp, u64, i32, i32, i32, vp],
         "nvshmem_perftest_signal_wait": [vp, i32, u64, vp, vp],

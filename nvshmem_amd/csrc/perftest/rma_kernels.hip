@@ -70,6 +70,12 @@ __global__ void p_g_kernel(uint64_t *words, uint64_t *out, uint64_t value_base) 
     for (int q = 0; q < np; ++q) mine[q] = nvshmem_uint64_g(words + (q + np - 1) % np, q);
 }
 
+// out is plain device memory here (used as it is): [z] = the PE block z acts as, [64 + z] = nvshmem_n_pes()
+__global__ void pe_identity_kernel(int *out) {
+    out[blockIdx.z] = nvshmem_my_pe();
+    out[64 + blockIdx.z] = nvshmem_n_pes();
+}
+
 __global__ void signal_op_kernel(uint64_t *sig, uint64_t value, int sig_op, int reps) {
     const int peer = (nvshmem_my_pe() + 1) % nvshmem_n_pes();
     for (int r = 0; r < reps; ++r) nvshmemx_signal_op(sig, value, sig_op, peer);
@@ -403,6 +409,12 @@ int nvshmem_perftest_p_g(uint64_t *words, uint64_t *out, uint64_t value_base, vo
     void *args[] = {&words, &out, &value_base};
     return nvshmemx_collective_launch((const void *)p_g_kernel, dim3(1), dim3(1), args, 0,
                                       (hipStream_t)stream);
+}
+
+int nvshmem_perftest_pe_identity(int *out, int grid_z, void *stream) {
+    if (!perftest::ready() || !out || grid_z < 1 || grid_z > 64) return NVSHMEMX_ERROR_INVALID_VALUE;
+    hipLaunchKernelGGL(pe_identity_kernel, dim3(1, 1, (unsigned)grid_z), dim3(1), 0, (hipStream_t)stream, out);
+    return perftest::launch_status("pe_identity");
 }
 
 int nvshmem_perftest_signal_op(uint64_t *sig, uint64_t value, int sig_op, int threads, int reps,

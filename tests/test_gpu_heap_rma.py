@@ -42,6 +42,26 @@ def test_identity_and_versions(rt):
     rt.free(buf)
 
 
+def test_pe_identity_follows_grid_z(rt):
+    """The one rule that makes a block a PE: a grid whose z extent equals the PE count is a PE grid (block z
+    acts as PE z); a kernel launched with any other z extent acts as PE 0 whatever its block index, so a
+    kernel that is not meant as a PE kernel must not use z == npes while it calls the device API."""
+    perf = rt.perftest()
+    out = rt.malloc(128 * 4)       # plain device memory for this kernel: PE 0's copy, used untranslated
+    for grid_z in (NPES, 1, 3, NPES - 1, NPES + 1, 2 * NPES):
+        note("pe identity, grid z", grid_z)
+        rt.fill(out, 0xFF, 128 * 4)
+        assert perf.nvshmem_perftest_pe_identity(out, grid_z, None) == 0
+        rt.sync()
+        got = rt.download(out, 0, (128,), np.int32)
+        want = np.arange(grid_z) if grid_z == NPES else np.zeros(grid_z, dtype=np.int32)
+        assert np.array_equal(got[:grid_z], want), (grid_z, got[:grid_z])
+        assert np.all(got[64:64 + grid_z] == NPES)
+        assert np.all(got[grid_z:64] == -1)
+    assert perf.nvshmem_perftest_pe_identity(out, 0, None) != 0
+    rt.free(out)
+
+
 def test_malloc_ptr_translation_matches_closed_form(rt):
     a = rt.malloc(1000)
     b = rt.malloc(1)
