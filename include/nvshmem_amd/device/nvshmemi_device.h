@@ -206,7 +206,9 @@ NVSHMEMI_DEVICE_INLINE nvshmemi_v4u nvshmemi_amd_stream_load16(const char *p) {
 }
 /* Where the stores of a copy go: streamed (non-temporal; the lines stay dirty in this XCD's L2 until
  * they are evicted or a release writes the L2 back) or written through the L2 to memory at agent scope,
- * which leaves nothing for a later release to write back. */
+ * which leaves nothing for a later release to write back.  (Write-through as the default of plain
+ * copies was measured too, as sc1 and as sc1 nt: +1.5 % when one-wavefront blocks fill the GPU, -3..4 %
+ * for a few 1024-thread blocks per PE, so plain copies keep nt.) */
 enum nvshmemi_amd_store_policy_t { NVSHMEMI_AMD_STORE_STREAM = 0, NVSHMEMI_AMD_STORE_WRITE_THROUGH = 1 };
 
 template <int STORE = NVSHMEMI_AMD_STORE_STREAM>

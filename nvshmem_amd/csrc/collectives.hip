@@ -61,9 +61,42 @@ __device__ __forceinline__ nvshmemi_v4u stream_load(const char *p) {
         return __builtin_nontemporal_load(reinterpret_cast<const nvshmemi_v4u *>(p));
     return *reinterpret_cast<const nvshmemi_v4u *>(p);
 }
+// How a kernel's result stores treat the caches.  All three stream (nothing here reads its output back);
+// they differ in where the line waits for memory.  Write-through stores (sc1) leave the L2 at once
+// instead of queuing behind its eviction of streaming lines: a write-only stream reaches 7.2 TB/s with
+// them against 6.3 TB/s with nt alone.  Which form wins depends on the kernel's mix (measured on MI355X,
+// random data): sc1 nt +4.5 % for the 8-member allreduce, +5..10 % for fcollect and cache-resident
+// broadcast, +1..3 % for alltoall and the gather allreduce; plain sc1 +5 % for the reducescatter, whose
+// one store per eight loads gains nothing from nt; and the kernels whose blocks share a piece through
+// the cache (destinations split over neighbouring blocks) lose 9..15 % with either, so they keep nt.
+enum { kStoreStream = 0 /* nt */, kStoreThrough = 1 /* sc1 */, kStoreThroughStream = 2 /* sc1 nt */ };
+#ifndef NVSHMEM_AMD_STORE_ALLTOALL
+#define NVSHMEM_AMD_STORE_ALLTOALL kStoreThroughStream
+#endif
+#ifndef NVSHMEM_AMD_STORE_REPLICATE /* fcollect and broadcast, one wavefront storing to every member */
+#define NVSHMEM_AMD_STORE_REPLICATE kStoreThroughStream
+#endif
+#ifndef NVSHMEM_AMD_STORE_REPLICATE_SPLIT /* the same with the members split over neighbouring blocks */
+#define NVSHMEM_AMD_STORE_REPLICATE_SPLIT kStoreStream
+#endif
+#ifndef NVSHMEM_AMD_STORE_REDUCE
+#define NVSHMEM_AMD_STORE_REDUCE kStoreThroughStream
+#endif
+#ifndef NVSHMEM_AMD_STORE_REDUCESCATTER
+#define NVSHMEM_AMD_STORE_REDUCESCATTER kStoreThrough
+#endif
+// The asm forms end in s_nop 1: the compiler does not know the statement is a store of more than 8 bytes
+// and would not keep the wait state this GPU needs before the data registers are written again.
+template <int STORE>
 __device__ __forceinline__ void stream_store(char *p, nvshmemi_v4u v) {
-    if (NVSHMEM_AMD_COLL_NT & 2) __builtin_nontemporal_store(v, reinterpret_cast<nvshmemi_v4u *>(p));
-    else *reinterpret_cast<nvshmemi_v4u *>(p) = v;
+    if (STORE == kStoreThrough)
+        asm volatile("global_store_dwordx4 %0, %1, off sc1\n\ts_nop 1" : : "v"(p), "v"(v) : "memory");
+    else if (STORE == kStoreThroughStream)
+        asm volatile("global_store_dwordx4 %0, %1, off sc1 nt\n\ts_nop 1" : : "v"(p), "v"(v) : "memory");
+    else if (NVSHMEM_AMD_COLL_NT & 2)
+        __builtin_nontemporal_store(v, reinterpret_cast<nvshmemi_v4u *>(p));
+    else
+        *reinterpret_cast<nvshmemi_v4u *>(p) = v;
 }
 
 // ---------------------------------------------------------------------------------------------
@@ -81,7 +114,7 @@ enum { kModeFcollect = 0, kModeAlltoall = 1, kModeBroadcast = 2 };
 
 // Copies the vectors v0 + t + u*kCopyThreads (u < unroll) that fall inside [0, nvec); indices in front of
 // the segment wrap to huge unsigned values and are skipped the same way as those behind it.
-template <bool SRC_ALIGNED, bool REPLICATE, int kCopyUnroll, bool NTL>
+template <bool SRC_ALIGNED, bool REPLICATE, int kCopyUnroll, bool NTL, int STORE>
 __device__ __forceinline__ void copy_tile(char *__restrict__ dst, const char *__restrict__ src,
                                           uint64_t v0, uint64_t nvec, uint64_t rep_stride, int r0,
                                           int r1) {
@@ -97,19 +130,19 @@ __device__ __forceinline__ void copy_tile(char *__restrict__ dst, const char *__
 #pragma unroll
             for (int u = 0; u < kCopyUnroll; ++u) {
                 const uint64_t i = v0 + threadIdx.x + (uint64_t)u * kCopyThreads;
-                if (i < nvec) stream_store(d + 16 * i, v[u]);
+                if (i < nvec) stream_store<STORE>(d + 16 * i, v[u]);
             }
         }
     } else {
 #pragma unroll
         for (int u = 0; u < kCopyUnroll; ++u) {
             const uint64_t i = v0 + threadIdx.x + (uint64_t)u * kCopyThreads;
-            if (i < nvec) stream_store(dst + 16 * i, v[u]);
+            if (i < nvec) stream_store<STORE>(dst + 16 * i, v[u]);
         }
     }
 }
 
-template <int MODE, int kCopyUnroll, bool NTL>
+template <int MODE, int kCopyUnroll, bool NTL, int STORE>
 __global__ __launch_bounds__(kCopyThreads) void segment_copy_kernel(char *base, uint64_t slice_bytes,
                                                                 const nvshmemi_amd_team_view_t *groups,
                                                                 int max_size, uint64_t dst_off,
@@ -172,11 +205,11 @@ __global__ __launch_bounds__(kCopyThreads) void segment_copy_kernel(char *base, 
         const int per = (nrep + (1 << part_shift) - 1) >> part_shift;
         const int r0 = (int)(blockIdx.x & ((1u << part_shift) - 1)) * per;
         const int r1 = r0 + per < nrep ? r0 + per : nrep;
-        if (aligned) copy_tile<true, true, kCopyUnroll, NTL>(d, s, v0, nvec_total, rep_stride, r0, r1);
-        else copy_tile<false, true, kCopyUnroll, NTL>(d, s, v0, nvec_total, rep_stride, r0, r1);
+        if (aligned) copy_tile<true, true, kCopyUnroll, NTL, STORE>(d, s, v0, nvec_total, rep_stride, r0, r1);
+        else copy_tile<false, true, kCopyUnroll, NTL, STORE>(d, s, v0, nvec_total, rep_stride, r0, r1);
     } else {
-        if (aligned) copy_tile<true, false, kCopyUnroll, NTL>(d, s, v0, nvec_total, rep_stride, 0, 1);
-        else copy_tile<false, false, kCopyUnroll, NTL>(d, s, v0, nvec_total, rep_stride, 0, 1);
+        if (aligned) copy_tile<true, false, kCopyUnroll, NTL, STORE>(d, s, v0, nvec_total, rep_stride, 0, 1);
+        else copy_tile<false, false, kCopyUnroll, NTL, STORE>(d, s, v0, nvec_total, rep_stride, 0, 1);
     }
 }
 
@@ -251,7 +284,7 @@ __global__ __launch_bounds__(NPES ? NPES * 64 : 1024) void reduce_vector_kernel(
         for (int u = 0; u < VPT; ++u) {
             const uint64_t v = v0 + ((uint64_t)u << lane_shift);
             const nvshmemi_v4u r = result[((unsigned)u << lane_shift) + i];
-            if (v < nvec && member) stream_store(base + (uint64_t)pe * pe_stride + dst_off + 16 * v, r);
+            if (v < nvec && member) stream_store<NVSHMEM_AMD_STORE_REDUCE>(base + (uint64_t)pe * pe_stride + dst_off + 16 * v, r);
         }
     }
     // elements behind the last full vector
@@ -314,7 +347,7 @@ __global__ __launch_bounds__(64) void reduce_gather_kernel(char *base, uint64_t 
         }
         char *dst = base + dst_off + 16 * v;
 #pragma unroll kStores
-        for (int p = 0; p < npes; ++p) stream_store(dst + (uint64_t)p * pe_stride, acc.v);
+        for (int p = 0; p < npes; ++p) stream_store<NVSHMEM_AMD_STORE_REDUCE>(dst + (uint64_t)p * pe_stride, acc.v);
     }
     // elements behind the last full vector
     const uint64_t done = nvec * VEC;
@@ -376,7 +409,7 @@ __global__ __launch_bounds__(64) void reducescatter_gather_kernel(char *base, ui
                 }
             }
     }
-    stream_store(base + (uint64_t)blockIdx.y * pe_stride + dst_off + 16 * v, acc.v);
+    stream_store<NVSHMEM_AMD_STORE_REDUCESCATTER>(base + (uint64_t)blockIdx.y * pe_stride + dst_off + 16 * v, acc.v);
 }
 
 // Element-at-a-time variant for buffers that are not 16-byte aligned.
@@ -412,6 +445,12 @@ __global__ __launch_bounds__(kThreads) void reduce_scalar_kernel(char *base, uin
 // split costs them up to 9 %.
 #ifndef NVSHMEM_AMD_REPLICAS_PER_WAVE
 #define NVSHMEM_AMD_REPLICAS_PER_WAVE 4
+#endif
+#ifndef NVSHMEM_AMD_FCOLLECT_SPLIT
+#define NVSHMEM_AMD_FCOLLECT_SPLIT 1
+#endif
+#ifndef NVSHMEM_AMD_BROADCAST_SPLIT
+#define NVSHMEM_AMD_BROADCAST_SPLIT 1
 #endif
 static uint32_t replica_part_shift(int max_size) {
     uint32_t shift = 0;
@@ -684,7 +723,7 @@ int broadcast_on_stream(nvshmem_team_t team, void *dest, const void *src, size_t
     }
     // a source that cannot stay in the Infinity Cache: split the destinations (see replica_part_shift)
     const bool big_source = bytes * (uint64_t)tl.ngroups > rt.cacheable_source_bytes;
-    const uint32_t part_shift = big_source ? replica_part_shift(tl.max_size) : 0;
+    const uint32_t part_shift = big_source && NVSHMEM_AMD_BROADCAST_SPLIT ? replica_part_shift(tl.max_size) : 0;
     const uint64_t tiles = ((bytes / 16 + 64 + kCopyThreads - 1) / kCopyThreads + 1) << part_shift;
     if (tiles > 0x7fffffffull) {
         set_error("broadcast: message too large");
@@ -692,14 +731,14 @@ int broadcast_on_stream(nvshmem_team_t team, void *dest, const void *src, size_t
     }
     const dim3 grid((unsigned)tiles, 1, (unsigned)tl.ngroups), block(kCopyThreads);
     // blocks that share a piece re-read it from the cache, so the loads stay cacheable then
-    if (part_shift == 0 && big_source)
-        hipLaunchKernelGGL((segment_copy_kernel<kModeBroadcast, 1, true>), grid, block, 0, stream,
-                           rt.base, rt.heap_size, tl.groups, tl.max_size, doff, soff,
-                           (uint64_t)bytes, root, part_shift);
-    else
-        hipLaunchKernelGGL((segment_copy_kernel<kModeBroadcast, 1, false>), grid, block, 0, stream,
-                           rt.base, rt.heap_size, tl.groups, tl.max_size, doff, soff,
-                           (uint64_t)bytes, root, part_shift);
+#define NVSHMEM_AMD_LAUNCH_BROADCAST(NTL, STORE)                                                      \
+    hipLaunchKernelGGL((segment_copy_kernel<kModeBroadcast, 1, NTL, STORE>), grid, block, 0, stream,    \
+                       rt.base, rt.heap_size, tl.groups, tl.max_size, doff, soff, (uint64_t)bytes, root, \
+                       part_shift)
+    if (part_shift != 0) NVSHMEM_AMD_LAUNCH_BROADCAST(false, NVSHMEM_AMD_STORE_REPLICATE_SPLIT);
+    else if (big_source) NVSHMEM_AMD_LAUNCH_BROADCAST(true, NVSHMEM_AMD_STORE_REPLICATE);
+    else NVSHMEM_AMD_LAUNCH_BROADCAST(false, NVSHMEM_AMD_STORE_REPLICATE);
+#undef NVSHMEM_AMD_LAUNCH_BROADCAST
     hipError_t e = hipGetLastError();
     if (e != hipSuccess) {
         set_error("broadcast: kernel launch failed: %s", hipGetErrorString(e));
@@ -732,7 +771,8 @@ static int segment_collective(int mode, const char *what, nvshmem_team_t team, v
     const uint64_t tile_vectors = (uint64_t)kCopyThreads * (mode == kModeFcollect ? NVSHMEM_AMD_FCOLLECT_UNROLL
                                                                               : NVSHMEM_AMD_ALLTOALL_UNROLL);
     const bool big_source = src_bytes * total_members(tl) > rt.cacheable_source_bytes;
-    const uint32_t part_shift = mode == kModeFcollect && big_source ? replica_part_shift(tl.max_size) : 0;
+    const uint32_t part_shift =
+        mode == kModeFcollect && big_source && NVSHMEM_AMD_FCOLLECT_SPLIT ? replica_part_shift(tl.max_size) : 0;
     const uint64_t tiles = ((seg_bytes / 16 + 64 + tile_vectors - 1) / tile_vectors + 1) << part_shift;
     const unsigned segs = mode == kModeFcollect ? (unsigned)n : (unsigned)(n * n);
     if (tiles > 0x7fffffffull) {
@@ -742,16 +782,20 @@ static int segment_collective(int mode, const char *what, nvshmem_team_t team, v
     // blocks that share a piece re-read it from the cache, so the loads stay cacheable then
     const bool stream_source = part_shift == 0 && big_source;
     const dim3 grid((unsigned)tiles, segs, (unsigned)tl.ngroups), block(kCopyThreads);
-#define NVSHMEM_AMD_LAUNCH_SEGCOPY(MODE, U, NTL)                                                   \
-    hipLaunchKernelGGL((segment_copy_kernel<MODE, U, NTL>), grid, block, 0, stream, rt.base,       \
-                       rt.heap_size, tl.groups, tl.max_size, doff, soff, (uint64_t)seg_bytes, 0,  \
+#define NVSHMEM_AMD_LAUNCH_SEGCOPY(MODE, U, NTL, STORE)                                            \
+    hipLaunchKernelGGL((segment_copy_kernel<MODE, U, NTL, STORE>), grid, block, 0, stream, rt.base, \
+                       rt.heap_size, tl.groups, tl.max_size, doff, soff, (uint64_t)seg_bytes, 0,   \
                        part_shift)
     if (mode == kModeFcollect) {
-        if (stream_source) NVSHMEM_AMD_LAUNCH_SEGCOPY(kModeFcollect, NVSHMEM_AMD_FCOLLECT_UNROLL, true);
-        else NVSHMEM_AMD_LAUNCH_SEGCOPY(kModeFcollect, NVSHMEM_AMD_FCOLLECT_UNROLL, false);
+        if (part_shift != 0)
+            NVSHMEM_AMD_LAUNCH_SEGCOPY(kModeFcollect, NVSHMEM_AMD_FCOLLECT_UNROLL, false, NVSHMEM_AMD_STORE_REPLICATE_SPLIT);
+        else if (stream_source)
+            NVSHMEM_AMD_LAUNCH_SEGCOPY(kModeFcollect, NVSHMEM_AMD_FCOLLECT_UNROLL, true, NVSHMEM_AMD_STORE_REPLICATE);
+        else
+            NVSHMEM_AMD_LAUNCH_SEGCOPY(kModeFcollect, NVSHMEM_AMD_FCOLLECT_UNROLL, false, NVSHMEM_AMD_STORE_REPLICATE);
     } else {
-        if (stream_source) NVSHMEM_AMD_LAUNCH_SEGCOPY(kModeAlltoall, NVSHMEM_AMD_ALLTOALL_UNROLL, true);
-        else NVSHMEM_AMD_LAUNCH_SEGCOPY(kModeAlltoall, NVSHMEM_AMD_ALLTOALL_UNROLL, false);
+        if (stream_source) NVSHMEM_AMD_LAUNCH_SEGCOPY(kModeAlltoall, NVSHMEM_AMD_ALLTOALL_UNROLL, true, NVSHMEM_AMD_STORE_ALLTOALL);
+        else NVSHMEM_AMD_LAUNCH_SEGCOPY(kModeAlltoall, NVSHMEM_AMD_ALLTOALL_UNROLL, false, NVSHMEM_AMD_STORE_ALLTOALL);
     }
 #undef NVSHMEM_AMD_LAUNCH_SEGCOPY
     hipError_t e = hipGetLastError();
