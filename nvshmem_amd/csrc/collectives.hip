@@ -214,27 +214,28 @@ __global__ __launch_bounds__(kCopyThreads) void segment_copy_kernel(char *base, 
 }
 
 // ---------------------------------------------------------------------------------------------
-// Fused reduce, LDS staged.  A block owns a tile of `lanes` 16-byte vectors of the element range
-// (lanes = 64 when the team has at most 16 PEs, so one wavefront streams 1 KiB of one PE's source).
-// Thread (pe, i) loads vector i of the tile from PE pe's source into LDS - one load per thread, like
-// a plain copy, which HBM serves measurably faster than one lane gathering the same vector from
-// every PE.  After a barrier the tile's elements are folded out of LDS in PE order 0..n-1, one
-// element per thread, and thread (pe, i) stores result vector i into PE pe's destination.
+// Fused reduce, LDS staged.  A block owns a tile of 64 16-byte vectors of the element range and has one
+// wavefront per MPW members of the team, so a wavefront streams one aligned 1 KiB piece of a member's
+// source per load.  Thread (w, i) loads vector i of the tile from members w*MPW ... w*MPW + MPW-1 into
+// LDS - one load per lane and member, like a plain copy, which HBM serves measurably faster than one
+// lane gathering the same vector from every PE.  After a barrier the tile's elements are folded out of
+// LDS in PE order 0..n-1, one element per thread, and thread (w, i) stores result vector i into the
+// destinations of its members.
 // An element is read (by the loads of this block) before this block writes it and no other block
 // touches it, so dest == src (in place) needs no further staging.
 // ---------------------------------------------------------------------------------------------
-// NPES > 0 fixes the team size at compile time (fold fully unrolled, one wavefront per PE);
-// NPES == 0 takes both from the arguments.
+// NPES > 0 fixes the team size at compile time (fold fully unrolled); NPES == 0 takes it from the team
+// table, the block being sized for the largest team of the handle.
 // fold_next: one step of the fold, in the allreduce's operand order or (SCATTER) the reducescatter's.
 template <typename T, int OP, bool SCATTER>
 __device__ __forceinline__ T fold_next(int p, T acc, T x) {
     return SCATTER ? nvshmemi_amd_reduce_op<T, OP>(acc, x) : nvshmemi_amd_fold_step<T, OP>(p, acc, x);
 }
 
-template <typename T, int OP, int NPES, bool NTL, int VPT = NVSHMEM_AMD_REDUCE_VPT>
-__global__ __launch_bounds__(NPES ? NPES * 64 : 1024) void reduce_vector_kernel(char *base, uint64_t slice_bytes,
+template <typename T, int OP, int NPES, bool NTL, int VPT = NVSHMEM_AMD_REDUCE_VPT, int MPW = 1>
+__global__ __launch_bounds__(NPES ? NPES / MPW * 64 : 1024) void reduce_vector_kernel(char *base, uint64_t slice_bytes,
                                                              const nvshmemi_amd_team_view_t *groups,
-                                                             uint32_t lane_shift_arg, uint64_t dst_off,
+                                                             uint64_t dst_off,
                                                              uint64_t src_off, uint64_t nelems) {
     extern __shared__ __attribute__((aligned(16))) char lds[];
     constexpr int VEC = 16 / sizeof(T);
@@ -242,24 +243,26 @@ __global__ __launch_bounds__(NPES ? NPES * 64 : 1024) void reduce_vector_kernel(
     const nvshmemi_amd_team_view_t g = groups[blockIdx.z];
     const int npes = NPES ? NPES : g.size;
     base += (uint64_t)g.start * slice_bytes;
-    const uint32_t lane_shift = NPES ? 6u : lane_shift_arg;
-    const unsigned lanes = 1u << lane_shift;
-    const unsigned pe = threadIdx.x >> lane_shift, i = threadIdx.x & (lanes - 1);
+    constexpr uint32_t lane_shift = 6;  // a wavefront's 64 lanes move one aligned 1 KiB piece of a member
+    constexpr unsigned lanes = 1u << lane_shift;
+    // a wavefront serves MPW consecutive members (more than one only with a compile-time team size)
+    const unsigned pe0 = (threadIdx.x >> lane_shift) * MPW, i = threadIdx.x & (lanes - 1);
     const uint64_t nvec = nelems / VEC;
     // tiles are cut on absolute (16 * lanes)-byte boundaries of the destination, so a wavefront's
     // access is one aligned 1 KiB piece whatever the buffer's own alignment: `lead` vector slots of
     // the first tile lie in front of the buffer
     const uint64_t pe_stride = (uint64_t)g.stride * slice_bytes;  // from one member to the next
-    const bool member = NPES ? true : (int)pe < npes;        // the block is sized for the largest team
+    // the block is sized for the largest team of the handle: lanes of members a team does not have idle
+    auto member = [&](int m) { return NPES ? true : (int)pe0 + m < npes; };
     const uint64_t lead = ((uint64_t)(uintptr_t)(base + dst_off) >> 4) & (lanes - 1);
     // a tile is VPT pieces of `lanes` vectors per PE: thread (pe, i) loads vector i of each piece
-    const unsigned tile_vecs = (unsigned)VPT << lane_shift;
+    constexpr unsigned tile_vecs = (unsigned)VPT << lane_shift;
     const uint64_t ntiles = (nvec + lead + tile_vecs - 1) / tile_vecs;
     nvshmemi_v4u *stage = reinterpret_cast<nvshmemi_v4u *>(lds);           // [npes][tile_vecs]
     nvshmemi_v4u *result = stage + (size_t)npes * tile_vecs;               // [tile_vecs]
     const T *stage_e = reinterpret_cast<const T *>(stage);
     T *result_e = reinterpret_cast<T *>(result);
-    const unsigned tile_elems = tile_vecs * VEC;
+    constexpr unsigned tile_elems = tile_vecs * VEC;
 
     for (uint64_t tile = blockIdx.x; tile < ntiles; tile += gridDim.x) {
         // indices in front of the buffer wrap to huge values and are skipped like those behind it
@@ -267,16 +270,33 @@ __global__ __launch_bounds__(NPES ? NPES * 64 : 1024) void reduce_vector_kernel(
 #pragma unroll
         for (int u = 0; u < VPT; ++u) {
             const uint64_t v = v0 + ((uint64_t)u << lane_shift);
-            if (v < nvec && member)
-                stage[pe * tile_vecs + ((unsigned)u << lane_shift) + i] =
-                    stream_load<NTL>(base + (uint64_t)pe * pe_stride + src_off + 16 * v);
+            if (v < nvec) {
+#pragma unroll
+                for (int m = 0; m < MPW; ++m)
+                    if (member(m)) stage[(pe0 + m) * tile_vecs + ((unsigned)u << lane_shift) + i] =
+                        stream_load<NTL>(base + (uint64_t)(pe0 + m) * pe_stride + src_off + 16 * v);
+            }
         }
         __syncthreads();
         for (unsigned e = threadIdx.x; e < tile_elems; e += blockDim.x) {
             T acc = stage_e[e];
+            if (NPES) {
 #pragma unroll
-            for (int p = 1; p < npes; ++p)
-                acc = nvshmemi_amd_fold_step<T, OP>(p, acc, stage_e[(size_t)p * tile_elems + e]);
+                for (int p = 1; p < NPES; ++p)
+                    acc = nvshmemi_amd_fold_step<T, OP>(p, acc, stage_e[(size_t)p * tile_elems + e]);
+            } else {
+                // eight members' values fetched from LDS before they are folded, in member order
+                int p = 1;
+                for (; p + 8 <= npes; p += 8) {
+                    T x[8];
+#pragma unroll
+                    for (int k = 0; k < 8; ++k) x[k] = stage_e[(size_t)(p + k) * tile_elems + e];
+#pragma unroll
+                    for (int k = 0; k < 8; ++k) acc = nvshmemi_amd_fold_step<T, OP>(p + k, acc, x[k]);
+                }
+                for (; p < npes; ++p)
+                    acc = nvshmemi_amd_fold_step<T, OP>(p, acc, stage_e[(size_t)p * tile_elems + e]);
+            }
             result_e[e] = acc;
         }
         __syncthreads();
@@ -284,7 +304,11 @@ __global__ __launch_bounds__(NPES ? NPES * 64 : 1024) void reduce_vector_kernel(
         for (int u = 0; u < VPT; ++u) {
             const uint64_t v = v0 + ((uint64_t)u << lane_shift);
             const nvshmemi_v4u r = result[((unsigned)u << lane_shift) + i];
-            if (v < nvec && member) stream_store<NVSHMEM_AMD_STORE_REDUCE>(base + (uint64_t)pe * pe_stride + dst_off + 16 * v, r);
+            if (v < nvec) {
+#pragma unroll
+                for (int m = 0; m < MPW; ++m)
+                    if (member(m)) stream_store<NVSHMEM_AMD_STORE_REDUCE>(base + (uint64_t)(pe0 + m) * pe_stride + dst_off + 16 * v, r);
+            }
         }
     }
     // elements behind the last full vector
@@ -469,39 +493,54 @@ void launch_reduce(Runtime &rt, const TeamLaunch &tl, uint64_t dst_off, uint64_t
                    uint64_t nelems, hipStream_t stream) {
     const bool vector_ok = ((dst_off | src_off) & 15) == 0;
     const unsigned ngroups = (unsigned)tl.ngroups;
-    // Which vector kernel: the LDS-staged one only has the edge for teams of exactly 8 or 16 members
-    // with more than Runtime::lds_reduce_bytes (1 GiB) of sources in all (measured with random fp32 data, 8 members: 6.26 against
-    // 5.71 TB/s at 2 GiB, equal at 1 GiB, 49.6 against 40.8 us at 128 MiB; 16 members: +2..4 % from
-    // 512 MiB up); everything else - other team sizes, smaller messages - goes to the gather kernel
-    // (12 members +14 %, 32 +7 %, 64 +22 %, 4 +7 %).
+    // Which vector kernel.  Once the sources no longer fit the Infinity Cache - more than
+    // Runtime::lds_reduce_bytes (256 MiB, counted as 4-byte elements) in all - the LDS-staged kernel wins
+    // for every team of 3 to 64 members; below that, and for 2 members, the gather kernel does.
+    // Measured with random fp32 data and write-through stores, LDS-staged against gather, TB/s at
+    // 512 MiB / 2 GiB of sources: 4 members 6.54 / 6.55 against 6.19 / 6.24, 6 members 6.37 / 6.44
+    // against 5.89 / 5.58, 8 members 6.46 / 6.53 against 6.03 / 6.09, 12 members 6.28 / 6.28 against
+    // 5.73 / 5.83, 16 members 6.21 / 6.12 against 5.44 / 5.57, 32 members 6.17 / 6.10 against 5.22 / 5.49,
+    // 64 members 5.64 / 5.64 against 5.15 / 5.26; at 128 MiB the two are level, at 32 MiB the gather
+    // kernel leads by up to 20 % for up to 16 members.  A wavefront of the LDS kernel serves one member
+    // for the compile-time sizes 8 and 16, two members up to 32 and four beyond: one load and one store
+    // per lane measured best where the block stays within 16 wavefronts, and wavefronts of fewer than
+    // 64 lanes per member (512- or 256-byte accesses) lost 7-22 % against the gather kernel.  The
+    // compile-time team size is worth 6 % at 32 members (6.17 against 5.82), nothing at 64.
     const uint64_t total_bytes = total_members(tl) * nelems * sizeof(T);
     const int fixed_size = tl.min_size == tl.max_size ? tl.max_size : 0;
     const bool stream_source = total_bytes > rt.cacheable_source_bytes;
-    // the threshold counts elements (as 4-byte ones): narrow types fold more elements per byte, and the
-    // gather kernel does that arithmetic in one lane per vector (bf16 at 1 GiB: 5.3 against 6.0 TB/s)
-    if (vector_ok && (fixed_size == 8 || fixed_size == 16) &&
-        total_members(tl) * nelems > rt.lds_reduce_bytes / 4) {
+    // The threshold counts elements (as 4-byte ones): narrow types fold more elements per byte.
+    // mpw: members per wavefront of the LDS-staged kernel; ct_size: a compile-time team size, if any
+    int mpw = 0, ct_size = 0;
+    if (fixed_size == 8 || fixed_size == 16) ct_size = fixed_size, mpw = 1;
+    else if (fixed_size == 32) ct_size = 32, mpw = 2;
+    else if (tl.max_size >= 3 && tl.max_size <= 32) mpw = 2;
+    else if (tl.max_size > 32 && tl.max_size <= 64) mpw = 4;
+    if (vector_ok && mpw && total_members(tl) * nelems > rt.lds_reduce_bytes / 4) {
         const uint32_t lane_shift = 6;
-        const unsigned threads = (unsigned)fixed_size << lane_shift;
+        const unsigned threads = (unsigned)((tl.max_size + mpw - 1) / mpw) << lane_shift;
         const uint64_t nvec = nelems / (16 / sizeof(T));
         const uint64_t tile_vecs = (uint64_t)NVSHMEM_AMD_REDUCE_VPT << lane_shift;
         uint64_t blocks = (nvec + (1u << lane_shift) + tile_vecs - 1) / tile_vecs;  // room for the lead-in
         if (blocks > 0x7fffffffull) blocks = 0x7fffffffull;  // the tile loop covers the rest
-        const size_t lds = ((size_t)fixed_size + 1) * 16 * tile_vecs;
+        const size_t lds = ((size_t)tl.max_size + 1) * 16 * tile_vecs;
         const dim3 grid((unsigned)blocks, 1, ngroups);
-#define NVSHMEM_AMD_LAUNCH_REDUCE(N)                                                              \
+#define NVSHMEM_AMD_LAUNCH_REDUCE(N, MPW)                                                         \
     do {                                                                                          \
         if (stream_source)                                                                        \
-            hipLaunchKernelGGL((reduce_vector_kernel<T, OP, N, true>), grid, dim3(threads), lds,  \
-                               stream, rt.base, rt.heap_size, tl.groups, lane_shift, dst_off,    \
+            hipLaunchKernelGGL((reduce_vector_kernel<T, OP, N, true, NVSHMEM_AMD_REDUCE_VPT, MPW>), grid, dim3(threads), lds,  \
+                               stream, rt.base, rt.heap_size, tl.groups, dst_off,    \
                                src_off, nelems);                                                  \
         else                                                                                      \
-            hipLaunchKernelGGL((reduce_vector_kernel<T, OP, N, false>), grid, dim3(threads), lds, \
-                               stream, rt.base, rt.heap_size, tl.groups, lane_shift, dst_off,    \
+            hipLaunchKernelGGL((reduce_vector_kernel<T, OP, N, false, NVSHMEM_AMD_REDUCE_VPT, MPW>), grid, dim3(threads), lds, \
+                               stream, rt.base, rt.heap_size, tl.groups, dst_off,    \
                                src_off, nelems);                                                  \
     } while (0)
-        if (fixed_size == 8) NVSHMEM_AMD_LAUNCH_REDUCE(8);
-        else NVSHMEM_AMD_LAUNCH_REDUCE(16);
+        if (ct_size == 8) NVSHMEM_AMD_LAUNCH_REDUCE(8, 1);
+        else if (ct_size == 16) NVSHMEM_AMD_LAUNCH_REDUCE(16, 1);
+        else if (ct_size == 32) NVSHMEM_AMD_LAUNCH_REDUCE(32, 2);
+        else if (mpw == 2) NVSHMEM_AMD_LAUNCH_REDUCE(0, 2);
+        else NVSHMEM_AMD_LAUNCH_REDUCE(0, 4);
 #undef NVSHMEM_AMD_LAUNCH_REDUCE
     } else if (vector_ok) {
         const uint64_t nvec = nelems / (16 / sizeof(T));

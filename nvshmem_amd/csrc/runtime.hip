@@ -227,7 +227,7 @@ int nvshmemx_amd_init(int npes, size_t symmetric_size) {
     rt.dev.options = env_size("NVSHMEM_AMD_UNIT_PACKETS", 0) ? NVSHMEMI_AMD_OPTION_UNIT_PACKETS : 0;
     rt.plain_collective_launch = env_size("NVSHMEM_AMD_PLAIN_COLLECTIVE_LAUNCH", 0) != 0;
     rt.cacheable_source_bytes = env_size("NVSHMEM_AMD_CACHEABLE_SOURCE_BYTES", (size_t)256 << 20);
-    rt.lds_reduce_bytes = env_size("NVSHMEM_AMD_LDS_REDUCE_BYTES", (size_t)1 << 30);
+    rt.lds_reduce_bytes = env_size("NVSHMEM_AMD_LDS_REDUCE_BYTES", (size_t)256 << 20);
     if (!teams_init(rt)) {
         teams_finalize(rt);
         (void)hipFree(rt.base);

@@ -64,7 +64,7 @@ struct Runtime {
     // Allreduce on teams of exactly 8 or 16 members takes the LDS-staged kernel when the sources of
     // all PEs together hold more than this many bytes' worth of 4-byte elements:
     // NVSHMEM_AMD_LDS_REDUCE_BYTES, read at init
-    uint64_t lds_reduce_bytes = (uint64_t)1 << 30;
+    uint64_t lds_reduce_bytes = (uint64_t)256 << 20;
     uint64_t timeouts_seen = 0;  // bounded waits that gave up, as far as the host has reported them
 
     static Runtime &get();

@@ -223,3 +223,63 @@ def test_large_source_policy_of_fcollect_and_broadcast(npes, monkeypatch):
         assert np.array_equal(rt.download_all(fdst, (npes * n * 4,), np.uint8), O.alltoall(fdata.view(np.uint8)))
         for p in (src, dst, fsrc, fdst):
             rt.free(p)
+
+
+@pytest.mark.parametrize("npes", [3, 5, 12, 24, 32, 33, 48, 64])
+def test_lds_staged_allreduce_for_every_team_size_class(npes, monkeypatch):
+    """The LDS-staged allreduce serves teams of 3 to 64 members once the sources outgrow the cache
+    (NVSHMEM_AMD_LDS_REDUCE_BYTES, read at init): two members per wavefront up to 32, four beyond, 32 as a
+    compile-time size.  With the threshold at zero small messages take it too: ragged counts, buffers that
+    do not start on a 1 KiB boundary, in place, order-sensitive fp32 and bf16 sums, NaN-carrying max."""
+    monkeypatch.setenv("NVSHMEM_AMD_LDS_REDUCE_BYTES", "0")
+    rng = np.random.default_rng(7000 + npes)
+    with runtime(npes, 16 << 20) as rt:
+        cap = 40000
+        src = rt.malloc(cap * 8 + 1024); dst = rt.malloc(cap * 8 + 1024)
+        for n, off in ((1, 0), (255, 16), (256, 0), (4099, 48), (cap, 0), (30001, 1008)):
+            f = (rng.standard_normal((npes, n)) * 10.0 ** rng.integers(-3, 4, (npes, n))).astype(np.float32)
+            rt.upload_all(src, f, off)
+            rt.fill(dst, 0xCD, cap * 8 + 1024)
+            note("lds allreduce npes=%d float sum n=%d off=%d" % (npes, n, off))
+            rt.reduce("float", "sum", dst + off, src + off, n)
+            want = O.reduce("f32", "sum", f)
+            got = rt.download_all(dst, ((off + n * 4 + 64) // 4,), np.uint32)
+            for pe in range(npes):
+                assert bits_equal(got[pe, off // 4:off // 4 + n], want.view(np.uint32)), (n, off, pe)
+            assert (got[:, :off // 4] == 0xCDCDCDCD).all() and (got[:, off // 4 + n:] == 0xCDCDCDCD).all()
+        n = 12345
+        f = rng.standard_normal((npes, n)).astype(np.float32)
+        f[rng.integers(0, npes, 50), rng.integers(0, n, 50)] = np.nan
+        f[rng.integers(0, npes, 50), rng.integers(0, n, 50)] = -0.0
+        rt.upload_all(src, f)
+        note("lds allreduce npes=%d float max with NaN, in place" % npes)
+        rt.reduce("float", "max", src, src, n)
+        want = O.reduce("f32", "max", f)
+        assert all(bits_equal(rt.download(src, pe, (n,), np.float32), want) for pe in (0, npes // 2, npes - 1))
+        b = (rng.standard_normal((npes, n)).astype(np.float32).view(np.uint32) >> 16).astype(np.uint16)
+        rt.upload_all(src, b)
+        rt.reduce("bfloat16", "sum", dst, src, n)
+        assert bits_equal(rt.download(dst, npes - 1, (n,), np.uint16), O.reduce("bf16", "sum", b))
+        x = rng.integers(-2**63, 2**63 - 1, (npes, n), dtype=np.int64)
+        rt.upload_all(src, x)
+        rt.reduce("int64", "xor", dst, src, n)
+        assert np.array_equal(rt.download(dst, 1, (n,), np.int64), O.reduce("i64", "xor", x))
+        # a family of ragged teams on one handle: rows of a 2-D split, the last one shorter
+        xr = 5 if npes > 5 else 2
+        xt, yt = rt.team_split_2d(N.TEAM_WORLD, xr)
+        f = (rng.standard_normal((npes, n)) * 10.0 ** rng.integers(-3, 4, (npes, n))).astype(np.float32)
+        rt.upload_all(src, f)
+        note("lds allreduce npes=%d rows of %d" % (npes, xr))
+        rt.reduce("float", "sum", dst, src, n, team=xt)
+        for r0 in range(0, npes, xr):
+            members = list(range(r0, min(r0 + xr, npes)))
+            want = O.reduce("f32", "sum", f[members])
+            for pe in (members[0], members[-1]):
+                assert bits_equal(rt.download(dst, pe, (n,), np.float32), want), (r0, pe)
+        rt.reduce("float", "sum", dst, src, n, team=yt)       # columns: strided members
+        for c in (0, xr - 1):
+            members = list(range(c, npes, xr))
+            want = O.reduce("f32", "sum", f[members])
+            assert bits_equal(rt.download(dst, members[-1], (n,), np.float32), want), c
+        rt.team_destroy(xt); rt.team_destroy(yt)
+        rt.free(src); rt.free(dst)
