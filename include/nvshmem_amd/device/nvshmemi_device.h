@@ -214,7 +214,9 @@ enum nvshmemi_amd_store_policy_t { NVSHMEMI_AMD_STORE_STREAM = 0, NVSHMEMI_AMD_S
 template <int STORE = NVSHMEMI_AMD_STORE_STREAM>
 NVSHMEMI_DEVICE_INLINE void nvshmemi_amd_stream_store16(char *p, nvshmemi_v4u v) {
     if (STORE == NVSHMEMI_AMD_STORE_WRITE_THROUGH) {
-        nvshmemi_amd_store16_agent(p, v);
+        // sc1 nt: written through at agent scope and marked streaming (+3 % over plain sc1 on the per-row
+        // put_signal token dispatch); the s_nop for the same reason as in nvshmemi_amd_store16_agent
+        asm volatile("global_store_dwordx4 %0, %1, off sc1 nt\n\ts_nop 1" : : "v"(p), "v"(v) : "memory");
         return;
     }
 #if defined(NVSHMEMI_AMD_COPY_NT) && !(NVSHMEMI_AMD_COPY_NT & 2)
