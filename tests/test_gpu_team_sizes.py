@@ -180,7 +180,7 @@ def test_small_in_kernel_collectives_with_and_without_packets(disable, plain, mo
         rt.free(src); rt.free(dst)
 
 
-@pytest.mark.parametrize("npes", [3, 8, 13, 16])
+@pytest.mark.parametrize("npes", [3, 8, 13, 16, 33, 64])
 def test_large_source_policy_of_fcollect_and_broadcast(npes, monkeypatch):
     """Sources beyond NVSHMEM_AMD_CACHEABLE_SOURCE_BYTES (read at init) are streamed, and fcollect /
     broadcast then split the destinations of a piece over neighbouring blocks (at most four per
