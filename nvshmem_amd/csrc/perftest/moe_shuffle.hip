@@ -487,8 +487,9 @@ static int dispatch_pieces(void *recv, size_t recv_cap_rows, const void *send, c
     int rc = perftest::launch_status("moe_dispatch_pieces");
     if (rc != 0) return rc;
     // one block per PE scanning alone is bound by its own memory latency (65536 rows: 46 us); with a
-    // few blocks per PE - still at most 512 in all, co-resident on this GPU, so an ordinary launch is
-    // enough for the waits - the scan is short
+    // few blocks per PE the scan is short.  An ordinary launch is enough: a block announces its counts
+    // before it waits and only block 0 of each PE waits at all, so the blocks that wait (one per PE, at
+    // most 64) can never keep a block that still has to announce off the GPU
     const unsigned sig_blocks = (unsigned)(((size_t)tokens * (size_t)topk + 8191) / 8192 < 8 ? ((size_t)tokens * (size_t)topk + 8191) / 8192 : 8);
     if (static_sig)
         hipLaunchKernelGGL(moe_dispatch_signal_kernel<false>, dim3(sig_blocks, 1, (unsigned)nvshmem_n_pes()), dim3(1024),

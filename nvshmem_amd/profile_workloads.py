@@ -12,6 +12,7 @@ nvshmem_amd/profile_summary.py can cut the trace into workloads by counting mark
 workload is the counter calibration: a plain copy kernel that reads 1 GiB and writes 1 GiB.
 """
 import argparse
+import tempfile
 import json
 import os
 import sys
@@ -59,7 +60,7 @@ def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--iters", type=int, default=10)
     ap.add_argument("--only", default="", help="comma-separated workload names")
-    ap.add_argument("--manifest", default=os.path.join(ROOT, "gpurun_out", "profile_manifest.json"))
+    ap.add_argument("--manifest", default=os.path.join(tempfile.gettempdir(), "nvshmem_amd_profile_manifest.json"))
     args = ap.parse_args()
     import numpy as np
     import nvshmem_amd as N

@@ -292,8 +292,10 @@ class MoeShuffle(Group):
                    "moe_dispatch_pieces", rt)
 
         def combine():
+            # one block (one wavefront) per 2 KiB work item: 7 items per 14 KiB row
             _check(perf.nvshmem_perftest_moe_combine_pieces(self.out, self.recv, cap, self.d_pe, self.d_row, T, K, row,
-                                                            2048, 262144, 64, SCOPE_WARP, None), "moe_combine", rt)
+                                                            2048, rows * ((row + 2047) // 2048), 64, SCOPE_WARP, None),
+                   "moe_combine", rt)
         moved = npes * rows * row
         shape = "8 logical PEs x 8192 tokens x 7168 bf16, top-8 of 256 experts, Zipf(1.1)"
         common = {"npes": npes, "tokens": T, "topk": K, "experts": self.E, "row_bytes": row}
