@@ -264,7 +264,7 @@ class MoeShuffle(Group):
         self.heap_bytes = self.cap * self.row + self.rows * self.row + self.T * self.row + 64 * MiB
 
     def names(self):
-        return ["moe_dispatch_put_signal", "moe_dispatch_plain_store", "moe_combine"]
+        return ["moe_dispatch_put_signal", "moe_dispatch_put_quiet_signal", "moe_dispatch_plain_store", "moe_combine"]
 
     def setup(self, rt, gen):
         self.rt, self.perf = rt, rt.perftest()
@@ -284,6 +284,12 @@ class MoeShuffle(Group):
             _check(perf.nvshmem_perftest_moe_dispatch_put_signal(
                 self.recv, cap, self.send, self.d_pe, self.d_row, self.d_expected, self.sig, self.SIG_STRIDE, T, K,
                 row, 64, 256, SCOPE_WARP | 256 | 512, None), "moe_dispatch_put_signal", rt)
+
+        def put_quiet_signal():
+            _check(perf.nvshmem_perftest_fill_words(self.sig, 0, npes, None), "fill_words", rt)
+            _check(perf.nvshmem_perftest_moe_dispatch_ex(self.recv, cap, self.send, self.d_pe, self.d_row,
+                                                         self.d_expected, self.sig, T, K, row, 32, 256, SCOPE_WARP,
+                                                         None), "moe_dispatch_ex", rt)
 
         def plain_store():
             _check(perf.nvshmem_perftest_fill_words(self.sig, 0, npes, None), "fill_words", rt)
@@ -307,6 +313,12 @@ class MoeShuffle(Group):
                  "moe_dispatch_put_signal: one nvshmemx_putmem_signal_nbi_warp per row copy (NVSHMEM_SIGNAL_ADD of 1, "
                  "payload-only ordering, one signal word per source on its own 128-byte line), receivers "
                  "nvshmem_signal_wait_until(GE); " + shape, put_signal, dict(common, note=lower), scale=5),
+            Item("moe_dispatch_put_quiet_signal", "u8", moved + moved // K,
+                 "moe_dispatch_kernel<warp> (nvshmemx_putmem_nbi_warp per row, nvshmemx_quiet_block, nvshmemx_signal_op)",
+                 "moe_dispatch_put_quiet_signal: one nvshmemx_putmem_nbi_warp per row copy, rows per destination "
+                 "tallied per block, then one nvshmemx_quiet_block and one nvshmemx_signal_op(NVSHMEM_SIGNAL_ADD) per "
+                 "block and destination, receivers nvshmem_signal_wait_until(GE); " + shape, put_quiet_signal,
+                 dict(common, note=lower), scale=5),
             Item("moe_dispatch_plain_store", "u8", moved + moved // K,
                  "moe_dispatch_direct_kernel<1> + moe_dispatch_signal_kernel",
                  "moe_dispatch_plain_store: NOT the put API - 1 KiB work items stored through nvshmem_ptr by one "
@@ -316,7 +328,7 @@ class MoeShuffle(Group):
             Item("moe_combine", "u8", 2 * moved, "moe_combine_kernel<warp, 2048>",
                  "moe_combine: nvshmemx_getmem_nbi_warp per 2 KiB of a row; " + shape, combine, common, scale=5),
         ]
-        for it, what in zip(items, ("put_signal", "plain_store", "combine")):
+        for it, what in zip(items, ("put_signal", "plain_store", "plain_store", "combine")):
             it.what = what
         return items
 
