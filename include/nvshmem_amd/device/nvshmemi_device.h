@@ -114,12 +114,18 @@ NVSHMEMI_DEVICE_INLINE int nvshmemi_amd_my_pe() {
 }
 NVSHMEMI_DEVICE_INLINE int nvshmemi_amd_n_pes() { return nvshmemi_device_state_d.npes; }
 
-/* Offset inside its slice of an address anywhere in the heap.  Symmetric addresses are nearly always
- * canonical (PE 0's slice), where the offset is the distance from the heap base; the division only
- * runs for an address that names another PE's copy. */
+/* Offset inside its slice of an address anywhere in the heap (canonical addresses, PE 0's slice, are
+ * their own offset).  The slice index floor(d / size) is computed without a division or a branch: size
+ * is a multiple of 2 MiB, so it equals floor((d >> 21) / (size >> 21)), and for the fewer than 2^18
+ * units of a heap of at most 512 GiB that quotient is ((d >> 21) * heap_magic) >> 40 with
+ * heap_magic = floor(2^40 / (size >> 21)) + 1 (the error of the reciprocal, below 2^-22, is smaller than
+ * the 1 / (size >> 21) that separates a quotient from the next integer).  A dozen scalar instructions
+ * when the address is wave-uniform; a compare-and-divide form cost the small collectives 0.1-0.2 us. */
 NVSHMEMI_DEVICE_INLINE uint64_t nvshmemi_amd_slice_offset(const void *sym) {
     const uint64_t d = (uint64_t)((const char *)sym - nvshmemi_device_state_d.heap_base);
-    return d < nvshmemi_device_state_d.heap_size ? d : d % nvshmemi_device_state_d.heap_size;
+    const uint32_t slice =
+        (uint32_t)(((uint64_t)(uint32_t)(d >> 21) * nvshmemi_device_state_d.heap_magic) >> 40);
+    return d - (uint64_t)slice * nvshmemi_device_state_d.heap_size;
 }
 /* Address of PE `pe`'s copy of the symmetric object at `sym` (an address in any PE's slice). */
 NVSHMEMI_DEVICE_INLINE char *nvshmemi_amd_remote(const void *sym, int pe) {
@@ -1315,6 +1321,12 @@ NVSHMEMI_DEVICE_INLINE unsigned nvshmemi_amd_ll_reduce_group(size_t nbytes, int 
  * its elements in member order and stores them.  Flags, buffer rotation and the `done` word are those
  * of the 16-byte packets above (the two formats share the buffers: a stale word of the other format
  * cannot equal a later call's flag word).
+ *
+ * Compiled in only where the including translation unit defines NVSHMEMI_AMD_UNIT_PACKETS (every
+ * member's code must then be built that way).  It measured no faster than the staged one-barrier form
+ * it would replace (8 PEs, 256 threads: 1 KiB per member 3.83 against 3.41 us, 2 KiB 3.84 against
+ * 3.80), and its mere presence in a kernel - as a branch never taken - cost the reducescatter beside
+ * it 1.2 us per call, so the default build leaves it out.
  * ---------------------------------------------------------------------------------------------- */
 #define NVSHMEMI_AMD_UNIT_BYTES 64
 #define NVSHMEMI_AMD_UNIT_PAYLOAD 56
@@ -1659,11 +1671,12 @@ NVSHMEMI_DEVICE_INLINE int nvshmemi_reduce_threadgroup(nvshmem_team_t team, T *d
         nvshmemi_amd_ll_reduce<T, OP, SCOPE>(team, tv, dest, source, nreduce, group);
         return 0;
     }
-    if ((nvshmemi_device_state_d.options & NVSHMEMI_AMD_OPTION_UNIT_PACKETS) &&
-        nvshmemi_amd_units_fit<SCOPE>(nreduce * sizeof(T), npes)) {
+#ifdef NVSHMEMI_AMD_UNIT_PACKETS
+    if (nvshmemi_amd_units_fit<SCOPE>(nreduce * sizeof(T), npes)) {
         nvshmemi_amd_unit_reduce<T, OP, SCOPE, false>(team, tv, dest, source, nreduce);
         return 0;
     }
+#endif
     if (nvshmemi_amd_staged_fits<SCOPE, false>(dest, source, nreduce * sizeof(T), npes)) {
         nvshmemi_amd_staged_reduce<T, OP, SCOPE, false>(team, tv, dest, source, nreduce);
         return 0;
@@ -1943,11 +1956,12 @@ NVSHMEMI_DEVICE_INLINE int nvshmemi_reducescatter_threadgroup(nvshmem_team_t tea
         nvshmemi_amd_ll_reduce<T, OP, SCOPE, true>(team, tv, dest, source, nreduce, group);
         return 0;
     }
-    if ((nvshmemi_device_state_d.options & NVSHMEMI_AMD_OPTION_UNIT_PACKETS) &&
-        nvshmemi_amd_units_fit<SCOPE>(nreduce * sizeof(T), npes)) {
+#ifdef NVSHMEMI_AMD_UNIT_PACKETS
+    if (nvshmemi_amd_units_fit<SCOPE>(nreduce * sizeof(T), npes)) {
         nvshmemi_amd_unit_reduce<T, OP, SCOPE, true>(team, tv, dest, source, nreduce);
         return 0;
     }
+#endif
     if (nvshmemi_amd_staged_fits<SCOPE, true>(dest, source, nreduce * sizeof(T), npes)) {
         nvshmemi_amd_staged_reduce<T, OP, SCOPE, true>(team, tv, dest, source, nreduce);
         return 0;

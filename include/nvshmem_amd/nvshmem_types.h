@@ -232,7 +232,7 @@ typedef struct nvshmemi_device_state {
     uint32_t version;     /* (1 << 16) + sizeof(struct) */
     int32_t mype;         /* PE a kernel acts as when its grid is not PE-multiplexed */
     int32_t npes;
-    uint32_t options;     /* NVSHMEMI_AMD_OPTION_* bits */
+    uint32_t options;     /* reserved, 0 */
     char *heap_base;      /* start of PE 0's slice */
     uint64_t heap_size;   /* bytes from one PE's slice to the next (a multiple of 2 MiB, of 16 MiB for large heaps) */
     uint64_t *sync_flags; /* canonical address: NVSHMEMI_AMD_MAX_PES arrival words per PE */
@@ -246,11 +246,10 @@ typedef struct nvshmemi_device_state {
                             [MAX_TEAMS][npes][NVSHMEMI_AMD_STAGE_BUFFERS][NVSHMEMI_AMD_STAGE_BYTES] */
     uint64_t *runtime_words; /* one copy for the whole GPU (an address in PE 0's slice, used as it is):
                                 word NVSHMEMI_AMD_TIMEOUT_COUNT_WORD counts the bounded waits that gave up */
+    uint64_t heap_magic;     /* floor(2^40 / (heap_size >> 21)) + 1: the slice that holds heap offset d is
+                                ((d >> 21) * heap_magic) >> 40 (exact while the whole heap is at most 512 GiB) */
 } nvshmemi_device_state_t;
 
-/* in-kernel allreduce / reducescatter of up to 3.5 KiB per member through 64-byte line packets instead of
- * the staged one-barrier form (NVSHMEM_AMD_UNIT_PACKETS=1 at init; off by default: it measured no faster) */
-#define NVSHMEMI_AMD_OPTION_UNIT_PACKETS 1u
 #define NVSHMEMI_AMD_TIMEOUT_COUNT_WORD 0
 /* bytes at the end of every PE's slice that the runtime keeps for itself: barrier arrival row, epoch,
  * timeout record and runtime words, 512 bytes each */

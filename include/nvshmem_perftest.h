@@ -147,6 +147,9 @@ int nvshmem_perftest_api_matrix(void *a, void *b, uint64_t *sig, int *ints, int6
 /* In-kernel collectives, one thread group per PE (grid 1 x 1 x npes).  dtype/op use the numbering
  * of nvshmemi_amd_dtype_t / nvshmemi_amd_op_t; supported pairs: (i32,sum) (i64,xor) (f32,sum)
  * (f32,max) (bf16,sum) (bf16,max) (u64,and) (f64,prod) (i16,min).  Returns NOT_SUPPORTED else. */
+/* 1 if the in-kernel collective kernels of the library were built with NVSHMEMI_AMD_UNIT_PACKETS (the 64-byte
+ * line packets of the small allreduce / reducescatter; libnvshmem_amd_perftest_units.so is), else 0. */
+int nvshmem_perftest_unit_packets_compiled(void);
 int nvshmem_perftest_device_reduce(int dtype, int op, void *dest, const void *src, size_t nreduce,
                                    int scope, int threads, void *stream);
 int nvshmem_perftest_device_fcollect(void *dest, const void *src, size_t bytes, int scope,

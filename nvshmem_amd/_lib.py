@@ -138,6 +138,7 @@ def load_perftest():
         "nvshmem_perftest_signal_wait": [vp, i32, u64, vp, vp],
         "nvshmem_perftest_put_signal_pingpong": [vp, vp, sz, i32, i32, vp],
         "nvshmem_perftest_ring_reduce": [vp, vp, sz, vp, sz, i32, i32, vp],
+        "nvshmem_perftest_unit_packets_compiled": [],
         "nvshmem_perftest_device_reduce": [i32, i32, vp, vp, sz, i32, i32, vp],
         "nvshmem_perftest_device_fcollect": [vp, vp, sz, i32, i32, vp],
         "nvshmem_perftest_amo_matrix_cases": [],
@@ -172,6 +173,27 @@ def load_perftest():
         fn = getattr(lib, name)
         fn.restype, fn.argtypes = i32, args
     lib._typed = True
+    lib._signatures = sig
+    return lib
+
+
+def load_perftest_units():
+    """The in-kernel collective test kernels built with NVSHMEMI_AMD_UNIT_PACKETS: same entry point names as
+    in load_perftest(), so the library is opened on its own (RTLD_LOCAL) and only those names are typed."""
+    main = load_perftest()
+    name = "libnvshmem_amd_perftest_units.so"
+    if name in _cache:
+        return _cache[name]
+    path = os.path.join(LIBDIR, name)
+    if not os.path.exists(path):
+        raise LibraryMissing(
+            "%s is not built; run `python -m nvshmem_amd.build` (there is no CPU fallback)" % path)
+    lib = C.CDLL(path, mode=C.RTLD_LOCAL)
+    for fname, args in main._signatures.items():
+        if hasattr(lib, fname):
+            fn = getattr(lib, fname)
+            fn.restype, fn.argtypes = i32, args
+    _cache[name] = lib
     return lib
 
 

@@ -2,6 +2,8 @@
 
   nvshmem_amd/lib/libnvshmem_amd.so           host runtime + host-launched collectives (C ABI)
   nvshmem_amd/lib/libnvshmem_amd_perftest.so  kernels that call the device API + their C ABI drivers
+  nvshmem_amd/lib/libnvshmem_amd_perftest_units.so  the in-kernel collective kernels of that library built with
+                                              NVSHMEMI_AMD_UNIT_PACKETS (64-byte line packets), for their parity test
   oracle/liboracle.so                         CPU oracle (test infrastructure only)
 
 Run as ``python -m nvshmem_amd.build``.  hipcc cross-compiles without a GPU.
@@ -41,9 +43,16 @@ def _run(cmd):
         sys.stderr.write(out + "\n")
 
 
+UNITS_SOURCE = "perftest/coll_kernels.hip"     # built a second time with the line packets compiled in
+UNITS_TAG = "+units"
+
+
 def _compile(src):
-    obj = os.path.join(OBJDIR, src.replace("/", "_") + ".o")
-    cmd = [HIPCC] + HIP_FLAGS + ["-c", os.path.join(CSRC, src), "-o", obj]
+    extra = []
+    if src.endswith(UNITS_TAG):
+        src, extra = src[:-len(UNITS_TAG)], ["-DNVSHMEMI_AMD_UNIT_PACKETS"]
+    obj = os.path.join(OBJDIR, src.replace("/", "_") + ("_units" if extra else "") + ".o")
+    cmd = [HIPCC] + HIP_FLAGS + extra + ["-c", os.path.join(CSRC, src), "-o", obj]
     if src.endswith(".cpp"):
         cmd.insert(1, "-x")
         cmd.insert(2, "hip")
@@ -76,6 +85,8 @@ def build_native(jobs=8):
     os.makedirs(BINDIR, exist_ok=True)
     sources = RUNTIME_SOURCES + [s for s in PERFTEST_SOURCES + [DRIVER_SOURCE]
                                  if os.path.exists(os.path.join(CSRC, s))]
+    if UNITS_SOURCE in sources:
+        sources.append(UNITS_SOURCE + UNITS_TAG)
     with ThreadPoolExecutor(max_workers=jobs) as pool:
         objs = dict(zip(sources, pool.map(_compile, sources)))
     runtime = os.path.join(LIBDIR, "libnvshmem_amd.so")
@@ -84,6 +95,10 @@ def build_native(jobs=8):
     if perf:
         _link(perf, os.path.join(LIBDIR, "libnvshmem_amd_perftest.so"),
               ["-L" + LIBDIR, "-lnvshmem_amd", "-Wl,-rpath,$ORIGIN"])
+    if UNITS_SOURCE + UNITS_TAG in objs:
+        # the same entry point names as the library above: bound inside the library, loaded on its own
+        _link([objs[UNITS_SOURCE + UNITS_TAG]], os.path.join(LIBDIR, "libnvshmem_amd_perftest_units.so"),
+              ["-L" + LIBDIR, "-lnvshmem_amd", "-Wl,-rpath,$ORIGIN", "-Wl,-Bsymbolic"])
     if perf and DRIVER_SOURCE in objs:
         _run([HIPCC, "--offload-arch=gfx950", "-o", os.path.join(BINDIR, "nvshmem_perftest"),
               objs[DRIVER_SOURCE], "-L" + LIBDIR, "-lnvshmem_amd_perftest", "-lnvshmem_amd",

@@ -266,6 +266,14 @@ int launch_scoped(int scope, void (*kb)(Args...), void (*kw)(Args...), void (*kt
 
 extern "C" {
 
+int nvshmem_perftest_unit_packets_compiled(void) {
+#ifdef NVSHMEMI_AMD_UNIT_PACKETS
+    return 1;
+#else
+    return 0;
+#endif
+}
+
 int nvshmem_perftest_device_reducescatter(int dtype, int op, void *dest, const void *src,
                                           size_t nreduce, int scope, int threads, void *stream) {
     static const size_t esize[NVSHMEMI_DT_COUNT] = {1, 2, 4, 8, 1, 2, 4, 8, 2, 2, 4, 8};

@@ -187,6 +187,11 @@ int nvshmemx_amd_init(int npes, size_t symmetric_size) {
         return NVSHMEMX_ERROR_INTERNAL;
     }
     const uint64_t total = (uint64_t)npes * slice_bytes;
+    // (the device code's division-free slice index is exact up to this size)
+    if (total > (1ull << 39)) {
+        set_error("nvshmemx_amd_init: %d PEs x %llu bytes exceed 512 GiB", npes, (unsigned long long)slice_bytes);
+        return NVSHMEMX_ERROR_INVALID_VALUE;
+    }
     void *mem = nullptr;
     hipError_t e = hipMalloc(&mem, total);
     if (e != hipSuccess || !mem) {
@@ -224,7 +229,8 @@ int nvshmemx_amd_init(int npes, size_t symmetric_size) {
     rt.dev.timeout_record = (uint64_t *)(uintptr_t)trec;
     rt.dev.runtime_words = (uint64_t *)(uintptr_t)(trec + NVSHMEMI_MALLOC_ALIGNMENT);
     rt.dev.spin_limit = env_size("NVSHMEM_AMD_SPIN_LIMIT", 1ull << 22);
-    rt.dev.options = env_size("NVSHMEM_AMD_UNIT_PACKETS", 0) ? NVSHMEMI_AMD_OPTION_UNIT_PACKETS : 0;
+    rt.dev.options = 0;
+    rt.dev.heap_magic = (1ull << 40) / (rt.heap_size >> 21) + 1;
     rt.plain_collective_launch = env_size("NVSHMEM_AMD_PLAIN_COLLECTIVE_LAUNCH", 0) != 0;
     rt.cacheable_source_bytes = env_size("NVSHMEM_AMD_CACHEABLE_SOURCE_BYTES", (size_t)256 << 20);
     rt.lds_reduce_bytes = env_size("NVSHMEM_AMD_LDS_REDUCE_BYTES", (size_t)256 << 20);

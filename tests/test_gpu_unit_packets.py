@@ -1,6 +1,6 @@
-"""The 64-byte line packets (f4: the reference's LL128 re-derived, off by default) switched on with
-NVSHMEM_AMD_UNIT_PACKETS=1: in-kernel allreduce and reducescatter of 257 B ... 3.5 KiB per member then
-travel as units of 56 payload bytes + flag word.  Bit-exact against the oracle over element types,
+"""The 64-byte line packets (f4: the reference's LL128 re-derived; compiled in only where a translation unit
+defines NVSHMEMI_AMD_UNIT_PACKETS, as libnvshmem_amd_perftest_units.so is): in-kernel allreduce and
+reducescatter of 257 B ... 3.5 KiB per member then travel as units of 56 payload bytes + flag word.  Bit-exact against the oracle over element types,
 sizes around both ends of the range, odd offsets, in place, wavefront and block scope, and 40 rounds of
 reduce / broadcast / fcollect / alltoall / reducescatter with data that changes every round (a torn or
 stale unit would show)."""
@@ -16,13 +16,16 @@ pytestmark = pytest.mark.gpu
 
 @pytest.fixture(scope="module")
 def rt8():
-    import os
-    os.environ["NVSHMEM_AMD_UNIT_PACKETS"] = "1"
-    try:
-        with runtime(8, 1 << 24) as r:
-            yield r
-    finally:
-        del os.environ["NVSHMEM_AMD_UNIT_PACKETS"]
+    with runtime(8, 1 << 24) as r:
+        yield r
+
+
+def _units():
+    from nvshmem_amd import _lib
+    lib = _lib.load_perftest_units()
+    assert lib.nvshmem_perftest_unit_packets_compiled() == 1
+    assert _lib.load_perftest().nvshmem_perftest_unit_packets_compiled() == 0     # the default build has none
+    return lib
 
 
 def _data(rng, kind, shape):
@@ -38,7 +41,7 @@ def _data(rng, kind, shape):
 
 @pytest.mark.parametrize("scope,threads", [(N.SCOPE_BLOCK, 256), (N.SCOPE_BLOCK, 1024), (N.SCOPE_WARP, 64)])
 def test_reduce_and_reducescatter_through_line_packets(rt8, scope, threads):
-    perf = rt8.perftest()
+    perf = _units()
     rng = np.random.default_rng(threads)
     src = rt8.malloc(1 << 17); dst = rt8.malloc(1 << 17)
     lanes = threads if scope == N.SCOPE_BLOCK else 64
@@ -77,7 +80,7 @@ def test_reduce_and_reducescatter_through_line_packets(rt8, scope, threads):
 
 def test_forty_rounds_of_changing_data_through_line_packets(rt8):
     from test_gpu_small_collectives import _expected_checks
-    perf = rt8.perftest()
+    perf = _units()
     for n, fc_bytes in ((300, 64), (512, 256), (896, 8)):       # 1200, 2048 and 3584 bytes per member
         src = rt8.malloc(5000 * 4); dst = rt8.malloc(8 * 2052 + 5000 * 4); check = rt8.calloc(1, 8)
         note("coll sequence through line packets n=%d" % n)
