@@ -1597,20 +1597,24 @@ NVSHMEMI_DEVICE_INLINE void nvshmemi_amd_staged_reduce(nvshmem_team_t team, cons
     const T *src = reinterpret_cast<const T *>(nvshmemi_amd_local(source));
     /* push: member idx gets src (SCATTER: block idx of src) in slot me */
     for (size_t v = tid; v < nvec; v += nthr) {
+        /* (plain 16-byte vectors: as an array of the element union the batch was kept in scratch memory) */
         for (int i0 = 0; i0 < npes; i0 += 8) {
-            pack_t x[8];
+            nvshmemi_v4u x[8];
 #pragma unroll
             for (int k = 0; k < 8; ++k) {
                 const int ii = i0 + k < npes ? i0 + k : npes - 1; /* past the end: the last member once more */
                 const int idx = me + ii < npes ? me + ii : me + ii - npes;
-                x[k] = *reinterpret_cast<const pack_t *>(src + (SCATTER ? (size_t)idx * nreduce : 0) + v * VEC);
+                if (SCATTER || k == 0)
+                    x[k] = *reinterpret_cast<const nvshmemi_v4u *>(src + (SCATTER ? (size_t)idx * nreduce : 0) + v * VEC);
+                else
+                    x[k] = x[0];
             }
 #pragma unroll
             for (int k = 0; k < 8; ++k) {
                 const int ii = i0 + k < npes ? i0 + k : npes - 1;
                 const int idx = me + ii < npes ? me + ii : me + ii - npes;
                 char *to = nvshmemi_amd_stage_buffer(team, nvshmemi_amd_team_pe(tv, idx), which) + (size_t)me * slot;
-                *reinterpret_cast<pack_t *>(to + 16 * v) = x[k];
+                *reinterpret_cast<nvshmemi_v4u *>(to + 16 * v) = x[k];
             }
         }
     }
