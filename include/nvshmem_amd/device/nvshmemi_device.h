@@ -317,7 +317,10 @@ NVSHMEMI_DEVICE_INLINE void nvshmemi_amd_copy_vectors(char *__restrict__ dst,
                                                      const char *__restrict__ src, size_t nvec,
                                                      size_t tid, size_t nthr, bool stream_loads) {
 #if NVSHMEMI_AMD_COPY_DEEP_UNROLL > NVSHMEMI_AMD_COPY_UNROLL
-    if (SRC_ALIGNED && (nthr & 63) == 0 && nvec >= (size_t)NVSHMEMI_AMD_COPY_DEEP_MIN * nthr) {
+    /* (the second bound follows from the first for whole wavefronts; spelled out, it lets the compiler drop
+     * the deep rounds and their registers where the caller's length is known to be short) */
+    if (SRC_ALIGNED && (nthr & 63) == 0 && nvec >= (size_t)NVSHMEMI_AMD_COPY_DEEP_MIN * nthr &&
+        nvec >= (size_t)NVSHMEMI_AMD_COPY_DEEP_MIN * 64) {
         const size_t done =
             stream_loads ? nvshmemi_amd_copy_deep_rounds<true, STORE, NVSHMEMI_AMD_COPY_DEEP_UNROLL>(
                                dst, src, nvec, (unsigned)tid, nthr)

@@ -37,7 +37,15 @@ __device__ __forceinline__ bool row_ok(int pe, int64_t row, int np, size_t cap_r
 // The wavefront's index is deliberately left a per-lane value: the routing entries indexed with it are
 // then fetched by vector loads of one address.  Making it a scalar (readfirstlane) turns them into
 // scalar loads, which measured 5 % slower here: the tables stream through the small scalar cache.
-__device__ __forceinline__ unsigned wave_in_block() { return threadIdx.x / NVSHMEMI_WARP_SIZE; }
+// (the same for every lane of a wavefront: as a scalar it keeps row indices, routing entries and the
+// addresses derived from them in scalar registers)
+__device__ __forceinline__ unsigned wave_in_block() {
+    return __builtin_amdgcn_readfirstlane(threadIdx.x / NVSHMEMI_WARP_SIZE);
+}
+// The same value left in a vector register: the routing entries are then fetched with vector loads.  The
+// kernel that pushes its rows with plain puts and signals once per block is 5 % faster that way (its few
+// long-lived wavefronts stream the tables through the small scalar cache otherwise), the others are not.
+__device__ __forceinline__ unsigned wave_in_block_per_lane() { return threadIdx.x / NVSHMEMI_WARP_SIZE; }
 
 // Dispatch.  Rows are dealt round-robin to the thread groups of the PE's blocks.  Each group tallies
 // what it sent to every destination; once all its puts are complete it adds the tallies to the
@@ -57,7 +65,7 @@ __global__ void moe_dispatch_kernel(char *recv, const char *send, const int32_t 
 
     if (WARP_SCOPED) {
         const size_t waves_per_block = blockDim.x / NVSHMEMI_WARP_SIZE;
-        const size_t wave = blockIdx.x * waves_per_block + wave_in_block();
+        const size_t wave = blockIdx.x * waves_per_block + wave_in_block_per_lane();
         const size_t nwaves = (size_t)gridDim.x * waves_per_block;
         const bool lane0 = (threadIdx.x % NVSHMEMI_WARP_SIZE) == 0;
         // A wavefront takes a token and pushes its topk copies back to back: the first put streams
@@ -288,10 +296,14 @@ __global__ void moe_combine_kernel(char *out, const char *recv, const int32_t *d
         const size_t wave = blockIdx.x * waves_per_block + wave_in_block();
         const size_t nwaves = (size_t)gridDim.x * waves_per_block;
         if (PIECE > 0) {
-            const size_t pieces = (row_bytes + PIECE - 1) / PIECE;
-            for (size_t item = wave; item < rows * pieces; item += nwaves) {
-                const size_t r = item / pieces, off = (item - r * pieces) * PIECE;
+            // (the item index is wave-uniform and, as the host entry point checks, below 2^32: a scalar
+            // 32-bit division instead of a 64-bit one per lane, which took some 40 vector registers)
+            const uint32_t pieces = (uint32_t)((row_bytes + PIECE - 1) / PIECE);
+            const uint32_t items = (uint32_t)rows * pieces;
+            for (uint32_t item = (uint32_t)wave; item < items; item += (uint32_t)nwaves) {
+                const size_t r = item / pieces, off = (size_t)(item - (uint32_t)r * pieces) * PIECE;
                 const size_t len = row_bytes - off < (size_t)PIECE ? row_bytes - off : (size_t)PIECE;
+                __builtin_assume(len <= (size_t)PIECE);   // short copies: the engine's long-copy code drops out
                 if (row_ok(my_dest_pe[r], my_dest_row[r], np, recv_cap_rows))
                     nvshmemx_getmem_nbi_warp(out + r * row_bytes + off,
                                              recv + (size_t)my_dest_row[r] * row_bytes + off, len,
@@ -542,6 +554,10 @@ int nvshmem_perftest_moe_combine_pieces(void *out, const void *recv, size_t recv
         !perftest::check_range(out, (size_t)tokens * (size_t)topk * row_bytes) ||
         !perftest::check_range(recv, recv_cap_rows * row_bytes))
         return NVSHMEMX_ERROR_INVALID_VALUE;
+    if (piece_bytes > 0 &&
+        (size_t)tokens * (size_t)topk * ((row_bytes + (size_t)piece_bytes - 1) / (size_t)piece_bytes) +
+                (size_t)blocks_per_pe * (size_t)(threads / NVSHMEMI_WARP_SIZE) > 0xffffffffull)
+        return NVSHMEMX_ERROR_INVALID_VALUE;   // the kernel counts work items in 32 bits
     const dim3 grid((unsigned)blocks_per_pe, 1, (unsigned)nvshmem_n_pes());
 #define LAUNCH_COMBINE(...)                                                                        \
     hipLaunchKernelGGL((moe_combine_kernel<__VA_ARGS__>), grid, dim3(threads), 0, (hipStream_t)stream, \
