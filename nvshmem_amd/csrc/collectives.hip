@@ -252,7 +252,9 @@ __global__ __launch_bounds__(NPES ? NPES / MPW * 64 : 1024) void reduce_vector_k
     constexpr uint32_t lane_shift = 6;  // a wavefront's 64 lanes move one aligned 1 KiB piece of a member
     constexpr unsigned lanes = 1u << lane_shift;
     // a wavefront serves MPW consecutive members (more than one only with a compile-time team size)
-    const unsigned pe0 = (threadIdx.x >> lane_shift) * MPW, i = threadIdx.x & (lanes - 1);
+    // (the wavefront's index as a scalar: the members' base addresses then stay in scalar registers)
+    const unsigned pe0 = (unsigned)__builtin_amdgcn_readfirstlane(threadIdx.x >> lane_shift) * MPW,
+                   i = threadIdx.x & (lanes - 1);
     const uint64_t nvec = nelems / VEC;
     // tiles are cut on absolute (16 * lanes)-byte boundaries of the destination, so a wavefront's
     // access is one aligned 1 KiB piece whatever the buffer's own alignment: `lead` vector slots of
