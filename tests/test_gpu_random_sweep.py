@@ -1,7 +1,12 @@
 """GPU parity on seeded random cases: host-launched collectives on random strided teams with random
 element types, operators, counts and byte offsets, each compared with the CPU oracle bit for bit
 (integers, copies) or bit for bit with the fixed PE order (floating point).  The cases are drawn from
-a fixed seed, so a failure names a reproducible case."""
+a fixed seed, so a failure names a reproducible case.  NVSHMEM_AMD_TEST_SEED_OFFSET shifts the seeds for a longer
+run over other cases; the kernel-selection thresholds can be lowered from the environment as for any program
+(NVSHMEM_AMD_LDS_REDUCE_BYTES=0 NVSHMEM_AMD_CACHEABLE_SOURCE_BYTES=0 sends these small messages through the
+kernels meant for large ones)."""
+import os
+
 import numpy as np
 import pytest
 
@@ -12,6 +17,7 @@ from nvshmem_amd.host import REDUCE_TYPES_BITWISE, REDUCE_TYPES_STANDARD, RMA_TY
 
 pytestmark = pytest.mark.gpu
 
+SEED_OFFSET = int(os.environ.get("NVSHMEM_AMD_TEST_SEED_OFFSET", "0"))
 CAP = 1 << 20          # bytes of source / destination per PE
 GUARD = 256
 
@@ -43,6 +49,7 @@ def _count(rng, limit):
 
 @pytest.mark.parametrize("npes,seed", [(4, 101), (5, 105), (8, 102), (12, 103), (16, 104), (33, 107), (64, 106)])
 def test_random_collectives_on_random_teams(npes, seed):
+    seed += SEED_OFFSET
     rng = np.random.default_rng(seed)
     world = (0, 1, npes)
     with runtime(npes, 4 * (CAP + 2 * GUARD) + (4 << 20)) as rt:
@@ -119,6 +126,7 @@ def test_random_collectives_on_random_teams(npes, seed):
 
 @pytest.mark.parametrize("npes,seed", [(6, 201), (8, 202), (16, 203)])
 def test_random_in_kernel_collectives(npes, seed):
+    seed += SEED_OFFSET
     """The same collectives called from inside a kernel (one block per PE) in a random scope with a
     random block size: float sum reduce / reducescatter and the untyped copies, sizes on both sides of
     the packet path's limit."""
