@@ -823,7 +823,7 @@ static int segment_collective(int mode, const char *what, nvshmem_team_t team, v
     // fcollect lets the wavefronts of one block share the piece (the same speed as neighbouring blocks,
     // measured 5.8-6.0 TB/s either way for 8 to 32 members, and the piece crosses the fabric once instead
     // of once per sharer); the broadcast keeps neighbouring blocks (6.05 against 5.5 TB/s)
-    const bool wave_split = part_shift != 0 && NVSHMEM_AMD_FCOLLECT_SPLIT == 2;
+    const bool wave_split = part_shift != 0 && NVSHMEM_AMD_FCOLLECT_SPLIT == 2 && (kCopyThreads << part_shift) <= 1024;
     const uint64_t tiles = ((seg_bytes / 16 + 64 + tile_vectors - 1) / tile_vectors + 1) << (wave_split ? 0 : part_shift);
     const unsigned segs = mode == kModeFcollect ? (unsigned)n : (unsigned)(n * n);
     if (tiles > 0x7fffffffull) {
