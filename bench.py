@@ -29,13 +29,16 @@ HBM_PEAK_GBS = 8000.0   # MI355X published HBM3E peak
 METRIC = "achieved GB/s and % of HBM peak: put_block, sum_reduce, alltoall (1 GPU)"
 
 
-def measured_traffic(name):
+def measured_traffic(name, fingerprint):
     """HBM bytes per launch of the workload's dominant kernel, from the rocprofv3 FETCH_SIZE / WRITE_SIZE
-    summary committed under profiles/ (None when there is none)."""
+    summary committed under profiles/.  None when there is no summary, or when the summary was measured
+    on kernel sources other than the ones in this tree (it records their fingerprint)."""
     for path in glob.glob(os.path.join(ROOT, "profiles", "*__%s.txt" % name)):
         with open(path) as fh:
-            m = re.search(r"^measured_traffic_bytes: (\d+) read \+ (\d+) written", fh.read(), re.M)
-        if m:
+            text = fh.read()
+        m = re.search(r"^measured_traffic_bytes: (\d+) read \+ (\d+) written", text, re.M)
+        f = re.search(r"^kernel_sources_fingerprint: (\w+)", text, re.M)
+        if m and f and f.group(1) == fingerprint:
             return int(m.group(1)) + int(m.group(2))
     return None
 
@@ -238,19 +241,60 @@ def oracle_moe_plan(O, np, npes, T, K, E):
     return dest_pe, dest_row, expected, recv_rows
 
 
-def summarise(item, wall, ev, ok, cpu):
+def summarise(item, wall, ev, ok, cpu, fingerprint):
     gbs = item.algorithmic_bytes / wall / 1e6
     kernel_gbs = item.algorithmic_bytes / ev / 1e6
     cfg = dict(item.config, workload=item.workload)
     if "bytes_per_pe" in item.config:
         cfg["payload_only_GBs"] = round(item.config["npes"] * item.config["bytes_per_pe"] / ev / 1e6, 1)
+    cached = bool(getattr(item, "cache_resident", False))      # then the rate is no HBM figure: no fraction
     return {
-        "GBs": round(gbs, 1), "frac_of_hbm_peak": round(gbs / HBM_PEAK_GBS, 4),
+        "GBs": round(gbs, 1), "frac_of_hbm_peak": None if cached else round(gbs / HBM_PEAK_GBS, 4),
         "ms_per_step": round(wall, 5), "kernel_ms": round(ev, 5), "kernel_GBs": round(kernel_gbs, 1),
-        "kernel_frac_of_hbm_peak": round(kernel_gbs / HBM_PEAK_GBS, 4),
-        "algorithmic_bytes": item.algorithmic_bytes, "traffic": measured_traffic(item.name),
+        "kernel_frac_of_hbm_peak": None if cached else round(kernel_gbs / HBM_PEAK_GBS, 4),
+        "cache_resident": cached,
+        "algorithmic_bytes": item.algorithmic_bytes, "traffic": measured_traffic(item.name, fingerprint),
         "dtype": item.dtype, "verified": ok, "config": cfg, "kernel": item.kernel, "cpu_baseline": cpu,
     }
+
+
+MAX_LINE_BYTES = 4096    # the result line is read back from a bounded tail of stdout
+
+
+def result_line(results, headline, warmup):
+    """The ONE result line, from the per-workload records of summarise(): the headline workload's figures
+    in full, every other workload as [kernel GB/s, fraction of the HBM peak or None when the working set
+    stays in the Infinity Cache, verified].  Kept well under MAX_LINE_BYTES; the full records are printed
+    on earlier lines."""
+    head = results[headline]
+    cpu = dict(head["cpu_baseline"])
+    config = {k: v for k, v in head["config"].items() if k != "note"}
+    line = {
+        "metric": METRIC,
+        "value": head["GBs"],
+        "unit": "GB/s",
+        "n_gpus": 1,
+        "steps": head["steps"],
+        "warmup": warmup,
+        "ms_per_step": head["ms_per_step"],
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": head["dtype"],
+        "data": "synthetic",
+        "config": config,
+        "roofline": {"bound": "hbm", "achieved": head["kernel_GBs"], "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                     "frac": round(head["kernel_GBs"] / HBM_PEAK_GBS, 4), "traffic": head["traffic"],
+                     "kernel": head["kernel"]},
+        "cpu_baseline": cpu,
+        "verified": all(r["verified"] for r in results.values()),
+        "workloads_format": "name: [kernel GB/s, fraction of HBM peak (null: cache resident), verified]",
+        "workloads": {name: [r["kernel_GBs"], r["kernel_frac_of_hbm_peak"], r["verified"]]
+                      for name, r in results.items()},
+    }
+    if len(json.dumps(line, separators=(",", ":"))) >= MAX_LINE_BYTES:
+        raise RuntimeError("bench.py: the result line outgrew %d bytes" % MAX_LINE_BYTES)
+    return line
 
 
 def main():
@@ -273,7 +317,9 @@ def main():
     import numpy as np
     import nvshmem_amd as N          # raises if the HIP libraries are not built
     from nvshmem_amd import hip, workloads
+    from nvshmem_amd.fingerprint import kernel_source_fingerprint
     import oracle_lib as O           # the checker / CPU baseline only
+    fingerprint = kernel_source_fingerprint()
 
     if hip.device_count() < 1:
         print("bench.py: no GPU visible", file=sys.stderr)
@@ -305,7 +351,7 @@ def main():
                                      "algorithmic_bytes": item.algorithmic_bytes})
                 ok = getattr(check, g.kind + "_verify")(g, item)
                 cpu = getattr(check, g.kind + "_baseline")(g, item)
-                results[item.name] = summarise(item, wall, ev, ok, cpu)
+                results[item.name] = summarise(item, wall, ev, ok, cpu, fingerprint)
                 results[item.name]["steps"] = steps
         finally:
             rt.finalize()
@@ -313,29 +359,11 @@ def main():
     if args.trace_manifest:
         with open(args.trace_manifest, "w") as fh:
             json.dump(manifest, fh, indent=1)
-    head = results[workloads.HEADLINE]
-    line = {
-        "metric": METRIC,
-        "value": head["GBs"],
-        "unit": "GB/s",
-        "n_gpus": 1,
-        "steps": head["steps"],
-        "warmup": args.warmup,
-        "ms_per_step": head["ms_per_step"],
-        "higher_is_better": True,
-        "scaling": "weak",
-        "vs_baseline": None,
-        "dtype": head["dtype"],
-        "data": "synthetic",
-        "config": head["config"],
-        "roofline": {"bound": "hbm", "achieved": head["kernel_GBs"], "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                     "frac": round(head["kernel_GBs"] / HBM_PEAK_GBS, 4), "traffic": head["traffic"],
-                     "kernel": head["kernel"]},
-        "cpu_baseline": head["cpu_baseline"],
-        "verified": all(r["verified"] for r in results.values()),
-        "workloads": results,
-    }
-    print(json.dumps(line))
+    for name, rec in results.items():          # the full records, one line per workload, before the result line
+        print(json.dumps({"workload_record": name, **rec}))
+    line = result_line(results, workloads.HEADLINE, args.warmup)
+    print(json.dumps(line, separators=(",", ":")))
+    sys.stdout.flush()
     return 0 if line["verified"] else 1
 
 

@@ -17,6 +17,10 @@ import json
 import os
 import re
 import sqlite3
+import sys
+
+sys.path.insert(0, os.path.dirname(os.path.dirname(os.path.abspath(__file__))))
+from nvshmem_amd.fingerprint import kernel_source_fingerprint  # noqa: E402
 
 MARKER = "profile_marker_kernel"
 CALIBRATION = "calibration"
@@ -161,6 +165,8 @@ def main():
             calls, avg, lo, hi, shape, vg = st[k]
             lines.append("%-58s %6d %11.2f %11.2f %11.2f  %dx%dx%d / %d, %s" % (k[:58], calls, avg, lo, hi, shape[0], shape[1],
                                                                             shape[2], shape[3], vg))
+        lines += ["", "kernel_sources_fingerprint: %s (nvshmem_amd/fingerprint.py, of the tree this was measured on)"
+                  % kernel_source_fingerprint()]
         lines += ["", "dominant kernel: " + dominant]
         calls, avg = st[dominant][0], st[dominant][1]
         step_us = sum(st[k][0] * st[k][1] for k in st) / max(1, entry["launches"])

@@ -25,6 +25,8 @@ class Item:
         self.kernel, self.workload, self.step = kernel, workload, step
         self.config = dict(config or {})
         self.scale = scale          # divides the requested number of steps (very long steps)
+        self.cache_resident = False  # True: the working set stays in the 256 MiB Infinity Cache between steps,
+                                     # so its rate is not an HBM figure and no fraction of the HBM peak is quoted
 
 
 class Group:
@@ -133,6 +135,7 @@ class Reduce(Group):
                       % (name, type_name, op, self.npes, self.n, self.tag), step,
                       {"npes": self.npes, "nreduce": self.n, "type": type_name, "op": op})
             it.prepare, it.oracle_dtype, it.op, it.elem_bytes = prepare, kind, op, es
+            it.cache_resident = 2 * self.npes * self.n * es <= 256 * MiB
             items.append(it)
         return items
 
@@ -180,6 +183,7 @@ class Collect(Group):
                                 "not an HBM-bound figure" % (npes * n * es // MiB) if cached else
                                 "sources larger than the Infinity Cache: HBM-bound")})]
         items[0].what = "alltoall"
+        items[0].cache_resident = cached
         if self.with_fcollect:
             self.fc_dst = rt.malloc(npes * n * es)
             fc = _lib.typed_coll(rt.lib, "nvshmemx_%s_fcollect_on_stream" % self.type_name, True)
