@@ -272,13 +272,29 @@ NVSHMEMI_DEVICE_INLINE size_t nvshmemi_amd_copy_rounds(char *__restrict__ dst,
 #define NVSHMEMI_AMD_COPY_NT_ALWAYS false
 #endif
 
-/* Deep rounds of a long copy by whole wavefronts: per round the group moves U * nthr consecutive
- * vectors, of which wavefront w owns the U KiB [w * U, (w + 1) * U) and moves them with U loads issued
- * back to back, then U stores.  The wavefront's base addresses are wave-uniform (scalar registers) and a
- * lane adds its 16 * lane and a constant u * 1024, so the U vectors in flight cost 4 U vector registers
- * and no address registers of their own (one address pair per vector made the compiler serialise the
- * round to stay within its register budget).  Returns the number of vectors moved, a multiple of
- * U * nthr. */
+/* Deep rounds of a long copy by whole wavefronts: per round the group moves U * nthr consecutive vectors
+ * with U loads per lane issued back to back, then U stores.  All addresses are wave-uniform bases (scalar
+ * registers) plus the lane's 16 * lane, so the U vectors in flight cost 4 U vector registers and no
+ * address registers of their own (one address pair per vector made the compiler serialise the round to
+ * stay within its register budget).  Returns the number of vectors moved, a multiple of U * nthr.
+ *
+ * Two layouts of a round:
+ * - blocks of fewer than NVSHMEMI_AMD_COPY_PHASED_THREADS threads: wavefront w owns the U consecutive KiB
+ *   [w * U, (w + 1) * U) of the round;
+ * - larger blocks (block scope only): the u-th instruction of all wavefronts covers the nthr * 16
+ *   consecutive bytes [u * nthr * 16, (u + 1) * nthr * 16), wavefront w its w-th KiB, so the block sweeps the
+ *   round in address order, and the wavefronts stay in step: they meet after the loads of a round are
+ *   issued and again after its stores are issued, so the compute unit's memory pipeline sees the round as
+ *   one run of loads followed by one run of stores instead of the two interleaved.  Interleaved, the
+ *   stores' acknowledgements take as long as the loads between them (L1-to-L2 write latency 950 cycles
+ *   against 320 in runs) and fill the L1's store queue, which then holds up the loads behind it.  16 blocks
+ *   of 1024 threads per PE move 4.73 TB/s interleaved, 5.56 in runs and 6.05 in runs swept in address order;
+ *   one such block 61, 77 and 78 GB/s.  Blocks of 256 threads or fewer share their compute unit with other
+ *   blocks, whose requests interleave anyway: neither the barriers nor the sweep changes their rate.  (The
+ *   number of rounds is the same for every wavefront of the block, so all of them reach every barrier.) */
+#ifndef NVSHMEMI_AMD_COPY_PHASED_THREADS
+#define NVSHMEMI_AMD_COPY_PHASED_THREADS 512
+#endif
 template <bool NT_LOAD, int STORE, int U, bool BLOCK_WIDE>
 NVSHMEMI_DEVICE_INLINE size_t nvshmemi_amd_copy_deep_rounds(char *__restrict__ dst, const char *__restrict__ src,
                                                            size_t nvec, unsigned tid, size_t nthr) {
@@ -286,8 +302,11 @@ NVSHMEMI_DEVICE_INLINE size_t nvshmemi_amd_copy_deep_rounds(char *__restrict__ d
     const size_t rounds = nvec / per_round;
     const size_t wave = (size_t)__builtin_amdgcn_readfirstlane(tid >> 6);
     const unsigned lane_off = (tid & 63u) * 16u;
-    const char *s0 = src + wave * (size_t)(U * 1024);
-    char *d0 = dst + wave * (size_t)(U * 1024);
+    const bool phased = BLOCK_WIDE && nthr >= NVSHMEMI_AMD_COPY_PHASED_THREADS;
+    const size_t step = phased ? nthr * 16 : (size_t)1024;              /* from one instruction to the next */
+    const size_t wave_off = wave * (phased ? (size_t)1024 : (size_t)(U * 1024));
+    const char *s0 = src + wave_off;
+    char *d0 = dst + wave_off;
     /* The rounds are walked from a start that differs from block to block, wrapping at the end.  Blocks
      * that each stream a slice of one large message otherwise march in step, at equal offsets in slices
      * that lie a power of two (or the PE distance) apart, and keep meeting on the same memory channels. */
@@ -299,29 +318,16 @@ NVSHMEMI_DEVICE_INLINE size_t nvshmemi_amd_copy_deep_rounds(char *__restrict__ d
         const unsigned h = (blockIdx.x * 0x9E3779B1u) ^ (blockIdx.y * 0x85EBCA77u) ^ (blockIdx.z * 0xC2B2AE3Du);
         r = (size_t)(((uint64_t)h * (uint64_t)(rounds & 0xffffffffu)) >> 32);  /* in [0, rounds) */
     }
-    /* A block of NVSHMEMI_AMD_COPY_PHASED_THREADS threads or more keeps its wavefronts in step: they meet
-     * after the loads of a round are issued and again after its stores are issued, so the compute unit's
-     * memory pipeline sees the round as one run of loads followed by one run of stores instead of the two
-     * interleaved.  Interleaved, the stores' acknowledgements take as long as the loads between them
-     * (L1-to-L2 write latency 950 cycles against 320 in runs) and fill the L1's store queue, which then holds
-     * up the loads behind it: 16 blocks of 1024 threads per PE move 4.73 TB/s interleaved and 5.56 in runs,
-     * one such block 61 against 77 GB/s.  Blocks of 256 threads or fewer share their compute unit with
-     * other blocks, whose requests interleave anyway; they gain nothing and skip the barriers.  (The
-     * number of rounds is the same for every wavefront of the block, so all of them reach every barrier.) */
-#ifndef NVSHMEMI_AMD_COPY_PHASED_THREADS
-#define NVSHMEMI_AMD_COPY_PHASED_THREADS 512
-#endif
-    const bool phased = BLOCK_WIDE && nthr >= NVSHMEMI_AMD_COPY_PHASED_THREADS;
     for (size_t k = 0; k < rounds; ++k) {
         const char *s = s0 + r * (16 * per_round);
         char *d = d0 + r * (16 * per_round);
         if (++r == rounds) r = 0;
         nvshmemi_v4u v[U];
 #pragma unroll
-        for (int u = 0; u < U; ++u) v[u] = nvshmemi_amd_stream_load16<true, NT_LOAD>(s + u * 1024 + lane_off);
+        for (int u = 0; u < U; ++u) v[u] = nvshmemi_amd_stream_load16<true, NT_LOAD>(s + u * step + lane_off);
         if (BLOCK_WIDE && phased) asm volatile("s_barrier" ::: "memory");
 #pragma unroll
-        for (int u = 0; u < U; ++u) nvshmemi_amd_stream_store16<STORE>(d + u * 1024 + lane_off, v[u]);
+        for (int u = 0; u < U; ++u) nvshmemi_amd_stream_store16<STORE>(d + u * step + lane_off, v[u]);
         if (BLOCK_WIDE && phased) asm volatile("s_barrier" ::: "memory");
     }
     return rounds * per_round;
