@@ -44,7 +44,20 @@ namespace {
 #define NVSHMEM_AMD_REDUCE_VPT 1
 #endif
 #ifndef NVSHMEM_AMD_REDUCE_VPT_NARROW /* the same for 1- and 2-byte elements on the compile-time team sizes 8 and 16 */
-#define NVSHMEM_AMD_REDUCE_VPT_NARROW 2
+#define NVSHMEM_AMD_REDUCE_VPT_NARROW 1
+#endif
+/* Members per wavefront of the fused reduce on the compile-time team sizes 8 and 16, for 1- and 2-byte
+ * elements (NARROW) and for wider ones (WIDE).  Narrow elements fold twice to four times as many elements
+ * per byte, and a block has nothing in flight while it folds: with two members per wavefront the blocks
+ * are half as large and twice as many share a compute unit, so more of them are in their load or store
+ * phase at any time (bf16 sum and max, 8 x 128 MiB: 6.05-6.15 TB/s with one member per wavefront and two
+ * vectors per thread, 6.21-6.25 with two members and one vector; four members 5.74-5.96).  4- and 8-byte
+ * elements lose 5 % with two members per wavefront and 11 % with four. */
+#ifndef NVSHMEM_AMD_REDUCE_NARROW_MPW
+#define NVSHMEM_AMD_REDUCE_NARROW_MPW 2
+#endif
+#ifndef NVSHMEM_AMD_REDUCE_WIDE_MPW
+#define NVSHMEM_AMD_REDUCE_WIDE_MPW 1
 #endif
 #ifndef NVSHMEM_AMD_COLL_NT /* bit 0: non-temporal loads allowed, bit 1: non-temporal stores */
 #define NVSHMEM_AMD_COLL_NT 3
@@ -271,9 +284,14 @@ __global__ __launch_bounds__(NPES ? NPES / MPW * 64 : 1024) void reduce_vector_k
     const uint64_t ntiles = (nvec + lead + tile_vecs - 1) / tile_vecs;
     nvshmemi_v4u *stage = reinterpret_cast<nvshmemi_v4u *>(lds);           // [npes][tile_vecs]
     nvshmemi_v4u *result = stage + (size_t)npes * tile_vecs;               // [tile_vecs]
-    const T *stage_e = reinterpret_cast<const T *>(stage);
-    T *result_e = reinterpret_cast<T *>(result);
-    constexpr unsigned tile_elems = tile_vecs * VEC;
+    // the unit of the fold: a 4-byte word (EPW elements) for 1- and 2-byte elements, else one element
+    constexpr int EPW = sizeof(T) < 4 ? 4 / (int)sizeof(T) : 1;
+    struct alignas(sizeof(T) * EPW) word_t {
+        T e[EPW];
+    };
+    const word_t *stage_w = reinterpret_cast<const word_t *>(stage);
+    word_t *result_w = reinterpret_cast<word_t *>(result);
+    constexpr unsigned tile_words = tile_vecs * VEC / EPW;
 
     for (uint64_t tile = blockIdx.x; tile < ntiles; tile += gridDim.x) {
         // indices in front of the buffer wrap to huge values and are skipped like those behind it
@@ -289,26 +307,37 @@ __global__ __launch_bounds__(NPES ? NPES / MPW * 64 : 1024) void reduce_vector_k
             }
         }
         __syncthreads();
-        for (unsigned e = threadIdx.x; e < tile_elems; e += blockDim.x) {
-            T acc = stage_e[e];
+        // a thread folds one 4-byte word of the tile at a time - one element of 4 or 8 bytes, or the 2 or 4
+        // narrower elements that share the word, each folded on its own in member order - so that a tile of
+        // 1- or 2-byte elements costs as many LDS instructions as one of 4-byte elements
+        for (unsigned w = threadIdx.x; w < tile_words; w += blockDim.x) {
+            word_t acc = stage_w[w];
             if (NPES) {
 #pragma unroll
-                for (int p = 1; p < NPES; ++p)
-                    acc = nvshmemi_amd_fold_step<T, OP>(p, acc, stage_e[(size_t)p * tile_elems + e]);
+                for (int p = 1; p < NPES; ++p) {
+                    const word_t x = stage_w[(size_t)p * tile_words + w];
+#pragma unroll
+                    for (int j = 0; j < EPW; ++j) acc.e[j] = nvshmemi_amd_fold_step<T, OP>(p, acc.e[j], x.e[j]);
+                }
             } else {
                 // eight members' values fetched from LDS before they are folded, in member order
                 int p = 1;
                 for (; p + 8 <= npes; p += 8) {
-                    T x[8];
+                    word_t x[8];
 #pragma unroll
-                    for (int k = 0; k < 8; ++k) x[k] = stage_e[(size_t)(p + k) * tile_elems + e];
+                    for (int k = 0; k < 8; ++k) x[k] = stage_w[(size_t)(p + k) * tile_words + w];
 #pragma unroll
-                    for (int k = 0; k < 8; ++k) acc = nvshmemi_amd_fold_step<T, OP>(p + k, acc, x[k]);
+                    for (int k = 0; k < 8; ++k)
+#pragma unroll
+                        for (int j = 0; j < EPW; ++j) acc.e[j] = nvshmemi_amd_fold_step<T, OP>(p + k, acc.e[j], x[k].e[j]);
                 }
-                for (; p < npes; ++p)
-                    acc = nvshmemi_amd_fold_step<T, OP>(p, acc, stage_e[(size_t)p * tile_elems + e]);
+                for (; p < npes; ++p) {
+                    const word_t x = stage_w[(size_t)p * tile_words + w];
+#pragma unroll
+                    for (int j = 0; j < EPW; ++j) acc.e[j] = nvshmemi_amd_fold_step<T, OP>(p, acc.e[j], x.e[j]);
+                }
             }
-            result_e[e] = acc;
+            result_w[w] = acc;
         }
         __syncthreads();
 #pragma unroll
@@ -523,7 +552,8 @@ void launch_reduce(Runtime &rt, const TeamLaunch &tl, uint64_t dst_off, uint64_t
     // The threshold counts elements (as 4-byte ones): narrow types fold more elements per byte.
     // mpw: members per wavefront of the LDS-staged kernel; ct_size: a compile-time team size, if any
     int mpw = 0, ct_size = 0;
-    if (fixed_size == 8 || fixed_size == 16) ct_size = fixed_size, mpw = 1;
+    constexpr int kNarrowMpw = sizeof(T) <= 2 ? NVSHMEM_AMD_REDUCE_NARROW_MPW : NVSHMEM_AMD_REDUCE_WIDE_MPW;
+    if (fixed_size == 8 || fixed_size == 16) ct_size = fixed_size, mpw = kNarrowMpw;
     else if (fixed_size == 32) ct_size = 32, mpw = 2;
     else if (tl.max_size >= 3 && tl.max_size <= 32) mpw = 2;
     else if (tl.max_size > 32 && tl.max_size <= 64) mpw = 4;
@@ -531,9 +561,9 @@ void launch_reduce(Runtime &rt, const TeamLaunch &tl, uint64_t dst_off, uint64_t
         const uint32_t lane_shift = 6;
         const unsigned threads = (unsigned)((tl.max_size + mpw - 1) / mpw) << lane_shift;
         const uint64_t nvec = nelems / (16 / sizeof(T));
-        // A tile of two vectors per thread halves the barriers per byte: worth 5 % for 16-bit elements, whose
-        // folds are twice as many per byte (bf16 sum at 8 x 128 MiB 5.83 -> 6.14 TB/s), and costs 4-byte and
-        // 8-byte elements 3-4 %.
+        // A tile of two vectors per thread halves the barriers per byte: worth 5 % for 16-bit elements with one
+        // member per wavefront (bf16 sum at 8 x 128 MiB 5.83 -> 6.14 TB/s), less than the two members per
+        // wavefront they now use with one vector; it costs 4-byte and 8-byte elements 3-4 %.
         constexpr int kVptNarrow = sizeof(T) <= 2 ? NVSHMEM_AMD_REDUCE_VPT_NARROW : NVSHMEM_AMD_REDUCE_VPT;
         const int vpt = (ct_size == 8 || ct_size == 16) ? kVptNarrow : NVSHMEM_AMD_REDUCE_VPT;
         const uint64_t tile_vecs = (uint64_t)vpt << lane_shift;
@@ -553,8 +583,8 @@ void launch_reduce(Runtime &rt, const TeamLaunch &tl, uint64_t dst_off, uint64_t
                                stream, rt.base, rt.heap_size, tl.groups, dst_off,    \
                                src_off, nelems);                                                  \
     } while (0)
-        if (ct_size == 8) NVSHMEM_AMD_LAUNCH_REDUCE_V(8, 1, kVptNarrow);
-        else if (ct_size == 16) NVSHMEM_AMD_LAUNCH_REDUCE_V(16, 1, kVptNarrow);
+        if (ct_size == 8) NVSHMEM_AMD_LAUNCH_REDUCE_V(8, kNarrowMpw, kVptNarrow);
+        else if (ct_size == 16) NVSHMEM_AMD_LAUNCH_REDUCE_V(16, kNarrowMpw, kVptNarrow);
         else if (ct_size == 32) NVSHMEM_AMD_LAUNCH_REDUCE(32, 2);
         else if (mpw == 2) NVSHMEM_AMD_LAUNCH_REDUCE(0, 2);
         else NVSHMEM_AMD_LAUNCH_REDUCE(0, 4);
