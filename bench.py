@@ -193,6 +193,7 @@ class Checker:
 
     # -- MoE -----------------------------------------------------------------------------------
     def moe_prepare(self, g, item):
+        item.prepare()
         if item.what != "combine":
             g.rt.fill(g.recv, 0, g.cap * g.row)
 
@@ -200,9 +201,11 @@ class Checker:
         np, rt = self.np, g.rt
         npes, K, row, rows = g.npes, g.K, g.row, g.rows
         ok = all(rt.read_timeout(pe)[0] == 0 for pe in range(npes))
-        if item.what == "put_signal":
+        if item.what in ("put_signal", "put_signal_head"):
             sig = rt.download_all(g.sig, (npes * g.SIG_STRIDE,), np.uint64)[:, ::g.SIG_STRIDE]
-            ok = ok and bool(np.array_equal(sig, g.expected))
+            ok = ok and bool(np.array_equal(sig, g.expected if item.what == "put_signal" else g.expected_head))
+        if item.what == "put_signal_head":
+            rows = g.FULL_ORDER_TOKENS * K       # only the first tokens were sent
         elif item.what == "plain_store":
             ok = ok and bool(np.array_equal(rt.download_all(g.sig, (npes,), np.uint64), g.expected))
         rng = np.random.default_rng(0)

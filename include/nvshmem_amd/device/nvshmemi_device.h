@@ -163,7 +163,10 @@ NVSHMEMI_DEVICE_INLINE void *nvshmemi_ptr(const void *ptr, int pe) {
 typedef unsigned int nvshmemi_v4u __attribute__((ext_vector_type(4)));
 typedef nvshmemi_v4u __attribute__((aligned(1))) nvshmemi_v4u_unaligned;
 
-/* Vectors per lane and round of the ordinary body. */
+/* Vectors per lane and round of the ordinary body.  A translation unit whose calls move rows of a known
+ * size does best with the number of vectors a lane moves per call - a 14 KiB row per wavefront: 14 - so
+ * that a call is one run of loads followed by one run of stores (the token dispatch with a signal per row:
+ * 4.53 TB/s at 8, 4.90 at 14; the price is 4 vector registers per vector). */
 #ifndef NVSHMEMI_AMD_COPY_UNROLL
 #define NVSHMEMI_AMD_COPY_UNROLL 4
 #endif
@@ -259,8 +262,10 @@ NVSHMEMI_DEVICE_INLINE size_t nvshmemi_amd_copy_rounds(char *__restrict__ dst,
 #pragma unroll
         for (int u = 0; u < U; ++u) nvshmemi_amd_stream_store16<STORE>(dst + 16 * (i + u * nthr), v[u]);
     }
+    /* next depth: half of a power of two, else the largest power of two below U (14 -> 8 -> 4 -> 2 -> 1) */
+    constexpr int NEXT = (U & (U - 1)) ? (U >= 16 ? 16 : U >= 8 ? 8 : U >= 4 ? 4 : 2) : U / 2;
     if constexpr (CASCADE && U > 1)
-        return nvshmemi_amd_copy_rounds<SRC_ALIGNED, NT_LOAD, STORE, U / 2, true>(dst, src, nvec, i, nthr);
+        return nvshmemi_amd_copy_rounds<SRC_ALIGNED, NT_LOAD, STORE, NEXT, true>(dst, src, nvec, i, nthr);
     return i;
 }
 
@@ -544,13 +549,17 @@ NVSHMEMI_DEVICE_INLINE void nvshmemi_signal_op_release(uint64_t *sig_addr, uint6
  *    meanwhile: a token dispatch that signals each 14 KiB row took 17-24 ms with a release per row
  *    (whether the payload was streamed or written through, and also when the wavefronts of an XCD
  *    shared write-backs through a ticket lock: a write-back under that load takes some 20 us), against
- *    1.7 ms with one release per block.  Without the fence the per-row form takes a few ms. */
+ *    1.7 ms with one release per block.  Without the fence the per-row form takes a few ms.
+ *    The library-wide option NVSHMEMI_AMD_OPTION_PUT_SIGNAL_PAYLOAD_ONLY (set from the environment or by
+ *    nvshmemx_amd_set_put_signal_order) selects this order for every call, for programs that cannot
+ *    edit their call sites. */
 template <typename T, int SCOPE>
 NVSHMEMI_DEVICE_INLINE void nvshmemi_put_signal(T *dest, const T *source, size_t nelems,
                                                 uint64_t *sig_addr, uint64_t signal, int sig_op,
                                                 int pe) {
     nvshmemi_threadgroup_sync<SCOPE>();
-    if (sig_op & NVSHMEMX_AMD_SIGNAL_PAYLOAD_ONLY) {
+    if ((sig_op & NVSHMEMX_AMD_SIGNAL_PAYLOAD_ONLY) ||
+        (nvshmemi_device_state_d.options & NVSHMEMI_AMD_OPTION_PUT_SIGNAL_PAYLOAD_ONLY)) {
         nvshmemi_memcpy_threadgroup<SCOPE, NVSHMEMI_AMD_STORE_WRITE_THROUGH>(
             nvshmemi_amd_remote(dest, pe), nvshmemi_amd_local(source), nelems * sizeof(T));
         nvshmemi_amd_wait_vm();

@@ -61,6 +61,11 @@ typedef enum {
  * the XCD's L2 per call.  No counterpart in the reference. */
 #define NVSHMEMX_AMD_SIGNAL_PAYLOAD_ONLY 0x100
 #define NVSHMEMI_AMD_SIGNAL_OP_MASK 0xff
+/* nvshmemi_device_state_t::options, bit 0: every device-side put-with-signal takes the payload-only order,
+ * as if NVSHMEMX_AMD_SIGNAL_PAYLOAD_ONLY were OR-ed into its sig_op (NVSHMEM_AMD_PUT_SIGNAL_ORDER=payload
+ * in the environment at nvshmem_init, or nvshmemx_amd_set_put_signal_order), so that code written for the
+ * reference's API can choose it without touching its call sites. */
+#define NVSHMEMI_AMD_OPTION_PUT_SIGNAL_PAYLOAD_ONLY 0x1u
 
 typedef int32_t nvshmem_team_t;
 #define NVSHMEM_TEAM_INVALID (-1)

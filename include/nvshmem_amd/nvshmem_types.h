@@ -232,7 +232,7 @@ typedef struct nvshmemi_device_state {
     uint32_t version;     /* (1 << 16) + sizeof(struct) */
     int32_t mype;         /* PE a kernel acts as when its grid is not PE-multiplexed */
     int32_t npes;
-    uint32_t options;     /* reserved, 0 */
+    uint32_t options;     /* NVSHMEMI_AMD_OPTION_* bits */
     char *heap_base;      /* start of PE 0's slice */
     uint64_t heap_size;   /* bytes from one PE's slice to the next (a multiple of 2 MiB, of 16 MiB for large heaps) */
     uint64_t *sync_flags; /* canonical address: NVSHMEMI_AMD_MAX_PES arrival words per PE */

@@ -94,6 +94,8 @@ def load():
         "nvshmemx_amd_collective_launch_query_gridsize": (i32, [vp] + [C.c_uint] * 3 + [sz, C.POINTER(i32)]),
         "nvshmemx_amd_module_init": (i32, []),
         "nvshmemx_amd_set_spin_limit": (None, [u64]),
+        "nvshmemx_amd_set_put_signal_order": (None, [i32]),
+        "nvshmemx_amd_get_put_signal_order": (i32, []),
         "nvshmemx_amd_read_timeout": (u64, [i32, C.POINTER(u64)]),
         "nvshmemx_amd_last_error": (C.c_char_p, []),
         "nvshmemi_amd_mspace_create": (vp, [u64, u64]),

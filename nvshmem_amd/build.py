@@ -29,7 +29,7 @@ HIP_FLAGS = [
 
 RUNTIME_SOURCES = ["mspace.cpp", "runtime.hip", "teams.cpp", "collectives.hip", "host_rma.hip"]
 PERFTEST_SOURCES = ["perftest/rma_kernels.hip", "perftest/coll_kernels.hip",
-                    "perftest/moe_shuffle.hip", "perftest/api_matrix.hip",
+                    "perftest/moe_shuffle.hip", "perftest/moe_rowsignal.hip", "perftest/api_matrix.hip",
                     "perftest/amo_kernels.hip"]
 
 

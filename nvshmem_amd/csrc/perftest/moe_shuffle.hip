@@ -11,11 +11,13 @@
 #include <cstdlib>
 
 // A row is 14 vectors per lane: rounds of 8 + 4 + 2 keep more loads in flight than the default
-// 4 + 4 + 4 + 2 (measured 5 % faster for dispatch and combine).
+// 4 + 4 + 4 + 2 (measured 5 % faster for dispatch and combine).  (The kernel that signals every row is
+// built with rounds of 14 in a translation unit of its own, moe_rowsignal.hip.)
 #define NVSHMEMI_AMD_COPY_UNROLL 8
 
 #include "nvshmem_perftest.h"
 #include "nvshmemx.h"
+#include "moe_common.hpp"
 #include "perftest_common.hpp"
 
 // Signal words of the dispatch that allocates nothing (nvshmem_perftest_moe_dispatch_pieces_static):
@@ -28,24 +30,6 @@ static __device__ __align__(256) uint64_t scratch[kStaticSignalPes * kStaticSign
 namespace {
 
 constexpr int kMaxPes = NVSHMEMI_AMD_MAX_PES;
-
-// A routing entry that points outside the receive buffer is skipped instead of written.
-__device__ __forceinline__ bool row_ok(int pe, int64_t row, int np, size_t cap_rows) {
-    return (unsigned)pe < (unsigned)np && (uint64_t)row < (uint64_t)cap_rows;
-}
-
-// The wavefront's index is deliberately left a per-lane value: the routing entries indexed with it are
-// then fetched by vector loads of one address.  Making it a scalar (readfirstlane) turns them into
-// scalar loads, which measured 5 % slower here: the tables stream through the small scalar cache.
-// (the same for every lane of a wavefront: as a scalar it keeps row indices, routing entries and the
-// addresses derived from them in scalar registers)
-__device__ __forceinline__ unsigned wave_in_block() {
-    return __builtin_amdgcn_readfirstlane(threadIdx.x / NVSHMEMI_WARP_SIZE);
-}
-// The same value left in a vector register: the routing entries are then fetched with vector loads.  The
-// kernel that pushes its rows with plain puts and signals once per block is 5 % faster that way (its few
-// long-lived wavefronts stream the tables through the small scalar cache otherwise), the others are not.
-__device__ __forceinline__ unsigned wave_in_block_per_lane() { return threadIdx.x / NVSHMEMI_WARP_SIZE; }
 
 // Dispatch.  Rows are dealt round-robin to the thread groups of the PE's blocks.  Each group tallies
 // what it sent to every destination; once all its puts are complete it adds the tallies to the
@@ -101,45 +85,6 @@ __global__ void moe_dispatch_kernel(char *recv, const char *send, const int32_t 
         const uint64_t *my_expected = (const uint64_t *)nvshmem_ptr(expected, me);
         for (int src = threadIdx.x; src < np; src += blockDim.x)
             nvshmem_signal_wait_until(sig + src, NVSHMEM_CMP_GE, my_expected[src]);
-    }
-}
-
-// Per-row signalling: the API-literal form, one nvshmemx_putmem_signal_nbi per row.
-template <bool WARP_SCOPED>
-__global__ void moe_dispatch_rowsignal_kernel(char *recv, const char *send, const int32_t *dest_pe,
-                                              const int64_t *dest_row, const uint64_t *expected,
-                                              uint64_t *sig, int tokens, int topk,
-                                              size_t row_bytes, size_t recv_cap_rows, int sig_op,
-                                              int sig_stride) {
-    const int me = nvshmem_my_pe(), np = nvshmem_n_pes();
-    const int32_t *my_dest_pe = (const int32_t *)nvshmem_ptr(dest_pe, me);
-    const int64_t *my_dest_row = (const int64_t *)nvshmem_ptr(dest_row, me);
-    const size_t rows = (size_t)tokens * (size_t)topk;
-    if (WARP_SCOPED) {
-        const size_t waves_per_block = blockDim.x / NVSHMEMI_WARP_SIZE;
-        const size_t wave = blockIdx.x * waves_per_block + wave_in_block();
-        const size_t nwaves = (size_t)gridDim.x * waves_per_block;
-        // a wavefront takes a token and sends its topk copies one behind the other, so that the
-        // copies after the first find the row in this XCD's L2
-        for (size_t t = wave; t < (size_t)tokens; t += nwaves)
-            for (int k = 0; k < topk; ++k) {
-                const size_t r = t * (size_t)topk + (size_t)k;
-                if (row_ok(my_dest_pe[r], my_dest_row[r], np, recv_cap_rows))
-                    nvshmemx_putmem_signal_nbi_warp(recv + (size_t)my_dest_row[r] * row_bytes,
-                                                    send + t * row_bytes, row_bytes,
-                                                    sig + (size_t)me * sig_stride, 1, sig_op, my_dest_pe[r]);
-            }
-    } else {
-        for (size_t r = blockIdx.x; r < rows; r += gridDim.x)
-            if (row_ok(my_dest_pe[r], my_dest_row[r], np, recv_cap_rows))
-            nvshmemx_putmem_signal_nbi_block(recv + (size_t)my_dest_row[r] * row_bytes,
-                                             send + (r / (size_t)topk) * row_bytes, row_bytes,
-                                             sig + (size_t)me * sig_stride, 1, sig_op, my_dest_pe[r]);
-    }
-    if (blockIdx.x == 0) {
-        const uint64_t *my_expected = (const uint64_t *)nvshmem_ptr(expected, me);
-        for (int src = threadIdx.x; src < np; src += blockDim.x)
-            nvshmem_signal_wait_until(sig + (size_t)src * sig_stride, NVSHMEM_CMP_GE, my_expected[src]);
     }
 }
 
@@ -415,12 +360,8 @@ int nvshmem_perftest_moe_dispatch_put_signal(void *recv, size_t recv_cap_rows, c
     const char *s = (const char *)send;
     void *args[] = {&r, &s, &dest_pe, &dest_row, &expected, &sig, &tokens, &topk, &row_bytes,
                     &recv_cap_rows, &sig_op, &sig_stride};
-    const void *fn;
-    if (per_row)
-        fn = warp ? (const void *)moe_dispatch_rowsignal_kernel<true>
-                  : (const void *)moe_dispatch_rowsignal_kernel<false>;
-    else
-        fn = warp ? (const void *)moe_dispatch_kernel<true> : (const void *)moe_dispatch_kernel<false>;
+    if (per_row) return perftest::launch_moe_rowsignal(warp, blocks_per_pe, threads, args, (hipStream_t)stream);
+    const void *fn = warp ? (const void *)moe_dispatch_kernel<true> : (const void *)moe_dispatch_kernel<false>;
     return nvshmemx_collective_launch(fn, dim3(blocks_per_pe), dim3(threads), args, 0,
                                       (hipStream_t)stream);
 }

@@ -230,6 +230,12 @@ int nvshmemx_amd_init(int npes, size_t symmetric_size) {
     rt.dev.runtime_words = (uint64_t *)(uintptr_t)(trec + NVSHMEMI_MALLOC_ALIGNMENT);
     rt.dev.spin_limit = env_size("NVSHMEM_AMD_SPIN_LIMIT", 1ull << 22);
     rt.dev.options = 0;
+    if (const char *order = getenv("NVSHMEM_AMD_PUT_SIGNAL_ORDER")) {
+        if (!strcmp(order, "payload")) rt.dev.options |= NVSHMEMI_AMD_OPTION_PUT_SIGNAL_PAYLOAD_ONLY;
+        else if (strcmp(order, "full") && *order)
+            fprintf(stderr, "nvshmem_amd: NVSHMEM_AMD_PUT_SIGNAL_ORDER=%s is neither \"payload\" nor \"full\"; "
+                            "using full\n", order);
+    }
     rt.dev.heap_magic = (1ull << 40) / (rt.heap_size >> 21) + 1;
     rt.plain_collective_launch = env_size("NVSHMEM_AMD_PLAIN_COLLECTIVE_LAUNCH", 0) != 0;
     rt.cacheable_source_bytes = env_size("NVSHMEM_AMD_CACHEABLE_SOURCE_BYTES", (size_t)256 << 20);
@@ -319,6 +325,23 @@ void nvshmemx_vendor_get_version_info(int *major, int *minor, int *patch) {
     if (major) *major = NVSHMEM_VENDOR_MAJOR_VERSION;
     if (minor) *minor = NVSHMEM_VENDOR_MINOR_VERSION;
     if (patch) *patch = NVSHMEM_VENDOR_PATCH_VERSION;
+}
+
+void nvshmemx_amd_set_put_signal_order(int payload_only) {
+    Runtime &rt = Runtime::get();
+    std::lock_guard<std::recursive_mutex> lock(rt.mu);
+    if (payload_only) rt.dev.options |= NVSHMEMI_AMD_OPTION_PUT_SIGNAL_PAYLOAD_ONLY;
+    else rt.dev.options &= ~NVSHMEMI_AMD_OPTION_PUT_SIGNAL_PAYLOAD_ONLY;
+    if (rt.initialized) {
+        NVSHMEM_AMD_HIP_CHECK(hipDeviceSynchronize());
+        refresh_symbols(rt, true);
+    }
+}
+
+int nvshmemx_amd_get_put_signal_order(void) {
+    Runtime &rt = Runtime::get();
+    std::lock_guard<std::recursive_mutex> lock(rt.mu);
+    return (rt.dev.options & NVSHMEMI_AMD_OPTION_PUT_SIGNAL_PAYLOAD_ONLY) ? 1 : 0;
 }
 
 void nvshmemx_amd_set_spin_limit(uint64_t polls) {

@@ -267,8 +267,11 @@ class MoeShuffle(Group):
         self.rows = self.T * self.K
         self.heap_bytes = self.cap * self.row + self.rows * self.row + self.T * self.row + 64 * MiB
 
+    FULL_ORDER_TOKENS = 512     # the reference-order row runs on the first tokens of every PE only: it takes 16x as long per row
+
     def names(self):
-        return ["moe_dispatch_put_signal", "moe_dispatch_put_quiet_signal", "moe_dispatch_plain_store", "moe_combine"]
+        return ["moe_dispatch_put_signal", "moe_dispatch_put_signal_full_order", "moe_dispatch_put_quiet_signal",
+                "moe_dispatch_plain_store", "moe_combine"]
 
     def setup(self, rt, gen):
         self.rt, self.perf = rt, rt.perftest()
@@ -279,15 +282,31 @@ class MoeShuffle(Group):
         self.sig = rt.calloc(npes * self.SIG_STRIDE, 8)
         rt.upload_all(self.d_pe, self.dest_pe); rt.upload_all(self.d_row, self.dest_row)
         rt.upload_all(self.d_expected, self.expected)
+        # the rows of the first FULL_ORDER_TOKENS tokens of every PE, counted per (destination, source)
+        Ts = self.FULL_ORDER_TOKENS
+        head = self.dest_pe[:, :Ts * K]
+        self.expected_head = np.stack([[int((head[s] == d).sum()) for s in range(npes)]
+                                       for d in range(npes)]).astype(np.uint64)
+        self.d_expected_head = rt.malloc(npes * 8)
+        rt.upload_all(self.d_expected_head, self.expected_head)
         self.payload = gen("u64", npes, T * row // 8, 7).view(np.uint8).reshape(npes, T, row)
         rt.upload_all(self.send, self.payload)
         perf = self.perf
 
         def put_signal():
+            # plain NVSHMEM_SIGNAL_ADD at the call sites; the payload-only order comes from the library option
+            # that NVSHMEM_AMD_PUT_SIGNAL_ORDER=payload sets, as for a program written for the reference
+            # (set by the item's prepare(), outside the timed steps)
             _check(perf.nvshmem_perftest_fill_words(self.sig, 0, npes * self.SIG_STRIDE, None), "fill_words", rt)
             _check(perf.nvshmem_perftest_moe_dispatch_put_signal(
                 self.recv, cap, self.send, self.d_pe, self.d_row, self.d_expected, self.sig, self.SIG_STRIDE, T, K,
-                row, 64, 256, SCOPE_WARP | 256 | 512, None), "moe_dispatch_put_signal", rt)
+                row, 64, 256, SCOPE_WARP | 256, None), "moe_dispatch_put_signal", rt)
+
+        def put_signal_full_order():
+            _check(perf.nvshmem_perftest_fill_words(self.sig, 0, npes * self.SIG_STRIDE, None), "fill_words", rt)
+            _check(perf.nvshmem_perftest_moe_dispatch_put_signal(
+                self.recv, cap, self.send, self.d_pe, self.d_row, self.d_expected_head, self.sig, self.SIG_STRIDE,
+                self.FULL_ORDER_TOKENS, K, row, 64, 256, SCOPE_WARP | 256, None), "moe_dispatch_put_signal", rt)
 
         def put_quiet_signal():
             _check(perf.nvshmem_perftest_fill_words(self.sig, 0, npes, None), "fill_words", rt)
@@ -314,9 +333,18 @@ class MoeShuffle(Group):
         items = [
             Item("moe_dispatch_put_signal", "u8", moved + moved // K,
                  "moe_dispatch_rowsignal_kernel<warp> (nvshmemx_putmem_signal_nbi_warp per row)",
-                 "moe_dispatch_put_signal: one nvshmemx_putmem_signal_nbi_warp per row copy (NVSHMEM_SIGNAL_ADD of 1, "
-                 "payload-only ordering, one signal word per source on its own 128-byte line), receivers "
+                 "moe_dispatch_put_signal: one nvshmemx_putmem_signal_nbi_warp per row copy (plain NVSHMEM_SIGNAL_ADD of 1 "
+                 "at the call sites, payload-only order chosen library-wide as NVSHMEM_AMD_PUT_SIGNAL_ORDER=payload "
+                 "does, one signal word per source on its own 128-byte line), receivers "
                  "nvshmem_signal_wait_until(GE); " + shape, put_signal, dict(common, note=lower), scale=5),
+            Item("moe_dispatch_put_signal_full_order", "u8", (moved + moved // K) * self.FULL_ORDER_TOKENS // T,
+                 "moe_dispatch_rowsignal_kernel<warp> (nvshmemx_putmem_signal_nbi_warp per row, reference order)",
+                 "moe_dispatch_put_signal_full_order: the same kernel with the library's default order of the signal, "
+                 "the reference's (a full release in front of every signal: an L2 write-back per row), on the first "
+                 "%d tokens of every PE; " % self.FULL_ORDER_TOKENS + shape, put_signal_full_order,
+                 dict(common, tokens=self.FULL_ORDER_TOKENS,
+                      note="a cost on record, not a rate to compare: what an unmodified caller pays per row until it "
+                           "opts into the payload-only order"), scale=5),
             Item("moe_dispatch_put_quiet_signal", "u8", moved + moved // K,
                  "moe_dispatch_kernel<warp> (nvshmemx_putmem_nbi_warp per row, nvshmemx_quiet_block, nvshmemx_signal_op)",
                  "moe_dispatch_put_quiet_signal: one nvshmemx_putmem_nbi_warp per row copy, rows per destination "
@@ -332,8 +360,10 @@ class MoeShuffle(Group):
             Item("moe_combine", "u8", 2 * moved, "moe_combine_kernel<warp, 2048>",
                  "moe_combine: nvshmemx_getmem_nbi_warp per 2 KiB of a row; " + shape, combine, common, scale=5),
         ]
-        for it, what in zip(items, ("put_signal", "plain_store", "plain_store", "combine")):
+        for it, what in zip(items, ("put_signal", "put_signal_head", "plain_store", "plain_store", "combine")):
             it.what = what
+            # the library-wide order of put-with-signal: payload-only for the first row, the default for the rest
+            it.prepare = (lambda on=(what == "put_signal"): rt.lib.nvshmemx_amd_set_put_signal_order(1 if on else 0))
         return items
 
 

@@ -272,6 +272,33 @@ def test_put_signal_never_overtakes_its_payload(rt, sig_op):
     assert perf.nvshmem_perftest_put_signal_stream(0, 0, 0, 0, 12, 1, 1, 1, N.SCOPE_BLOCK, sig_op, None) != 0
 
 
+def test_library_wide_put_signal_order(rt):
+    """Call sites that pass plain NVSHMEM_SIGNAL_ADD, as code written for the reference does, get the
+    payload-only order from the library option; the signal still never overtakes its payload, and the
+    option goes back to the reference's order afterwards."""
+    perf = rt.perftest()
+    assert rt.lib.nvshmemx_amd_get_put_signal_order() == 0
+    rt.lib.nvshmemx_amd_set_put_signal_order(1)
+    try:
+        assert rt.lib.nvshmemx_amd_get_put_signal_order() == 1
+        for scope, nbytes, slots, iters, blocks in ((N.SCOPE_BLOCK, 14336, 3, 200, 8), (N.SCOPE_WARP, 14336, 4, 400, 16),
+                                                    (N.SCOPE_THREAD, 256, 2, 50, 2)):
+            data = rt.malloc(blocks * slots * nbytes); stage = rt.malloc(blocks * nbytes)
+            sig = rt.calloc(2 * blocks, 8); errors = rt.calloc(1, 8)
+            rt.fill(data, 0xFF, blocks * slots * nbytes)
+            note("library-wide payload order: put_signal stream scope=%d bytes=%d" % (scope, nbytes))
+            assert perf.nvshmem_perftest_put_signal_stream(data, stage, sig, errors, nbytes, slots, iters, blocks,
+                                                           scope, SIGNAL_ADD, None) == 0
+            rt.sync()
+            assert all(rt.read_timeout(pe)[0] == 0 for pe in range(NPES))
+            assert (_words(rt, errors)[:, 0] == 0).all(), _words(rt, errors)[:, 0]
+            for p in (data, stage, sig, errors):
+                rt.free(p)
+    finally:
+        rt.lib.nvshmemx_amd_set_put_signal_order(0)
+    assert rt.lib.nvshmemx_amd_get_put_signal_order() == 0
+
+
 def test_collective_launch_refuses_grids_that_cannot_be_co_resident(rt):
     perf = rt.perftest()
     dst = rt.calloc(1 << 20, 4); src = rt.calloc(1 << 20, 4); sig = rt.calloc(65535, 8)
