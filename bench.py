@@ -121,7 +121,7 @@ class Checker:
         ok = True
         for lo, cnt in ((0, min(n, 1 << 22)), (max(0, n - (1 << 16)), min(n, 1 << 16))):
             want = O.reduce(item.oracle_dtype, item.op, data[:, lo:lo + cnt])
-            for pe in (0, 5, g.npes - 1):
+            for pe in sorted({0, min(5, g.npes - 1), g.npes - 1}):
                 got = g.rt.download(g.dst, pe, (cnt,), want.dtype, lo * es)
                 ok = ok and bool(np.array_equal(got.view(np.uint8), want.view(np.uint8)))
         return ok

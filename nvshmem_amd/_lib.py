@@ -132,6 +132,7 @@ def load_perftest():
     sig = {
         "nvshmem_perftest_ring_rma": [vp, vp, sz, i32, i32, i32, i32, i32, vp],
         "nvshmem_perftest_plain_copy": [vp, vp, sz, vp],
+        "nvshmem_perftest_stream_probe": [vp, sz, i32, i32, i32, vp],
         "nvshmem_perftest_profile_marker": [vp],
         "nvshmem_perftest_p_g": [vp, vp, u64, vp],
         "nvshmem_perftest_pe_identity": [vp, i32, vp],

@@ -256,6 +256,37 @@ __global__ void ring_reduce_kernel(int32_t *dst, const int32_t *src, size_t nred
     if (threadIdx.x == 0) *(uint64_t *)nvshmem_ptr(signal, me) = 0;  // ready for the next run
 }
 
+// One-sided stream probes for hardware counters: the deep rounds of a long block-scoped copy with one side
+// removed.  Every block reads (WRITE false) or writes (WRITE true) its contiguous slice of the calling
+// PE's buffer, 8 vectors per lane and round, wavefront w the w-th KiB of every 16 KiB.  What they show is
+// how many requests a compute unit keeps in flight when loads and stores do not share its queues.
+template <bool WRITE>
+__global__ __launch_bounds__(1024) void stream_probe_kernel(char *buf, size_t bytes, size_t per_block) {
+    char *mine = (char *)nvshmem_ptr(buf, nvshmem_my_pe()) + (size_t)blockIdx.x * per_block;
+    const unsigned wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6), lane_off = (threadIdx.x & 63u) * 16u;
+    const size_t step = (size_t)blockDim.x * 16, per_round = 8 * step;
+    nvshmemi_v4u acc = {0u, 0u, 0u, 0u};
+    for (size_t r = 0; r + per_round <= per_block; r += per_round) {
+        char *p = mine + r + (size_t)wave * 1024 + lane_off;
+        if (WRITE) {
+#pragma unroll
+            for (int u = 0; u < 8; ++u) {
+                const nvshmemi_v4u v = {(unsigned)r, threadIdx.x, (unsigned)u, blockIdx.x};
+                __builtin_nontemporal_store(v, reinterpret_cast<nvshmemi_v4u *>(p + u * step));
+            }
+        } else {
+            nvshmemi_v4u v[8];
+#pragma unroll
+            for (int u = 0; u < 8; ++u) v[u] = __builtin_nontemporal_load(reinterpret_cast<const nvshmemi_v4u *>(p + u * step));
+#pragma unroll
+            for (int u = 0; u < 8; ++u) acc ^= v[u];
+        }
+    }
+    // (keeps the loads alive; random data never matches)
+    if (!WRITE && acc.x == 0x9E3779B1u && acc.y == 0x85EBCA77u && acc.z == 0xC2B2AE3Du && acc.w == 1u)
+        *reinterpret_cast<nvshmemi_v4u *>(mine) = acc;
+}
+
 // Boundary between workloads in a profiler trace: does nothing, has a name of its own.
 __global__ void profile_marker_kernel() {}
 
@@ -395,6 +426,19 @@ int nvshmem_perftest_plain_copy(void *dst, const void *src, size_t bytes, void *
     hipLaunchKernelGGL(plain_copy_kernel, dim3((unsigned)((nvec + 255) / 256)), dim3(256), 0,
                        (hipStream_t)stream, (nvshmemi_v4u *)dst, (const nvshmemi_v4u *)src, nvec);
     return perftest::launch_status("plain_copy");
+}
+
+int nvshmem_perftest_stream_probe(void *buf, size_t bytes, int blocks_per_pe, int threads, int write, void *stream) {
+    if (!perftest::ready() || !perftest::check_launch(blocks_per_pe, threads) || (threads % 64) || !perftest::check_range(buf, bytes) ||
+        ((uintptr_t)buf % 16))
+        return NVSHMEMX_ERROR_INVALID_VALUE;
+    const size_t round = (size_t)threads * 16 * 8;
+    const size_t per_block = bytes / (size_t)blocks_per_pe / round * round;  // whole rounds only
+    if (per_block == 0) return NVSHMEMX_ERROR_INVALID_VALUE;
+    const dim3 grid((unsigned)blocks_per_pe, 1, (unsigned)nvshmem_n_pes());
+    if (write) hipLaunchKernelGGL(stream_probe_kernel<true>, grid, dim3(threads), 0, (hipStream_t)stream, (char *)buf, bytes, per_block);
+    else hipLaunchKernelGGL(stream_probe_kernel<false>, grid, dim3(threads), 0, (hipStream_t)stream, (char *)buf, bytes, per_block);
+    return perftest::launch_status("stream_probe");
 }
 
 int nvshmem_perftest_profile_marker(void *stream) {

@@ -26,17 +26,32 @@ MARKER = "profile_marker_kernel"
 CALIBRATION = "calibration"
 CALIBRATION_KIB = float(1 << 20)   # 1 GiB in KiB, read and written
 HBM_PEAK_GBS = 8000.0
+# rows of the table of L1 requests in flight, in this order
+INFLIGHT_WORKLOADS = ["put_block_256MiB_1blk", "put_block_256MiB_4blk", "put_block_256MiB_16blk", "get_block_256MiB_16blk",
+                      "put_block_256MiB_filled", "stream_read_16blk", "stream_write_16blk", "reducescatter", "sum_reduce",
+                      "alltoall_fp32_1GiB", "fcollect_int64", "broadcast", "moe_dispatch_put_signal", "moe_dispatch_plain_store",
+                      "moe_combine", "calibration"]
+INFLIGHT_TITLE = """L1-to-L2 requests a compute unit keeps in flight, by Little's law from the counters of ONE rocprofv3 pass
+(TCP_TCC_READ_REQ, TCP_TCC_READ_REQ_LATENCY, TCP_TCC_WRITE_REQ, TCP_TCC_WRITE_REQ_LATENCY, GRBM_GUI_ACTIVE / 8 as the cycles):
+in flight = requests x average latency / cycles / compute units occupied.  A read request is 128 bytes, a write
+request 64.  "rd lat" / "wr lat" are average cycles per request, "sum" = reads + writes in flight, "KiB" their bytes.
+Durations under the counter pass are a few percent longer than in the kernel trace; "kernel us" and GB/s
+(algorithmic bytes per second) are the kernel trace's."""
 
 
 COMMANDS = """Commands (on the GPU box, from the repository root; every file they run is committed):
   export OUT=<a scratch directory>; cd /tmp; export TMPDIR=/tmp
+  export NVSHMEM_AMD_PLAIN_COLLECTIVE_LAUNCH=1   (kernels that nvshmemx_collective_launch starts are started with a plain
+      launch: after a cooperative launch the profiled process crashes in an exit handler of the profiler's stack, behind
+      the written results; the kernels and their grids are the same)
   rocprofv3 --kernel-trace --stats -d $OUT/stats -- python3 $REPO/nvshmem_amd/profile_workloads.py --iters 4 --manifest $OUT/manifest.json
   rocprofv3 --pmc FETCH_SIZE -d $OUT/p1 -- python3 $REPO/nvshmem_amd/profile_workloads.py --iters 4 --manifest $OUT/manifest.json
-  rocprofv3 --pmc WRITE_SIZE -d $OUT/p2 -- python3 $REPO/nvshmem_amd/profile_workloads.py --iters 4 --manifest $OUT/manifest.json
-  rocprofv3 --pmc TCP_TCC_READ_REQ_sum TCP_TCC_READ_REQ_LATENCY_sum TCP_PENDING_STALL_CYCLES_sum TCP_TCR_TCP_STALL_CYCLES_sum -d $OUT/p3 -- (the same)
-  rocprofv3 --pmc SQ_WAVES SQ_BUSY_CYCLES SQ_WAIT_INST_ANY SQ_INSTS_VMEM_RD SQ_INSTS_VMEM_WR SQ_INST_LEVEL_VMEM GRBM_GUI_ACTIVE -d $OUT/p4 -- (the same)
+  rocprofv3 --pmc WRITE_SIZE -d $OUT/p2 -- (the same)
+  rocprofv3 --pmc TCP_TCC_READ_REQ_sum TCP_TCC_READ_REQ_LATENCY_sum TCP_TCC_WRITE_REQ_sum TCP_TCC_WRITE_REQ_LATENCY_sum GRBM_GUI_ACTIVE -d $OUT/p3 -- (the same)
+  rocprofv3 --pmc SQ_WAVES SQ_BUSY_CYCLES SQ_WAIT_INST_ANY SQ_INSTS_VMEM_RD SQ_INSTS_VMEM_WR SQ_INST_LEVEL_VMEM TCP_PENDING_STALL_CYCLES_sum TCP_TCR_TCP_STALL_CYCLES_sum -d $OUT/p4 -- (the same)
   rocprofv3 --pmc TCC_HIT_sum TCC_MISS_sum TCC_TAG_STALL_sum TCC_EA0_WRREQ_STALL_sum -d $OUT/p5 -- (the same)
-  cd $REPO; python3 nvshmem_amd/profile_summary.py --manifest $OUT/manifest.json --stats $OUT/stats --pmc $OUT/p1 ... --pmc $OUT/p5 --profiles-dir profiles
+  (every run must end with exit status 0)
+  cd $REPO; python3 nvshmem_amd/profile_summary.py --manifest $OUT/manifest.json --stats $OUT/stats --pmc $OUT/p1 ... --pmc $OUT/p5 --profiles-dir profiles --inflight-table profiles/l1_requests_in_flight.txt
 (a summary lists the counters of the passes that were run for it.)  Hardware: one MI355X (gfx950), ROCm 7.2.
 Durations are per dispatch from the kernel trace."""
 
@@ -106,6 +121,24 @@ def counters_of(rows):
     return {k: {c: sum(v) / len(v) for c, v in cs.items()} for k, cs in acc.items()}
 
 
+def in_flight(cs, shape):
+    """Little's law per compute unit: requests in flight = requests x latency / elapsed cycles, from the
+    L1-to-L2 request and latency counters of one pass and GRBM_GUI_ACTIVE (which sums the busy cycles of
+    the 8 XCDs).  shape = (grid threads x, y, z, block threads).  None when a counter is missing."""
+    need = ("TCP_TCC_READ_REQ_LATENCY_sum", "TCP_TCC_WRITE_REQ_LATENCY_sum", "GRBM_GUI_ACTIVE")
+    if any(k not in cs for k in need) or not cs["GRBM_GUI_ACTIVE"]:
+        return None
+    groups = shape[0] * shape[1] * shape[2] // max(1, shape[3])
+    cus = min(groups, 256)
+    cycles = cs["GRBM_GUI_ACTIVE"] / 8.0
+    rr, wr = cs.get("TCP_TCC_READ_REQ_sum", 0), cs.get("TCP_TCC_WRITE_REQ_sum", 0)
+    return {"groups": groups, "cus": cus, "cycles": cycles,
+            "reads": cs["TCP_TCC_READ_REQ_LATENCY_sum"] / cycles / cus,
+            "writes": cs["TCP_TCC_WRITE_REQ_LATENCY_sum"] / cycles / cus,
+            "read_latency": cs["TCP_TCC_READ_REQ_LATENCY_sum"] / rr if rr else 0.0,
+            "write_latency": cs["TCP_TCC_WRITE_REQ_LATENCY_sum"] / wr if wr else 0.0}
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--manifest", required=True)
@@ -115,6 +148,7 @@ def main():
     ap.add_argument("--only", default="")
     ap.add_argument("--table", default="", help="also write a one-line-per-workload table of the kernel trace there")
     ap.add_argument("--table-title", default="", help="first lines of that table")
+    ap.add_argument("--inflight-table", default="", help="write the table of L1 requests in flight per compute unit there")
     args = ap.parse_args()
     manifest = json.load(open(args.manifest))
     only = set(x for x in args.only.split(",") if x)
@@ -143,6 +177,7 @@ def main():
                                                                       entry.get("algorithmic_bytes", 0) / avg / 1e3))
         with open(args.table, "w") as fh:
             fh.write("\n".join(rows) + "\n")
+    flight_rows = []
     for entry in manifest:
         name = entry["name"]
         if only and name not in only:
@@ -175,6 +210,9 @@ def main():
         lines.append("achieved = algorithmic bytes / dominant kernel's average duration = %.0f GB/s = %.1f %% of the %.0f GB/s "
                      "HBM peak" % (alg / avg / 1e3, alg / avg / 1e3 / HBM_PEAK_GBS * 100, HBM_PEAK_GBS))
         cs = counters.get(dominant, {})
+        fl_row = in_flight(cs, st[dominant][4]) if cs else None
+        if fl_row and name in INFLIGHT_WORKLOADS:
+            flight_rows.append((name, dominant, st[dominant][1], alg / st[dominant][1] / 1e3, fl_row))
         if cs:
             lines += ["", "counters of the dominant kernel (average per dispatch):"]
             for c in sorted(cs):
@@ -185,16 +223,12 @@ def main():
             if "TCP_TCC_WRITE_REQ_LATENCY_sum" in cs and cs.get("TCP_TCC_WRITE_REQ_sum"):
                 lines.append("  -> average L1-to-L2 write latency: %.0f cycles per request"
                              % (cs["TCP_TCC_WRITE_REQ_LATENCY_sum"] / cs["TCP_TCC_WRITE_REQ_sum"]))
-            if ("TCP_TCC_READ_REQ_LATENCY_sum" in cs and cs.get("TCP_TCC_READ_REQ_sum") and cs.get("GRBM_GUI_ACTIVE")):
-                # Little's law per compute unit: requests in flight = requests x latency / elapsed cycles;
-                # GRBM_GUI_ACTIVE sums the busy cycles of the 8 XCDs
-                shape = st[dominant][4]
-                groups = shape[0] * shape[1] * shape[2] // max(1, shape[3])
-                cus = min(groups, 256)
-                cycles = cs["GRBM_GUI_ACTIVE"] / 8.0
-                lines.append("  -> %d work-groups on at most %d compute units, %.0f cycles: %.1f L1 read requests (128 bytes) "
-                             "in flight per compute unit on average"
-                             % (groups, cus, cycles, cs["TCP_TCC_READ_REQ_LATENCY_sum"] / cycles / cus))
+            fl = in_flight(cs, st[dominant][4])
+            if fl:
+                lines.append("  -> %d work-groups on at most %d compute units, %.0f cycles: per compute unit on average %.1f L1 read "
+                             "requests (128 bytes) and %.1f write requests (64 bytes) in flight, %.1f in all, %.1f KiB"
+                             % (fl["groups"], fl["cus"], fl["cycles"], fl["reads"], fl["writes"], fl["reads"] + fl["writes"],
+                                (128 * fl["reads"] + 64 * fl["writes"]) / 1024))
             if "TCC_EA0_RDREQ_LEVEL_sum" in cs and cs.get("TCC_EA0_RDREQ_sum"):
                 lines.append("  -> average L2-to-fabric read latency: %.0f cycles per request"
                              % (cs["TCC_EA0_RDREQ_LEVEL_sum"] / cs["TCC_EA0_RDREQ_sum"]))
@@ -216,6 +250,18 @@ def main():
                 os.remove(old)
             with open(os.path.join(args.profiles_dir, "%s__%s.txt" % (tag, name)), "w") as fh:
                 fh.write(text)
+
+
+    if args.inflight_table and flight_rows:
+        out = [INFLIGHT_TITLE, "", commands, "",
+               "%-26s %5s %9s %8s | %8s %9s | %8s %9s | %7s %7s" % ("workload", "CUs", "kernel us", "GB/s", "rd lat", "rd in fl", "wr lat",
+                                                                 "wr in fl", "sum", "KiB")]
+        for name, kernel, us, gbs, fl in sorted(flight_rows, key=lambda r: INFLIGHT_WORKLOADS.index(r[0])):
+            out.append("%-26s %5d %9.1f %8.0f | %8.0f %9.1f | %8.0f %9.1f | %7.1f %7.1f"
+                       % (name, fl["cus"], us, gbs, fl["read_latency"], fl["reads"], fl["write_latency"], fl["writes"],
+                          fl["reads"] + fl["writes"], (128 * fl["reads"] + 64 * fl["writes"]) / 1024))
+        with open(args.inflight_table, "w") as fh:
+            fh.write("\n".join(out) + "\n")
 
 
 if __name__ == "__main__":

@@ -110,7 +110,7 @@ def main():
     rt.finalize()
 
     plan = noise_plan(np, rng, 8, 8192, 8, 256, 1.1)
-    for g in workloads.all_groups(plan):
+    for g in workloads.all_groups(plan) + workloads.profile_only_groups():
         if only and not any(n in only for n in g.names()):
             continue
         rt = N.Runtime(npes=g.npes, symmetric_size=g.heap_bytes)

@@ -97,6 +97,35 @@ class RingRma(Group):
                      "is_get": is_get})
 
 
+class StreamProbe(Group):
+    """Counter probes, not API workloads (profile_workloads.py runs them, bench.py does not): the access
+    pattern of the 16-block put with one side removed."""
+    kind = "probe"
+    npes = 8
+    SIZE = 256 * MiB
+
+    def __init__(self):
+        self.heap_bytes = self.SIZE + 64 * MiB
+
+    def names(self):
+        return ["stream_read_16blk", "stream_write_16blk"]
+
+    def setup(self, rt, gen):
+        perf = rt.perftest()
+        buf = rt.malloc(self.SIZE)
+        rt.upload_all(buf, gen("bytes", self.npes, self.SIZE, 2))
+        items = []
+        for write, name in ((0, "stream_read_16blk"), (1, "stream_write_16blk")):
+            def step(write=write, name=name):
+                _check(perf.nvshmem_perftest_stream_probe(buf, self.SIZE, 16, 1024, write, None), name, rt)
+            items.append(Item(name, "u8", self.npes * self.SIZE, "stream_probe_kernel<%s>" % ("write" if write else "read"),
+                              "%s: counter probe, not an API call - 16 blocks x 1024 threads per PE %s their slice of 256 MiB "
+                              "per PE in the access pattern of the long block-scoped copy, the other side removed"
+                              % (name, "write" if write else "read"), step,
+                              {"npes": self.npes, "bytes_per_pe": self.SIZE, "blocks_per_pe": 16, "threads_per_block": 1024}))
+        return items
+
+
 # ------------------------------------------------------------------------------------------------
 # allreduce on a stream
 # ------------------------------------------------------------------------------------------------
@@ -367,11 +396,24 @@ class MoeShuffle(Group):
         return items
 
 
+def team_size_variant(npes):
+    return (("sum_reduce_fp32_%dpe" % npes, "float", "sum", "f32", 4, 3),)
+
+
+def profile_only_groups():
+    """Groups that only the profiler runs (counter probes)."""
+    return [StreamProbe()]
+
+
 def all_groups(moe_plan):
     """The groups in the order bench.py reports them.  moe_plan: see MoeShuffle."""
     return [RingRma(),
             Reduce(8, 1 << 20, CONFIG1, "config 1"),
             Reduce(8, 1 << 26, CONFIG3, "config 3: 256 MiB of fp32 per PE"),
+            # the same allreduce at other team sizes, 1 to 2 GiB of sources in all
+            Reduce(4, 1 << 26, team_size_variant(4), "4 members x 256 MiB"),
+            Reduce(16, 1 << 25, team_size_variant(16), "16 members x 128 MiB"),
+            Reduce(64, 1 << 23, team_size_variant(64), "64 members x 32 MiB"),
             Collect("float", 4, 1 << 22),
             Collect("int64", 8, 1 << 22),
             Collect("float", 4, 1 << 24, with_fcollect=False, suffix="_1GiB"),
