@@ -602,13 +602,14 @@ NVSHMEMI_DEVICE_INLINE void nvshmemi_amd_record_timeout(const void *addr, uint64
                                                         uint64_t expected) {
     uint64_t *rec = reinterpret_cast<uint64_t *>(
         nvshmemi_amd_remote(nvshmemi_device_state_d.timeout_record, nvshmemi_amd_my_pe()));
+    /* the count the host checks at its synchronisation points; the record's first word is this timeout's
+     * number in that count (never 0), so that a report can tell a record of its own period from an older one */
+    const uint64_t seq = __hip_atomic_fetch_add(nvshmemi_device_state_d.runtime_words + NVSHMEMI_AMD_TIMEOUT_COUNT_WORD,
+                                                (uint64_t)1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) + 1;
     rec[1] = (uint64_t)(uintptr_t)addr;
     rec[2] = found;
     rec[3] = expected;
-    __hip_atomic_store(rec, (uint64_t)1, __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_AGENT);
-    /* the count the host checks at its synchronisation points */
-    __hip_atomic_fetch_add(nvshmemi_device_state_d.runtime_words + NVSHMEMI_AMD_TIMEOUT_COUNT_WORD, (uint64_t)1,
-                           __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    __hip_atomic_store(rec, seq, __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_AGENT);
 }
 
 /* Spin until `*ivar cmp value`; `ivar` is a local operand.  Returns the value that ended the wait.
@@ -1447,20 +1448,33 @@ NVSHMEMI_DEVICE_INLINE void nvshmemi_amd_unit_reduce(nvshmem_team_t team, const 
         uint64_t polls = 0;
         for (;;) {
             bool missing = false;
+            /* The eight loads and their wait are ONE statement: between separate statements the compiler could
+             * copy or spill a destination register while its load is still in flight.  A slot that has nothing
+             * to fetch (an inactive lane, a member past the team, the PE itself) reads the start of the PE's own
+             * buffer, which is always mapped, and its value is not used. */
+            const char *from[8];
 #pragma unroll
             for (int q = 0; q < 8; ++q) {
                 const int p = p0 + q;
-                if (active && p < npes && p != me) {
-                    const char *from = mine + ((size_t)p * units + u) * NVSHMEMI_AMD_UNIT_BYTES + 16 * k;
-                    asm volatile("global_load_dwordx4 %0, %1, off sc1" : "=v"(x[q].v) : "v"(from) : "memory");
-                }
+                from[q] = (active && p < npes && p != me)
+                              ? mine + ((size_t)p * units + u) * NVSHMEMI_AMD_UNIT_BYTES + 16 * k
+                              : mine;
             }
-            /* the registers are operands so that no use of them moves in front of the wait */
-            asm volatile("s_waitcnt vmcnt(0)"
-                         : "+v"(x[0].v), "+v"(x[1].v), "+v"(x[2].v), "+v"(x[3].v), "+v"(x[4].v), "+v"(x[5].v),
-                           "+v"(x[6].v), "+v"(x[7].v)
-                         :
-                         : "memory");
+            asm volatile(
+                "global_load_dwordx4 %0, %8, off sc1\n\t"
+                "global_load_dwordx4 %1, %9, off sc1\n\t"
+                "global_load_dwordx4 %2, %10, off sc1\n\t"
+                "global_load_dwordx4 %3, %11, off sc1\n\t"
+                "global_load_dwordx4 %4, %12, off sc1\n\t"
+                "global_load_dwordx4 %5, %13, off sc1\n\t"
+                "global_load_dwordx4 %6, %14, off sc1\n\t"
+                "global_load_dwordx4 %7, %15, off sc1\n\t"
+                "s_waitcnt vmcnt(0)"
+                : "=&v"(x[0].v), "=&v"(x[1].v), "=&v"(x[2].v), "=&v"(x[3].v), "=&v"(x[4].v), "=&v"(x[5].v),
+                  "=&v"(x[6].v), "=&v"(x[7].v)
+                : "v"(from[0]), "v"(from[1]), "v"(from[2]), "v"(from[3]), "v"(from[4]), "v"(from[5]), "v"(from[6]),
+                  "v"(from[7])
+                : "memory");
 #pragma unroll
             for (int q = 0; q < 8; ++q) {
                 const int p = p0 + q;

@@ -380,7 +380,8 @@ NVSHMEMI_HOST_ONLY int nvshmemx_amd_module_init(void);
 
 /* Bounded device waits (counterpart of the reference's NVSHMEM_TIMEOUT_DEVICE_POLLING build,
  * src/include/non_abi/device/wait/nvshmemi_wait_until_apis.cuh:19-35): a wait that polls more than
- * `polls` times records {1, address, found, expected} and returns.  0 = wait forever. */
+ * `polls` times records {n, address, found, expected}, n >= 1 being its number among all timeouts of the GPU
+ * since nvshmem_init, and returns.  0 = wait forever. */
 NVSHMEMI_HOST_ONLY void nvshmemx_amd_set_spin_limit(uint64_t polls);
 /* Order of the signal of every device-side put-with-signal whose sig_op does not choose for itself:
  * 0 = the reference's (src/include/non_abi/device/common/nvshmemi_common_device.cuh:529-561: a full fence
@@ -389,7 +390,7 @@ NVSHMEMI_HOST_ONLY void nvshmemx_amd_set_spin_limit(uint64_t polls);
  * NVSHMEM_AMD_PUT_SIGNAL_ORDER=payload at nvshmem_init.  Waits for the device. */
 NVSHMEMI_HOST_ONLY void nvshmemx_amd_set_put_signal_order(int payload_only);
 NVSHMEMI_HOST_ONLY int nvshmemx_amd_get_put_signal_order(void); /* 1 = payload only, 0 = the reference's */
-/* Copies PE `pe`'s timeout record (4 words) to `out` and clears it; returns the flag word. */
+/* Copies PE `pe`'s timeout record (4 words) to `out` and clears it; returns its first word (0: none). */
 NVSHMEMI_HOST_ONLY uint64_t nvshmemx_amd_read_timeout(int pe, uint64_t out[4]);
 /* A wait that gives up does not stay silent.  The device counts every one; the host calls that wait
  * for the device - nvshmem_quiet, nvshmem_fence, nvshmem_barrier_all / nvshmem_sync_all, nvshmem_barrier /

@@ -238,7 +238,7 @@ typedef struct nvshmemi_device_state {
     uint64_t *sync_flags; /* canonical address: NVSHMEMI_AMD_MAX_PES arrival words per PE */
     uint64_t *sync_epoch; /* canonical address: that PE's barrier epoch */
     uint64_t spin_limit;  /* 0 = wait forever; else a bounded wait gives up after this many polls */
-    uint64_t *timeout_record; /* canonical address: 4 words {flag, addr, found, expected} */
+    uint64_t *timeout_record; /* canonical address: 4 words {number of the timeout (0: none), addr, found, expected} */
     const nvshmemi_amd_team_view_t *team_views; /* [NVSHMEMI_AMD_MAX_TEAMS][NVSHMEMI_AMD_MAX_PES] */
     uint64_t *team_sync; /* [MAX_TEAMS][MAX_PES][NVSHMEMI_AMD_TEAM_SYNC_WORDS]: barrier rows of the teams
                             other than WORLD, low-latency counters of all teams */

@@ -287,7 +287,12 @@ int nvshmem_perftest_moe_dispatch_pieces(void *recv, size_t recv_cap_rows, const
  * words from the caller: they live in a static device array of the library (8 KiB per GPU, rows for at
  * most 32 PEs; more PEs are refused with NVSHMEMX_ERROR_INVALID_VALUE and a message), which a kernel on
  * `stream` clears before the rows are sent.  It calls no hipMalloc, hipFree or other allocating routine.
- * All calls on one GPU share that array: calls that overlap in time on one GPU race. */
+ * All calls on one GPU share that array: calls that overlap in time on one GPU race (two host threads
+ * inside the call at once are refused; kernels of calls on different streams that overlap on the GPU are
+ * the caller's to avoid).  The array's address is looked up once per GPU, in nvshmem_perftest_static_init()
+ * or in the first call on that GPU; under stream capture no lookup is made, so a caller that captures its
+ * first call runs nvshmem_perftest_static_init() beforehand, with that GPU current. */
+int nvshmem_perftest_static_init(void);
 int nvshmem_perftest_moe_dispatch_pieces_static(void *recv, size_t recv_cap_rows, const void *send,
                                                 const int32_t *dest_pe, const int64_t *dest_row,
                                                 const uint64_t *expected, int tokens, int topk,

@@ -166,6 +166,7 @@ def load_perftest():
         "nvshmem_perftest_put_signal_stream": [vp, vp, vp, vp, sz, i32, i32, i32, i32, i32, vp],
         "nvshmem_perftest_moe_dispatch_put_signal": [vp, sz, vp, vp, vp, vp, vp, i32, i32, i32, sz, i32, i32, i32, vp],
         "nvshmem_perftest_moe_dispatch_pieces": [vp, sz, vp, vp, vp, vp, vp, i32, i32, sz, i32, i32, vp],
+        "nvshmem_perftest_static_init": [],
         "nvshmem_perftest_moe_dispatch_pieces_static": [vp, sz, vp, vp, vp, vp, i32, i32, sz, i32, i32, vp],
         "nvshmem_perftest_moe_combine": [vp, vp, sz, vp, vp, i32, i32, sz, i32, i32, vp],
         "nvshmem_perftest_moe_combine_ex": [vp, vp, sz, vp, vp, i32, i32, sz, i32, i32, i32, vp],

@@ -8,7 +8,9 @@
 // A row of 14336 bytes is 896 16-byte vectors: a wavefront moves it with 14 vectors per lane, so
 // the default scope is one row per wavefront with no block-wide synchronisation in the loop.
 #include <hip/hip_runtime.h>
+#include <atomic>
 #include <cstdlib>
+#include <mutex>
 
 // A row is 14 vectors per lane: rounds of 8 + 4 + 2 keep more loads in flight than the default
 // 4 + 4 + 4 + 2 (measured 5 % faster for dispatch and combine).  (The kernel that signals every row is
@@ -294,17 +296,33 @@ __global__ void clear_words_kernel(uint64_t *words, unsigned n) {
     if (i < n) words[i] = 0;
 }
 
-// Address of this device's copy of `scratch`, looked up once per device.
+// Address of this device's copy of `scratch`.  The lookup (hipGetSymbolAddress: a runtime call that may load
+// the code object) happens once per device, under a lock, in nvshmem_perftest_static_init or in the first
+// call of the entry point on that device - never under stream capture: `may_lookup` is false there, and an
+// address that is not known yet is then an error.
 constexpr int kMaxDevices = 64;
-uint64_t *scratch_address() {
-    static uint64_t *ptr[kMaxDevices];
+std::mutex scratch_lock;
+uint64_t *scratch_ptr[kMaxDevices];
+std::atomic<int> scratch_calls_in_progress[kMaxDevices];   // host threads inside the entry point, per device
+
+int current_device() {
     int dev = -1;
     if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= kMaxDevices) {
         (void)hipGetLastError();
         fprintf(stderr, "nvshmem_perftest: no current device for the static signal words\n");
-        return nullptr;
+        return -1;
     }
-    if (!ptr[dev]) {
+    return dev;
+}
+
+uint64_t *scratch_address(int dev, bool may_lookup) {
+    std::lock_guard<std::mutex> lock(scratch_lock);
+    if (!scratch_ptr[dev]) {
+        if (!may_lookup) {
+            fprintf(stderr, "nvshmem_perftest: the static signal words of device %d are not looked up yet and the "
+                            "stream is being captured; call nvshmem_perftest_static_init() first\n", dev);
+            return nullptr;
+        }
         void *p = nullptr;
         const hipError_t e = hipGetSymbolAddress(&p, HIP_SYMBOL(scratch));
         if (e != hipSuccess || !p) {
@@ -312,9 +330,9 @@ uint64_t *scratch_address() {
             fprintf(stderr, "nvshmem_perftest: hipGetSymbolAddress(scratch) failed: %s\n", hipGetErrorString(e));
             return nullptr;
         }
-        ptr[dev] = (uint64_t *)p;
+        scratch_ptr[dev] = (uint64_t *)p;
     }
-    return ptr[dev];
+    return scratch_ptr[dev];
 }
 
 bool moe_args_ok(const void *table_pe, const void *table_row, int tokens, int topk,
@@ -473,10 +491,34 @@ int nvshmem_perftest_moe_dispatch_pieces_static(void *recv, size_t recv_cap_rows
                 nvshmem_n_pes(), kStaticSignalPes);
         return NVSHMEMX_ERROR_INVALID_VALUE;
     }
-    uint64_t *words = scratch_address();
+    const int dev = current_device();
+    if (dev < 0) return NVSHMEMX_ERROR_INTERNAL;
+    hipStreamCaptureStatus capture = hipStreamCaptureStatusNone;
+    if (hipStreamIsCapturing((hipStream_t)stream, &capture) != hipSuccess) {
+        (void)hipGetLastError();
+        capture = hipStreamCaptureStatusNone;
+    }
+    uint64_t *words = scratch_address(dev, capture == hipStreamCaptureStatusNone);
     if (!words) return NVSHMEMX_ERROR_INTERNAL;
-    return dispatch_pieces(recv, recv_cap_rows, send, dest_pe, dest_row, expected, nullptr, words, tokens, topk,
-                           row_bytes, piece_bytes, threads, stream);
+    // every call on a device uses the same words: two host threads inside the call at once are refused (calls
+    // whose kernels overlap on the GPU from different streams cannot be seen from here and are the caller's
+    // to avoid)
+    if (scratch_calls_in_progress[dev].fetch_add(1) != 0) {
+        scratch_calls_in_progress[dev].fetch_sub(1);
+        fprintf(stderr, "nvshmem_perftest_moe_dispatch_pieces_static: another thread is inside this call on device %d; "
+                        "the static signal words serve one call at a time\n", dev);
+        return NVSHMEMX_ERROR_INVALID_VALUE;
+    }
+    const int rc = dispatch_pieces(recv, recv_cap_rows, send, dest_pe, dest_row, expected, nullptr, words, tokens, topk,
+                                   row_bytes, piece_bytes, threads, stream);
+    scratch_calls_in_progress[dev].fetch_sub(1);
+    return rc;
+}
+
+int nvshmem_perftest_static_init(void) {
+    const int dev = current_device();
+    if (dev < 0) return NVSHMEMX_ERROR_INTERNAL;
+    return scratch_address(dev, true) ? 0 : NVSHMEMX_ERROR_INTERNAL;
 }
 
 // piece_bytes: 0 = a work item is a whole row; 1024 / 2048 / 4096 (wavefront scope only) = a work

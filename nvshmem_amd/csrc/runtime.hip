@@ -72,18 +72,29 @@ uint64_t report_timeouts(Runtime &rt, const char *where) {
     if (count <= rt.timeouts_seen) return 0;
     const uint64_t fresh = count - rt.timeouts_seen;
     rt.timeouts_seen = count;
-    // the most recent record of the first PE that has one says where
+    // Where: the newest record among the PEs' whose number lies in this period (a record's first word is the
+    // timeout's number in the count; a PE keeps its latest one until nvshmemx_amd_read_timeout clears it).
+    const uint64_t period_start = count - fresh;
     uint64_t rec[4] = {0, 0, 0, 0};
     int pe_hit = -1;
     uint64_t off = 0;
     rt.offset_of(rt.dev.timeout_record, &off);
-    for (int pe = 0; pe < rt.npes && pe_hit < 0; ++pe)
-        if (hipMemcpy(rec, rt.slice(pe) + off, sizeof rec, hipMemcpyDeviceToHost) == hipSuccess && rec[0]) pe_hit = pe;
+    for (int pe = 0; pe < rt.npes; ++pe) {
+        uint64_t r[4] = {0, 0, 0, 0};
+        if (hipMemcpy(r, rt.slice(pe) + off, sizeof r, hipMemcpyDeviceToHost) != hipSuccess) continue;
+        if (r[0] > period_start && r[0] > rec[0]) {
+            pe_hit = pe;
+            for (int i = 0; i < 4; ++i) rec[i] = r[i];
+        }
+    }
+    (void)hipGetLastError();
+    char where_text[160] = "";
+    if (pe_hit >= 0)
+        snprintf(where_text, sizeof where_text, "; e.g. PE %d waited at %p for %llu and last saw %llu", pe_hit,
+                 (void *)(uintptr_t)rec[1], (unsigned long long)rec[3], (unsigned long long)rec[2]);
     set_error("%s: %llu device-side wait%s gave up after the spin limit of %llu polls (NVSHMEM_AMD_SPIN_LIMIT; 0 waits "
-              "forever) and the kernel went on as if satisfied - results may be incomplete; e.g. PE %d waited at %p "
-              "for %llu and last saw %llu",
-              where, (unsigned long long)fresh, fresh == 1 ? "" : "s", (unsigned long long)rt.dev.spin_limit, pe_hit,
-              (void *)(uintptr_t)rec[1], (unsigned long long)rec[3], (unsigned long long)rec[2]);
+              "forever) and the kernel went on as if satisfied - results may be incomplete%s",
+              where, (unsigned long long)fresh, fresh == 1 ? "" : "s", (unsigned long long)rt.dev.spin_limit, where_text);
     return fresh;
 }
 

@@ -102,7 +102,7 @@ def test_host_typed_sized_strided_rma_and_waits():
         s.synchronize()
         rt.lib.nvshmemx_amd_set_spin_limit(1 << 22)
         flag, rec = rt.read_timeout(0)
-        assert flag == 1 and rec[2] == 0xFFFFFFFB and rec[3] == 5      # found (uint)-5, expected 5
+        assert flag >= 1 and rec[2] == 0xFFFFFFFB and rec[3] == 5      # found (uint)-5, expected 5
         s.destroy()
 
 
@@ -134,7 +134,7 @@ def test_wait_until_all_vector_on_stream():
         s.synchronize()
         rt.lib.nvshmemx_amd_set_spin_limit(1 << 22)
         flag, rec = rt.read_timeout(0)
-        assert flag == 1 and rec[2] == 10 and rec[3] == 11
+        assert flag >= 1 and rec[2] == 10 and rec[3] == 11
         # ... and with 13 in the set the wait gives up there, having passed the twelve in front of it
         st[13] = 0
         rt.upload(mstat, 0, st)
@@ -143,7 +143,7 @@ def test_wait_until_all_vector_on_stream():
         s.synchronize()
         rt.lib.nvshmemx_amd_set_spin_limit(1 << 22)
         flag, rec = rt.read_timeout(0)
-        assert flag == 1 and rec[2] == 39 and rec[3] == 40, rec
+        assert flag >= 1 and rec[2] == 39 and rec[3] == 40, rec
         assert rec[1] == rt.ptr(many, 0) + 13 * 8
         wait(flags, 4, None, 17, values, s.ptr)
         assert b"unknown comparison" in lib.nvshmemx_amd_last_error()

@@ -112,7 +112,7 @@ def test_bounded_wait_gives_up_and_records_the_timeout(rt):
         assert rt.lib.nvshmemx_amd_timeout_count() == before + 2 * NPES
         for pe in range(NPES):
             flag, rec = rt.read_timeout(pe)
-            assert flag == 1
+            assert flag >= 1          # the number of this timeout in the GPU-wide count
             assert rec[1] == rt.ptr(sig, pe) and rec[2] == 0 and rec[3] == 5
             assert rt.read_timeout(pe)[0] == 0         # reading clears the record
     finally:

@@ -27,6 +27,7 @@ def test_static_dispatch_matches_the_dispatch_with_caller_signal_words():
     Tmax = max(c[0] for c in calls)
     with runtime(npes, 2 * cap * row + Tmax * row + (32 << 20)) as rt:
         perf = rt.perftest()
+        assert perf.nvshmem_perftest_static_init() == 0      # the address of the static words, looked up up front
         send = rt.malloc(Tmax * row); recv_a = rt.malloc(cap * row); recv_b = rt.malloc(cap * row)
         d_pe = rt.malloc(Tmax * K * 4); d_row = rt.malloc(Tmax * K * 8)
         expected = rt.malloc(npes * 8); sig = rt.calloc(npes, 8)
