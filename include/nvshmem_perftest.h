@@ -42,7 +42,7 @@ int nvshmem_perftest_ring_rma(void *dest, const void *src, size_t bytes, int blo
  * `bytes` each. */
 int nvshmem_perftest_plain_copy(void *dst, const void *src, size_t bytes, void *stream);
 /* Stream probes for hardware counters (no counterpart in the reference): every block of every PE reads
- * (write == 0) or writes its contiguous slice of the PE's `bytes` at buf, in the access pattern of a long
+ * (write == 0) or writes (1: streaming stores, 2: write-through stores) its contiguous slice of the PE's `bytes` at buf, in the access pattern of a long
  * block-scoped copy with the other side removed; the slice is cut to whole rounds of threads x 128 bytes. */
 int nvshmem_perftest_stream_probe(void *buf, size_t bytes, int blocks_per_pe, int threads, int write, void *stream);
 

@@ -260,7 +260,7 @@ __global__ void ring_reduce_kernel(int32_t *dst, const int32_t *src, size_t nred
 // removed.  Every block reads (WRITE false) or writes (WRITE true) its contiguous slice of the calling
 // PE's buffer, 8 vectors per lane and round, wavefront w the w-th KiB of every 16 KiB.  What they show is
 // how many requests a compute unit keeps in flight when loads and stores do not share its queues.
-template <bool WRITE>
+template <int WRITE>   // 0 read, 1 write with streaming (nt) stores, 2 write with write-through (sc1 nt) stores
 __global__ __launch_bounds__(1024) void stream_probe_kernel(char *buf, size_t bytes, size_t per_block) {
     char *mine = (char *)nvshmem_ptr(buf, nvshmem_my_pe()) + (size_t)blockIdx.x * per_block;
     const unsigned wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6), lane_off = (threadIdx.x & 63u) * 16u;
@@ -272,7 +272,8 @@ __global__ __launch_bounds__(1024) void stream_probe_kernel(char *buf, size_t by
 #pragma unroll
             for (int u = 0; u < 8; ++u) {
                 const nvshmemi_v4u v = {(unsigned)r, threadIdx.x, (unsigned)u, blockIdx.x};
-                __builtin_nontemporal_store(v, reinterpret_cast<nvshmemi_v4u *>(p + u * step));
+                if (WRITE == 2) nvshmemi_amd_stream_store16<NVSHMEMI_AMD_STORE_WRITE_THROUGH>(p + u * step, v);
+                else __builtin_nontemporal_store(v, reinterpret_cast<nvshmemi_v4u *>(p + u * step));
             }
         } else {
             nvshmemi_v4u v[8];
@@ -436,8 +437,9 @@ int nvshmem_perftest_stream_probe(void *buf, size_t bytes, int blocks_per_pe, in
     const size_t per_block = bytes / (size_t)blocks_per_pe / round * round;  // whole rounds only
     if (per_block == 0) return NVSHMEMX_ERROR_INVALID_VALUE;
     const dim3 grid((unsigned)blocks_per_pe, 1, (unsigned)nvshmem_n_pes());
-    if (write) hipLaunchKernelGGL(stream_probe_kernel<true>, grid, dim3(threads), 0, (hipStream_t)stream, (char *)buf, bytes, per_block);
-    else hipLaunchKernelGGL(stream_probe_kernel<false>, grid, dim3(threads), 0, (hipStream_t)stream, (char *)buf, bytes, per_block);
+    if (write == 2) hipLaunchKernelGGL(stream_probe_kernel<2>, grid, dim3(threads), 0, (hipStream_t)stream, (char *)buf, bytes, per_block);
+    else if (write) hipLaunchKernelGGL(stream_probe_kernel<1>, grid, dim3(threads), 0, (hipStream_t)stream, (char *)buf, bytes, per_block);
+    else hipLaunchKernelGGL(stream_probe_kernel<0>, grid, dim3(threads), 0, (hipStream_t)stream, (char *)buf, bytes, per_block);
     return perftest::launch_status("stream_probe");
 }
 

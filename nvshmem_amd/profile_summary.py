@@ -28,7 +28,8 @@ CALIBRATION_KIB = float(1 << 20)   # 1 GiB in KiB, read and written
 HBM_PEAK_GBS = 8000.0
 # rows of the table of L1 requests in flight, in this order
 INFLIGHT_WORKLOADS = ["put_block_256MiB_1blk", "put_block_256MiB_4blk", "put_block_256MiB_16blk", "get_block_256MiB_16blk",
-                      "put_block_256MiB_filled", "stream_read_16blk", "stream_write_16blk", "reducescatter", "sum_reduce",
+                      "put_block_256MiB_filled", "stream_read_16blk", "stream_write_16blk", "stream_write_8blk", "stream_read_filled",
+                      "stream_write_filled", "stream_write_through_filled", "reducescatter", "sum_reduce",
                       "alltoall_fp32_1GiB", "fcollect_int64", "broadcast", "moe_dispatch_put_signal", "moe_dispatch_plain_store",
                       "moe_combine", "calibration"]
 INFLIGHT_TITLE = """L1-to-L2 requests a compute unit keeps in flight, by Little's law from the counters of ONE rocprofv3 pass

@@ -107,22 +107,29 @@ class StreamProbe(Group):
     def __init__(self):
         self.heap_bytes = self.SIZE + 64 * MiB
 
+    # (name, blocks per PE, threads, mode: 0 read, 1 write with streaming stores, 2 write with write-through stores)
+    SHAPES = (("stream_read_16blk", 16, 1024, 0), ("stream_write_16blk", 16, 1024, 1), ("stream_write_8blk", 8, 1024, 1),
+              ("stream_read_filled", 1024, 256, 0), ("stream_write_filled", 32768, 64, 1),
+              ("stream_write_through_filled", 32768, 64, 2))
+
     def names(self):
-        return ["stream_read_16blk", "stream_write_16blk"]
+        return [s[0] for s in self.SHAPES]
 
     def setup(self, rt, gen):
         perf = rt.perftest()
         buf = rt.malloc(self.SIZE)
         rt.upload_all(buf, gen("bytes", self.npes, self.SIZE, 2))
         items = []
-        for write, name in ((0, "stream_read_16blk"), (1, "stream_write_16blk")):
-            def step(write=write, name=name):
-                _check(perf.nvshmem_perftest_stream_probe(buf, self.SIZE, 16, 1024, write, None), name, rt)
-            items.append(Item(name, "u8", self.npes * self.SIZE, "stream_probe_kernel<%s>" % ("write" if write else "read"),
-                              "%s: counter probe, not an API call - 16 blocks x 1024 threads per PE %s their slice of 256 MiB "
+        for name, blocks, threads, mode in self.SHAPES:
+            def step(name=name, blocks=blocks, threads=threads, mode=mode):
+                _check(perf.nvshmem_perftest_stream_probe(buf, self.SIZE, blocks, threads, mode, None), name, rt)
+            what = ("read", "write with streaming (nt) stores", "write with write-through (sc1 nt) stores")[mode]
+            items.append(Item(name, "u8", self.npes * self.SIZE, "stream_probe_kernel<%d>" % mode,
+                              "%s: counter probe, not an API call - %d blocks x %d threads per PE %s their slice of 256 MiB "
                               "per PE in the access pattern of the long block-scoped copy, the other side removed"
-                              % (name, "write" if write else "read"), step,
-                              {"npes": self.npes, "bytes_per_pe": self.SIZE, "blocks_per_pe": 16, "threads_per_block": 1024}))
+                              % (name, blocks, threads, what), step,
+                              {"npes": self.npes, "bytes_per_pe": self.SIZE, "blocks_per_pe": blocks,
+                               "threads_per_block": threads}))
         return items
 
 
