@@ -169,7 +169,7 @@ __global__ __launch_bounds__(WAVE_SPLIT ? 1024 : kCopyThreads) void segment_copy
                                                                 const nvshmemi_amd_team_view_t *groups,
                                                                 int max_size, uint64_t dst_off,
                                                                 uint64_t src_off, uint64_t seg_bytes,
-                                                                int root, uint32_t part_shift) {
+                                                                int root, uint32_t part_shift, uint32_t chunk_shift) {
     // this block's team: members are the PEs start + i*stride, i < size
     const nvshmemi_amd_team_view_t g = groups[blockIdx.z];
     const unsigned npes = (unsigned)g.size;
@@ -218,14 +218,25 @@ __global__ __launch_bounds__(WAVE_SPLIT ? 1024 : kCopyThreads) void segment_copy
     const uint64_t lead = ((uint64_t)(uintptr_t)(dst + head) >> 4) & 63;
     constexpr uint64_t kTileVectors = (uint64_t)kCopyThreads * kCopyUnroll;
     // fcollect / broadcast: 2^part_shift consecutive blocks share a tile and split its destinations
-    const uint64_t v0 = (uint64_t)(WAVE_SPLIT ? blockIdx.x : blockIdx.x >> part_shift) * kTileVectors - lead;
+    // With chunk_shift > 0 the sharers of a tile are 2^chunk_shift blocks apart instead of neighbours: the grid walks a
+    // chunk of 2^chunk_shift tiles once per group of destinations, so the blocks in flight write to few destinations
+    // at a time, each a run of consecutive pieces, and re-read the chunk from the L2 of the XCD that fetched it
+    // (sharers are a multiple of 8 blocks apart).
+    uint64_t tile_index = WAVE_SPLIT ? blockIdx.x : blockIdx.x >> part_shift;
+    unsigned part_index = WAVE_SPLIT ? threadIdx.x / kCopyThreads : blockIdx.x & ((1u << part_shift) - 1);
+    if (!WAVE_SPLIT && chunk_shift) {
+        part_index = (blockIdx.x >> chunk_shift) & ((1u << part_shift) - 1);
+        tile_index = (blockIdx.x & ((1u << chunk_shift) - 1)) +
+                     (((uint64_t)blockIdx.x >> (chunk_shift + part_shift)) << chunk_shift);
+    }
+    const uint64_t v0 = tile_index * kTileVectors - lead;
     if ((int64_t)v0 >= (int64_t)nvec_total) return;
     const char *s = src + head;
     char *d = dst + head;
     const bool aligned = (((uintptr_t)s) & 15) == 0;
     if (MODE != kModeAlltoall) {
         const int per = (nrep + (1 << part_shift) - 1) >> part_shift;
-        const int r0 = (int)(WAVE_SPLIT ? threadIdx.x / kCopyThreads : blockIdx.x & ((1u << part_shift) - 1)) * per;
+        const int r0 = (int)part_index * per;
         const int r1 = r0 + per < nrep ? r0 + per : nrep;
         if (aligned) copy_tile<true, true, kCopyUnroll, NTL, STORE>(d, s, v0, nvec_total, rep_stride, r0, r1);
         else copy_tile<false, true, kCopyUnroll, NTL, STORE>(d, s, v0, nvec_total, rep_stride, r0, r1);
@@ -498,28 +509,51 @@ __global__ __launch_bounds__(kThreads) void reduce_scalar_kernel(char *base, uin
     }
 }
 
-// fcollect / broadcast of sources too large to stay in the Infinity Cache: a wavefront stores its
-// piece to at most four destinations; the blocks that share a piece are neighbours in the grid.
-// Neighbouring work-groups run on different XCDs, so the sharers' loads miss in their L2 and are
-// served by the Infinity Cache (FETCH_SIZE counts the piece once per sharer, HBM reads it once).
-// Putting the sharers on one XCD (8 apart in blockIdx.x) makes L2 serve them and halves FETCH_SIZE,
-// but measured slower (broadcast of 512 MiB: 5.4 against 6.0 TB/s), so they stay neighbours.  Measured with random data: broadcast of 512 MiB to 8 PEs
-// 5.05 -> 6.03 TB/s, fcollect of 16 x 32 MiB 5.25 -> 6.10, of 8 x 64 MiB 5.55 -> 6.2; two or eight
-// destinations per wavefront are slower.  Cache-resident sources keep one wavefront per piece: the
-// split costs them up to 9 %.
+// fcollect / broadcast of sources too large to stay in the Infinity Cache split the destinations of a piece
+// over several wavefronts.  Earlier forms, kept selectable (NVSHMEM_AMD_*_SPLIT 1 and 2): at most four
+// destinations per wavefront, the sharers being neighbouring blocks (they run on different XCDs, so the piece
+// is fetched once per sharer from the Infinity Cache) or the wavefronts of one block: broadcast of 512 MiB to
+// 8 PEs 5.05 -> 6.03 TB/s, fcollect of 16 x 32 MiB 5.25 -> 5.85.  The default is the chunked form below.
+// Cache-resident sources keep one wavefront per piece: a split costs them up to 9 %.
 #ifndef NVSHMEM_AMD_REPLICAS_PER_WAVE
 #define NVSHMEM_AMD_REPLICAS_PER_WAVE 4
 #endif
-#ifndef NVSHMEM_AMD_FCOLLECT_SPLIT /* 0: one wavefront stores to all members; 1: neighbouring blocks share; 2: the wavefronts of one block */
-#define NVSHMEM_AMD_FCOLLECT_SPLIT 2
+#ifndef NVSHMEM_AMD_FCOLLECT_SPLIT /* 0: one wavefront stores to all members; 1: neighbouring blocks share; 2: the wavefronts of one block; 3: chunked */
+#define NVSHMEM_AMD_FCOLLECT_SPLIT 3
 #endif
-#ifndef NVSHMEM_AMD_BROADCAST_SPLIT
-#define NVSHMEM_AMD_BROADCAST_SPLIT 1
+#ifndef NVSHMEM_AMD_BROADCAST_SPLIT /* 0, 1 or 3, as above */
+#define NVSHMEM_AMD_BROADCAST_SPLIT 3
 #endif
-static uint32_t replica_part_shift(int max_size) {
+#ifndef NVSHMEM_AMD_STORE_FCOLLECT_CHUNKED
+#define NVSHMEM_AMD_STORE_FCOLLECT_CHUNKED kStoreThroughStream /* +2 % over nt */
+#endif
+#ifndef NVSHMEM_AMD_STORE_BROADCAST_CHUNKED
+#define NVSHMEM_AMD_STORE_BROADCAST_CHUNKED kStoreStream /* +2.5 % over sc1 nt */
+#endif
+static uint32_t replica_part_shift(int max_size, int per_wave = NVSHMEM_AMD_REPLICAS_PER_WAVE) {
     uint32_t shift = 0;
-    while (((max_size + (1 << shift) - 1) >> shift) > NVSHMEM_AMD_REPLICAS_PER_WAVE) ++shift;
+    while (((max_size + (1 << shift) - 1) >> shift) > per_wave) ++shift;
     return shift;
+}
+
+// Chunked sharing, the form fcollect and broadcast of sources beyond the Infinity Cache take: a wavefront stores
+// its piece to two destinations, and the grid walks a chunk of tiles once per pair of destinations before it moves
+// on (segment_copy_kernel, chunk_shift).  A write-dominated kernel is bound by how the memory system takes its
+// writes, and that favours few write fronts: a write-only stream runs at 6.9 TB/s as ONE front sweeping memory,
+// 5.7-6.2 as 64 fronts, 4.6-5.3 as 256.  With every block storing to all 8 or 16 destinations the blocks in flight
+// feed 8 or 16 fronts of a few KiB each; chunked, they feed a few fronts of 2-4 MiB.  Measured (random data, 16 x
+// 32 MiB fcollect / 512 MiB broadcast to 8): fcollect 5.85 -> 6.30 TB/s, broadcast 6.07 -> 6.48; the chunk that
+// measured best makes chunk x groups = 16384 blocks, twice what the GPU holds at a time (fcollect: 2^11 tiles x
+// 8 pairs; broadcast: 2^12 x 4; half or double that chunk loses 1-12 %), one destination per wavefront 20 %.
+#ifndef NVSHMEM_AMD_CHUNKED_REPLICAS_PER_WAVE
+#define NVSHMEM_AMD_CHUNKED_REPLICAS_PER_WAVE 2
+#endif
+#ifndef NVSHMEM_AMD_CHUNK_CYCLE_SHIFT /* log2 of chunk tiles x destination groups */
+#define NVSHMEM_AMD_CHUNK_CYCLE_SHIFT 14
+#endif
+static uint32_t chunk_shift_for(uint32_t part_shift) {
+    const uint32_t cycle = NVSHMEM_AMD_CHUNK_CYCLE_SHIFT;
+    return cycle > part_shift + 8 ? cycle - part_shift : 8;   // at least 256 tiles (a multiple of the 8 XCDs) per chunk
 }
 
 // members of all teams of the handle together
@@ -810,8 +844,12 @@ int broadcast_on_stream(nvshmem_team_t team, void *dest, const void *src, size_t
     }
     // a source that cannot stay in the Infinity Cache: split the destinations (see replica_part_shift)
     const bool big_source = bytes * (uint64_t)tl.ngroups > rt.cacheable_source_bytes;
-    const uint32_t part_shift = big_source && NVSHMEM_AMD_BROADCAST_SPLIT ? replica_part_shift(tl.max_size) : 0;
-    const uint64_t tiles = ((bytes / 16 + 64 + kCopyThreads - 1) / kCopyThreads + 1) << part_shift;
+    const bool chunked = big_source && NVSHMEM_AMD_BROADCAST_SPLIT == 3;
+    const uint32_t part_shift = chunked ? replica_part_shift(tl.max_size, NVSHMEM_AMD_CHUNKED_REPLICAS_PER_WAVE)
+                                : big_source && NVSHMEM_AMD_BROADCAST_SPLIT ? replica_part_shift(tl.max_size) : 0;
+    const uint32_t chunk_shift = chunked && part_shift ? chunk_shift_for(part_shift) : 0;
+    uint64_t tiles = (bytes / 16 + 64 + kCopyThreads - 1) / kCopyThreads + 1;
+    tiles = ((tiles + (1ull << chunk_shift) - 1) >> chunk_shift << chunk_shift) << part_shift;  // whole chunks
     if (tiles > 0x7fffffffull) {
         set_error("broadcast: message too large");
         return NVSHMEMX_ERROR_INVALID_VALUE;
@@ -821,8 +859,9 @@ int broadcast_on_stream(nvshmem_team_t team, void *dest, const void *src, size_t
 #define NVSHMEM_AMD_LAUNCH_BROADCAST(NTL, STORE)                                                      \
     hipLaunchKernelGGL((segment_copy_kernel<kModeBroadcast, 1, NTL, STORE>), grid, block, 0, stream,    \
                        rt.base, rt.heap_size, tl.groups, tl.max_size, doff, soff, (uint64_t)bytes, root, \
-                       part_shift)
-    if (part_shift != 0) NVSHMEM_AMD_LAUNCH_BROADCAST(false, NVSHMEM_AMD_STORE_REPLICATE_SPLIT);
+                       part_shift, chunk_shift)
+    if (chunk_shift != 0) NVSHMEM_AMD_LAUNCH_BROADCAST(false, NVSHMEM_AMD_STORE_BROADCAST_CHUNKED);
+    else if (part_shift != 0) NVSHMEM_AMD_LAUNCH_BROADCAST(false, NVSHMEM_AMD_STORE_REPLICATE_SPLIT);
     else if (big_source) NVSHMEM_AMD_LAUNCH_BROADCAST(true, NVSHMEM_AMD_STORE_REPLICATE);
     else NVSHMEM_AMD_LAUNCH_BROADCAST(false, NVSHMEM_AMD_STORE_REPLICATE);
 #undef NVSHMEM_AMD_LAUNCH_BROADCAST
@@ -858,13 +897,15 @@ static int segment_collective(int mode, const char *what, nvshmem_team_t team, v
     const uint64_t tile_vectors = (uint64_t)kCopyThreads * (mode == kModeFcollect ? NVSHMEM_AMD_FCOLLECT_UNROLL
                                                                               : NVSHMEM_AMD_ALLTOALL_UNROLL);
     const bool big_source = src_bytes * total_members(tl) > rt.cacheable_source_bytes;
+    const bool chunked = mode == kModeFcollect && big_source && NVSHMEM_AMD_FCOLLECT_SPLIT == 3;
     const uint32_t part_shift =
-        mode == kModeFcollect && big_source && NVSHMEM_AMD_FCOLLECT_SPLIT ? replica_part_shift(tl.max_size) : 0;
-    // fcollect lets the wavefronts of one block share the piece (the same speed as neighbouring blocks,
-    // measured 5.8-6.0 TB/s either way for 8 to 32 members, and the piece crosses the fabric once instead
-    // of once per sharer); the broadcast keeps neighbouring blocks (6.05 against 5.5 TB/s)
+        chunked ? replica_part_shift(tl.max_size, NVSHMEM_AMD_CHUNKED_REPLICAS_PER_WAVE)
+        : mode == kModeFcollect && big_source && NVSHMEM_AMD_FCOLLECT_SPLIT ? replica_part_shift(tl.max_size) : 0;
+    const uint32_t chunk_shift = chunked && part_shift ? chunk_shift_for(part_shift) : 0;
+    // (NVSHMEM_AMD_FCOLLECT_SPLIT 2: the wavefronts of one block share the piece)
     const bool wave_split = part_shift != 0 && NVSHMEM_AMD_FCOLLECT_SPLIT == 2 && (kCopyThreads << part_shift) <= 1024;
-    const uint64_t tiles = ((seg_bytes / 16 + 64 + tile_vectors - 1) / tile_vectors + 1) << (wave_split ? 0 : part_shift);
+    uint64_t tiles = (seg_bytes / 16 + 64 + tile_vectors - 1) / tile_vectors + 1;
+    tiles = ((tiles + (1ull << chunk_shift) - 1) >> chunk_shift << chunk_shift) << (wave_split ? 0 : part_shift);  // whole chunks
     const unsigned segs = mode == kModeFcollect ? (unsigned)n : (unsigned)(n * n);
     if (tiles > 0x7fffffffull) {
         set_error("%s: message too large", what);
@@ -876,12 +917,14 @@ static int segment_collective(int mode, const char *what, nvshmem_team_t team, v
 #define NVSHMEM_AMD_LAUNCH_SEGCOPY(MODE, U, NTL, STORE)                                            \
     hipLaunchKernelGGL((segment_copy_kernel<MODE, U, NTL, STORE>), grid, block, 0, stream, rt.base, \
                        rt.heap_size, tl.groups, tl.max_size, doff, soff, (uint64_t)seg_bytes, 0,   \
-                       part_shift)
+                       part_shift, chunk_shift)
     if (mode == kModeFcollect) {
         if (wave_split)
             hipLaunchKernelGGL((segment_copy_kernel<kModeFcollect, NVSHMEM_AMD_FCOLLECT_UNROLL, true, NVSHMEM_AMD_STORE_WAVE_SPLIT, true>),
                                grid, block, 0, stream, rt.base, rt.heap_size, tl.groups, tl.max_size, doff, soff,
-                               (uint64_t)seg_bytes, 0, part_shift);
+                               (uint64_t)seg_bytes, 0, part_shift, chunk_shift);
+        else if (chunk_shift != 0)
+            NVSHMEM_AMD_LAUNCH_SEGCOPY(kModeFcollect, NVSHMEM_AMD_FCOLLECT_UNROLL, false, NVSHMEM_AMD_STORE_FCOLLECT_CHUNKED);
         else if (part_shift != 0)
             NVSHMEM_AMD_LAUNCH_SEGCOPY(kModeFcollect, NVSHMEM_AMD_FCOLLECT_UNROLL, false, NVSHMEM_AMD_STORE_REPLICATE_SPLIT);
         else if (stream_source)

@@ -183,8 +183,8 @@ def test_small_in_kernel_collectives_with_and_without_packets(disable, plain, mo
 @pytest.mark.parametrize("npes", [3, 8, 13, 16, 33, 64])
 def test_large_source_policy_of_fcollect_and_broadcast(npes, monkeypatch):
     """Sources beyond NVSHMEM_AMD_CACHEABLE_SOURCE_BYTES (read at init) are streamed, and fcollect /
-    broadcast then split the destinations of a piece over neighbouring blocks (at most four per
-    wavefront).  With the threshold at zero every size takes that path: ragged, misaligned messages
+    broadcast then split the destinations of a piece over several wavefronts (two per wavefront, the
+    grid walking a chunk of the message once per pair).  With the threshold at zero every size takes that path: ragged, misaligned messages
     must come out the same, bytes outside the destination untouched."""
     monkeypatch.setenv("NVSHMEM_AMD_CACHEABLE_SOURCE_BYTES", "0")
     monkeypatch.setenv("NVSHMEM_AMD_LDS_REDUCE_BYTES", "0")      # 8 and 16 members: the LDS-staged allreduce
@@ -223,6 +223,37 @@ def test_large_source_policy_of_fcollect_and_broadcast(npes, monkeypatch):
         assert np.array_equal(rt.download_all(fdst, (npes * n * 4,), np.uint8), O.alltoall(fdata.view(np.uint8)))
         for p in (src, dst, fsrc, fdst):
             rt.free(p)
+
+
+@pytest.mark.parametrize("npes", [5, 8, 16])
+def test_large_source_fcollect_and_broadcast_across_several_chunks(npes, monkeypatch):
+    """The large-source form of fcollect / broadcast walks the message in chunks of a few MiB, once per
+    group of destinations: a message of several chunks plus a ragged rest, misaligned at both ends, must
+    arrive whole on every member, with the bytes around the destination untouched."""
+    monkeypatch.setenv("NVSHMEM_AMD_CACHEABLE_SOURCE_BYTES", "0")
+    rng = np.random.default_rng(4100 + npes)
+    nbytes = (9 << 20) + 1234
+    with runtime(npes, (npes + 1) * (10 << 20) + (8 << 20)) as rt:
+        src = rt.malloc(nbytes + 64); dst = rt.malloc(npes * nbytes + 256)
+        data = rng.integers(0, 256, (npes, nbytes), dtype=np.uint8)
+        for soff, doff in ((0, 0), (3, 21)):
+            rt.upload_all(src, data, soff)
+            rt.fill(dst, 0xCD, npes * nbytes + 256)
+            note("chunked fcollect npes=%d bytes=%d soff=%d doff=%d" % (npes, nbytes, soff, doff))
+            rt.fcollectmem(dst + doff, src + soff, nbytes)
+            want = O.fcollect(data)
+            for pe in (0, npes // 2, npes - 1):
+                got = rt.download(dst, pe, (npes * nbytes + doff + 32,), np.uint8)
+                assert np.array_equal(got[doff:doff + npes * nbytes], want[pe]), (pe, soff, doff)
+                assert (got[:doff] == 0xCD).all() and (got[doff + npes * nbytes:] == 0xCD).all()
+            root = npes - 2
+            rt.fill(dst, 0xCD, npes * nbytes + 256)
+            note("chunked broadcast npes=%d bytes=%d root=%d" % (npes, nbytes, root))
+            rt.broadcastmem(dst + doff, src + soff, nbytes, root)
+            got = rt.download_all(dst, (nbytes + doff + 32,), np.uint8)
+            assert np.array_equal(got[:, doff:doff + nbytes], O.broadcast(data, root)), (soff, doff)
+            assert (got[:, :doff] == 0xCD).all() and (got[:, doff + nbytes:] == 0xCD).all()
+        rt.free(src); rt.free(dst)
 
 
 @pytest.mark.parametrize("npes", [3, 5, 12, 24, 32, 33, 48, 64])
