@@ -30,16 +30,26 @@ __global__ void moe_dispatch_rowsignal_kernel(char *recv, const char *send, cons
         const size_t waves_per_block = blockDim.x / NVSHMEMI_WARP_SIZE;
         const size_t wave = blockIdx.x * waves_per_block + wave_in_block();
         const size_t nwaves = (size_t)gridDim.x * waves_per_block;
-        // a wavefront takes a token and sends its topk copies one behind the other, so that the
-        // copies after the first find the row in this XCD's L2
-        for (size_t t = wave; t < (size_t)tokens; t += nwaves)
-            for (int k = 0; k < topk; ++k) {
+        // Up to four consecutive wavefronts of a block share a token and send a quarter of its topk copies each,
+        // one behind the other: the token's row is fetched from memory once, by whichever of them comes first,
+        // and every other read of it hits in this XCD's L2.  (A wavefront that sent all topk copies of its own
+        // token re-read the row seven times while 255 other wavefronts of the XCD streamed their rows through the
+        // same 4 MiB: about one re-read in seven missed - measured traffic 1.13 times the algorithmic bytes, 1.00
+        // with the sharing, at the same or a slightly better rate.)
+        unsigned share = 1;
+        while (share < 4 && waves_per_block % (2 * share) == 0 && topk % (int)(2 * share) == 0) share *= 2;
+        const int per = topk / (int)share;
+        for (size_t u = wave; u < (size_t)tokens * share; u += nwaves) {
+            const size_t t = u / share;
+            const int k0 = (int)(u % share) * per;
+            for (int k = k0; k < k0 + per; ++k) {
                 const size_t r = t * (size_t)topk + (size_t)k;
                 if (row_ok(my_dest_pe[r], my_dest_row[r], np, recv_cap_rows))
                     nvshmemx_putmem_signal_nbi_warp(recv + (size_t)my_dest_row[r] * row_bytes,
                                                     send + t * row_bytes, row_bytes,
                                                     sig + (size_t)me * sig_stride, 1, sig_op, my_dest_pe[r]);
             }
+        }
     } else {
         for (size_t r = blockIdx.x; r < rows; r += gridDim.x)
             if (row_ok(my_dest_pe[r], my_dest_row[r], np, recv_cap_rows))

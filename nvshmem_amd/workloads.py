@@ -400,6 +400,12 @@ class MoeShuffle(Group):
             it.what = what
             # the library-wide order of put-with-signal: payload-only for the first row, the default for the rest
             it.prepare = (lambda on=(what == "put_signal"): rt.lib.nvshmemx_amd_set_put_signal_order(1 if on else 0))
+
+        def prepare_combine():
+            # the combine gathers what a dispatch delivered: run one (whatever ran before may have sent a part only)
+            rt.lib.nvshmemx_amd_set_put_signal_order(0)
+            plain_store()
+        items[-1].prepare = prepare_combine
         return items
 
 
