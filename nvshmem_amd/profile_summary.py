@@ -45,8 +45,8 @@ COMMANDS = """Commands (on the GPU box, from the repository root; every file the
   export NVSHMEM_AMD_PLAIN_COLLECTIVE_LAUNCH=1   (kernels that nvshmemx_collective_launch starts are started with a plain
       launch: after a cooperative launch the profiled process crashes in an exit handler of the profiler's stack, behind
       the written results; the kernels and their grids are the same)
-  rocprofv3 --kernel-trace --stats -d $OUT/stats -- python3 $REPO/nvshmem_amd/profile_workloads.py --iters 4 --manifest $OUT/manifest.json
-  rocprofv3 --pmc FETCH_SIZE -d $OUT/p1 -- python3 $REPO/nvshmem_amd/profile_workloads.py --iters 4 --manifest $OUT/manifest.json
+  rocprofv3 --kernel-trace --stats -d $OUT/stats -- python3 $REPO/nvshmem_amd/profile_workloads.py --iters 8 --manifest $OUT/manifest.json
+  rocprofv3 --pmc FETCH_SIZE -d $OUT/p1 -- python3 $REPO/nvshmem_amd/profile_workloads.py --iters 8 --manifest $OUT/manifest.json
   rocprofv3 --pmc WRITE_SIZE -d $OUT/p2 -- (the same)
   rocprofv3 --pmc TCP_TCC_READ_REQ_sum TCP_TCC_READ_REQ_LATENCY_sum TCP_TCC_WRITE_REQ_sum TCP_TCC_WRITE_REQ_LATENCY_sum GRBM_GUI_ACTIVE -d $OUT/p3 -- (the same)
   rocprofv3 --pmc SQ_WAVES SQ_BUSY_CYCLES SQ_WAIT_INST_ANY SQ_INSTS_VMEM_RD SQ_INSTS_VMEM_WR SQ_INST_LEVEL_VMEM TCP_PENDING_STALL_CYCLES_sum TCP_TCR_TCP_STALL_CYCLES_sum -d $OUT/p4 -- (the same)
