@@ -172,11 +172,11 @@ typedef nvshmemi_v4u __attribute__((aligned(1))) nvshmemi_v4u_unaligned;
 #endif
 /* Long copies - a lane owns at least NVSHMEMI_AMD_COPY_DEEP_MIN vectors - run rounds of
  * NVSHMEMI_AMD_COPY_DEEP_UNROLL vectors per lane first (0 switches them off).  Eight is what fits the
- * registers the rest of the engine needs anyway.  Sixteen measured 6 % more for 16 blocks of 1024
- * threads that each stream a 16 MiB slice, but its 28 extra vector registers lower the occupancy of
- * every kernel that inlines the engine, and kernels of one-wavefront blocks that move 1-2 KiB each -
- * the fastest shapes on this GPU - lost 9-13 %.  (A block that streams a long slice alone on its
- * compute unit moves about 31 GB/s of payload whatever the depth: see the counter profiles.) */
+ * registers the rest of the engine needs anyway.  Sixteen takes 30 more vector registers (82 in all: five
+ * wavefronts per SIMD instead of eight), which cost kernels of one-wavefront blocks that move 1-2 KiB each
+ * 9-13 %, and buys nothing any more: large blocks, whose loads and stores run in separate runs (below),
+ * measure the same at 8, 12 and 16.  (A block that streams a long slice alone on its compute unit moves
+ * about 39 GB/s of payload whatever the depth: the unit keeps some 15 KiB of requests in flight.) */
 #ifndef NVSHMEMI_AMD_COPY_DEEP_UNROLL
 #define NVSHMEMI_AMD_COPY_DEEP_UNROLL 8
 #endif

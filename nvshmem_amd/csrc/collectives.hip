@@ -238,6 +238,7 @@ __global__ __launch_bounds__(WAVE_SPLIT ? 1024 : kCopyThreads) void segment_copy
         const int per = (nrep + (1 << part_shift) - 1) >> part_shift;
         const int r0 = (int)part_index * per;
         const int r1 = r0 + per < nrep ? r0 + per : nrep;
+        if (r0 >= nrep) return;  // a team smaller than the grid's largest: nothing left for this sharer
         if (aligned) copy_tile<true, true, kCopyUnroll, NTL, STORE>(d, s, v0, nvec_total, rep_stride, r0, r1);
         else copy_tile<false, true, kCopyUnroll, NTL, STORE>(d, s, v0, nvec_total, rep_stride, r0, r1);
     } else {
@@ -381,7 +382,8 @@ __global__ __launch_bounds__(NPES ? NPES / MPW * 64 : 1024) void reduce_vector_k
 // wavefront, lane i loads vector i of a 1 KiB piece from every member, eight loads in flight at a time,
 // folds in member order and stores the result to every member.
 // NPES > 0 fixes the team size at compile time (loads, fold and stores fully unrolled).
-template <typename T, int OP, int NPES, bool NTL>
+// ROOT_ONLY: the result goes to member 0's destination only (the first half of the two-step allreduce of large teams).
+template <typename T, int OP, int NPES, bool NTL, bool ROOT_ONLY = false>
 __global__ __launch_bounds__(64) void reduce_gather_kernel(char *base, uint64_t slice_bytes,
                                                            const nvshmemi_amd_team_view_t *groups,
                                                            uint64_t dst_off, uint64_t src_off, uint64_t nelems) {
@@ -421,8 +423,12 @@ __global__ __launch_bounds__(64) void reduce_gather_kernel(char *base, uint64_t 
                 }
         }
         char *dst = base + dst_off + 16 * v;
+        if (ROOT_ONLY) {
+            stream_store<NVSHMEM_AMD_STORE_REDUCESCATTER>(dst, acc.v);
+        } else {
 #pragma unroll kStores
-        for (int p = 0; p < npes; ++p) stream_store<NVSHMEM_AMD_STORE_REDUCE>(dst + (uint64_t)p * pe_stride, acc.v);
+            for (int p = 0; p < npes; ++p) stream_store<NVSHMEM_AMD_STORE_REDUCE>(dst + (uint64_t)p * pe_stride, acc.v);
+        }
     }
     // elements behind the last full vector
     const uint64_t done = nvec * VEC;
@@ -434,7 +440,7 @@ __global__ __launch_bounds__(64) void reduce_gather_kernel(char *base, uint64_t 
         const uint64_t es = pe_stride / sizeof(T);
         T acc = s[k];
         for (int p = 1; p < npes; ++p) acc = nvshmemi_amd_fold_step<T, OP>(p, acc, s[(uint64_t)p * es + k]);
-        for (int p = 0; p < npes; ++p) d[(uint64_t)p * es + k] = acc;
+        for (int p = 0; p < (ROOT_ONLY ? 1 : npes); ++p) d[(uint64_t)p * es + k] = acc;
     }
 }
 
@@ -551,6 +557,14 @@ static uint32_t replica_part_shift(int max_size, int per_wave = NVSHMEM_AMD_REPL
 #ifndef NVSHMEM_AMD_CHUNK_CYCLE_SHIFT /* log2 of chunk tiles x destination groups */
 #define NVSHMEM_AMD_CHUNK_CYCLE_SHIFT 14
 #endif
+// Groups of the chunked form: the largest power of two that leaves every group at least
+// NVSHMEM_AMD_CHUNKED_REPLICAS_PER_WAVE destinations (16 members: 8 groups of 2; 24: 8 of 3; 5: 2 groups of 3 and 2),
+// so that no group is empty.
+static uint32_t chunked_part_shift(int max_size) {
+    uint32_t shift = 0;
+    while ((max_size >> (shift + 1)) >= NVSHMEM_AMD_CHUNKED_REPLICAS_PER_WAVE) ++shift;
+    return shift;
+}
 static uint32_t chunk_shift_for(uint32_t part_shift) {
     const uint32_t cycle = NVSHMEM_AMD_CHUNK_CYCLE_SHIFT;
     return cycle > part_shift + 8 ? cycle - part_shift : 8;   // at least 256 tiles (a multiple of the 8 XCDs) per chunk
@@ -560,6 +574,40 @@ static uint32_t chunk_shift_for(uint32_t part_shift) {
 static uint64_t total_members(const TeamLaunch &tl) {
     // sizes lie between min and max; the exact sum only matters for the cache policy threshold
     return (uint64_t)tl.ngroups * (uint64_t)tl.max_size;
+}
+
+// Launches the broadcast kernel: member `root`'s [soff, +bytes) to every member's [doff, +bytes).
+static int launch_broadcast(Runtime &rt, const TeamLaunch &tl, uint64_t doff, uint64_t soff, uint64_t bytes, int root,
+                            hipStream_t stream, bool force_chunked = false) {
+    // a source that cannot stay in the Infinity Cache: split the destinations (see replica_part_shift)
+    const bool big_source = force_chunked || bytes * (uint64_t)tl.ngroups > rt.cacheable_source_bytes;
+    const bool chunked = big_source && NVSHMEM_AMD_BROADCAST_SPLIT == 3;
+    const uint32_t part_shift = chunked ? chunked_part_shift(tl.max_size)
+                                : big_source && NVSHMEM_AMD_BROADCAST_SPLIT ? replica_part_shift(tl.max_size) : 0;
+    const uint32_t chunk_shift = chunked && part_shift ? chunk_shift_for(part_shift) : 0;
+    uint64_t tiles = (bytes / 16 + 64 + kCopyThreads - 1) / kCopyThreads + 1;
+    tiles = ((tiles + (1ull << chunk_shift) - 1) >> chunk_shift << chunk_shift) << part_shift;  // whole chunks
+    if (tiles > 0x7fffffffull) {
+        set_error("broadcast: message too large");
+        return NVSHMEMX_ERROR_INVALID_VALUE;
+    }
+    const dim3 grid((unsigned)tiles, 1, (unsigned)tl.ngroups), block(kCopyThreads);
+    // blocks that share a piece re-read it from the cache, so the loads stay cacheable then
+#define NVSHMEM_AMD_LAUNCH_BROADCAST(NTL, STORE)                                                      \
+    hipLaunchKernelGGL((segment_copy_kernel<kModeBroadcast, 1, NTL, STORE>), grid, block, 0, stream,    \
+                       rt.base, rt.heap_size, tl.groups, tl.max_size, doff, soff, (uint64_t)bytes, root, \
+                       part_shift, chunk_shift)
+    if (chunk_shift != 0) NVSHMEM_AMD_LAUNCH_BROADCAST(false, NVSHMEM_AMD_STORE_BROADCAST_CHUNKED);
+    else if (part_shift != 0) NVSHMEM_AMD_LAUNCH_BROADCAST(false, NVSHMEM_AMD_STORE_REPLICATE_SPLIT);
+    else if (big_source) NVSHMEM_AMD_LAUNCH_BROADCAST(true, NVSHMEM_AMD_STORE_REPLICATE);
+    else NVSHMEM_AMD_LAUNCH_BROADCAST(false, NVSHMEM_AMD_STORE_REPLICATE);
+#undef NVSHMEM_AMD_LAUNCH_BROADCAST
+    hipError_t e = hipGetLastError();
+    if (e != hipSuccess) {
+        set_error("broadcast: kernel launch failed: %s", hipGetErrorString(e));
+        return NVSHMEMX_ERROR_INTERNAL;
+    }
+    return 0;
 }
 
 template <typename T, int OP>
@@ -591,6 +639,31 @@ void launch_reduce(Runtime &rt, const TeamLaunch &tl, uint64_t dst_off, uint64_t
     else if (fixed_size == 32) ct_size = 32, mpw = 2;
     else if (tl.max_size >= 3 && tl.max_size <= 32) mpw = 2;
     else if (tl.max_size > 32 && tl.max_size <= 64) mpw = 4;
+    // Two-step allreduce of large teams: fold into member 0's destination (n loads and ONE store per vector, the
+    // shape of the reducescatter), then broadcast that in the chunked form.  It moves 2 n + 2 units where the fused
+    // kernel moves 2 n, but every block of the fused kernel feeds n write fronts of 1 KiB pieces, and its fold
+    // serialises n steps between two barriers.  fp32 sum, TB/s, fused / two-step at 512 MiB and 2 GiB of sources in
+    // all: 12 members 6.41 / 6.18 and 6.28 / 6.29, 16: 6.26 / 6.19 and 6.02 / 6.41, 24: 5.84 / 5.71 and 5.69 / 6.23,
+    // 32: 6.09 / 6.09 and 6.09 / 6.51, 48: 5.68 / 5.78 and 5.57 / 6.25, 64: 5.55 / 5.97 and 5.59 / 6.56.  So: from
+    // Runtime::two_step_reduce_members (16) members on when the sources hold two_step_reduce_bytes (1 GiB) or more,
+    // and from three times that many members whatever the size.
+    if (vector_ok && rt.two_step_reduce_members && tl.min_size >= (int)rt.two_step_reduce_members &&
+        (total_bytes >= rt.two_step_reduce_bytes || tl.min_size >= 3 * (int)rt.two_step_reduce_members) &&
+        total_members(tl) * nelems > rt.lds_reduce_bytes / 4) {
+        const uint64_t nvec = nelems / (16 / sizeof(T));
+        uint64_t blocks = (nvec + 63 + 63) / 64;
+        if (blocks <= 0x7fffffffull) {
+            const dim3 grid((unsigned)blocks, 1, ngroups);
+            if (stream_source)
+                hipLaunchKernelGGL((reduce_gather_kernel<T, OP, 0, true, true>), grid, dim3(64), 0, stream, rt.base,
+                                   rt.heap_size, tl.groups, dst_off, src_off, nelems);
+            else
+                hipLaunchKernelGGL((reduce_gather_kernel<T, OP, 0, false, true>), grid, dim3(64), 0, stream, rt.base,
+                                   rt.heap_size, tl.groups, dst_off, src_off, nelems);
+            (void)launch_broadcast(rt, tl, dst_off, dst_off, nelems * sizeof(T), 0, stream, true);
+            return;
+        }
+    }
     if (vector_ok && mpw && total_members(tl) * nelems > rt.lds_reduce_bytes / 4) {
         const uint32_t lane_shift = 6;
         const unsigned threads = (unsigned)((tl.max_size + mpw - 1) / mpw) << lane_shift;
@@ -842,35 +915,7 @@ int broadcast_on_stream(nvshmem_team_t team, void *dest, const void *src, size_t
         set_error("broadcast: dest and source overlap without being identical");
         return NVSHMEMX_ERROR_INVALID_VALUE;
     }
-    // a source that cannot stay in the Infinity Cache: split the destinations (see replica_part_shift)
-    const bool big_source = bytes * (uint64_t)tl.ngroups > rt.cacheable_source_bytes;
-    const bool chunked = big_source && NVSHMEM_AMD_BROADCAST_SPLIT == 3;
-    const uint32_t part_shift = chunked ? replica_part_shift(tl.max_size, NVSHMEM_AMD_CHUNKED_REPLICAS_PER_WAVE)
-                                : big_source && NVSHMEM_AMD_BROADCAST_SPLIT ? replica_part_shift(tl.max_size) : 0;
-    const uint32_t chunk_shift = chunked && part_shift ? chunk_shift_for(part_shift) : 0;
-    uint64_t tiles = (bytes / 16 + 64 + kCopyThreads - 1) / kCopyThreads + 1;
-    tiles = ((tiles + (1ull << chunk_shift) - 1) >> chunk_shift << chunk_shift) << part_shift;  // whole chunks
-    if (tiles > 0x7fffffffull) {
-        set_error("broadcast: message too large");
-        return NVSHMEMX_ERROR_INVALID_VALUE;
-    }
-    const dim3 grid((unsigned)tiles, 1, (unsigned)tl.ngroups), block(kCopyThreads);
-    // blocks that share a piece re-read it from the cache, so the loads stay cacheable then
-#define NVSHMEM_AMD_LAUNCH_BROADCAST(NTL, STORE)                                                      \
-    hipLaunchKernelGGL((segment_copy_kernel<kModeBroadcast, 1, NTL, STORE>), grid, block, 0, stream,    \
-                       rt.base, rt.heap_size, tl.groups, tl.max_size, doff, soff, (uint64_t)bytes, root, \
-                       part_shift, chunk_shift)
-    if (chunk_shift != 0) NVSHMEM_AMD_LAUNCH_BROADCAST(false, NVSHMEM_AMD_STORE_BROADCAST_CHUNKED);
-    else if (part_shift != 0) NVSHMEM_AMD_LAUNCH_BROADCAST(false, NVSHMEM_AMD_STORE_REPLICATE_SPLIT);
-    else if (big_source) NVSHMEM_AMD_LAUNCH_BROADCAST(true, NVSHMEM_AMD_STORE_REPLICATE);
-    else NVSHMEM_AMD_LAUNCH_BROADCAST(false, NVSHMEM_AMD_STORE_REPLICATE);
-#undef NVSHMEM_AMD_LAUNCH_BROADCAST
-    hipError_t e = hipGetLastError();
-    if (e != hipSuccess) {
-        set_error("broadcast: kernel launch failed: %s", hipGetErrorString(e));
-        return NVSHMEMX_ERROR_INTERNAL;
-    }
-    return 0;
+    return launch_broadcast(rt, tl, doff, soff, bytes, root, stream);
 }
 
 static int segment_collective(int mode, const char *what, nvshmem_team_t team, void *dest,
@@ -899,7 +944,7 @@ static int segment_collective(int mode, const char *what, nvshmem_team_t team, v
     const bool big_source = src_bytes * total_members(tl) > rt.cacheable_source_bytes;
     const bool chunked = mode == kModeFcollect && big_source && NVSHMEM_AMD_FCOLLECT_SPLIT == 3;
     const uint32_t part_shift =
-        chunked ? replica_part_shift(tl.max_size, NVSHMEM_AMD_CHUNKED_REPLICAS_PER_WAVE)
+        chunked ? chunked_part_shift(tl.max_size)
         : mode == kModeFcollect && big_source && NVSHMEM_AMD_FCOLLECT_SPLIT ? replica_part_shift(tl.max_size) : 0;
     const uint32_t chunk_shift = chunked && part_shift ? chunk_shift_for(part_shift) : 0;
     // (NVSHMEM_AMD_FCOLLECT_SPLIT 2: the wavefronts of one block share the piece)

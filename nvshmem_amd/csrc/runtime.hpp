@@ -65,6 +65,12 @@ struct Runtime {
     // all PEs together hold more than this many bytes' worth of 4-byte elements:
     // NVSHMEM_AMD_LDS_REDUCE_BYTES, read at init
     uint64_t lds_reduce_bytes = (uint64_t)256 << 20;
+    // An allreduce beyond the cache takes two steps - fold into member 0, chunked broadcast - instead of the fused
+    // kernel from this team size on (NVSHMEM_AMD_TWO_STEP_REDUCE_MEMBERS, read at init; 0 = never) when the
+    // sources of all members together hold at least two_step_reduce_bytes (NVSHMEM_AMD_TWO_STEP_REDUCE_BYTES), and
+    // from three times the team size at any size
+    unsigned two_step_reduce_members = 16;
+    uint64_t two_step_reduce_bytes = (uint64_t)1 << 30;
     uint64_t timeouts_seen = 0;  // bounded waits that gave up, as far as the host has reported them
 
     static Runtime &get();

@@ -263,7 +263,24 @@ def test_lds_staged_allreduce_for_every_team_size_class(npes, monkeypatch):
     compile-time size.  With the threshold at zero small messages take it too: ragged counts, buffers that
     do not start on a 1 KiB boundary, in place, order-sensitive fp32 and bf16 sums, NaN-carrying max."""
     monkeypatch.setenv("NVSHMEM_AMD_LDS_REDUCE_BYTES", "0")
-    rng = np.random.default_rng(7000 + npes)
+    monkeypatch.setenv("NVSHMEM_AMD_TWO_STEP_REDUCE_MEMBERS", "0")     # (the two-step form has its own test)
+    _allreduce_battery(npes, np.random.default_rng(7000 + npes), "lds")
+
+
+@pytest.mark.parametrize("npes", [4, 16, 24, 33, 64])
+def test_two_step_allreduce(npes, monkeypatch):
+    """Large teams with sources beyond the cache fold into member 0's destination and broadcast that
+    (NVSHMEM_AMD_TWO_STEP_REDUCE_MEMBERS / _BYTES, read at init).  With the thresholds lowered every size and
+    team takes that path: the same battery as the fused kernel - ragged counts, misaligned buffers, in place,
+    NaN-carrying max, bf16, int64, families of ragged teams - must come out bit for bit the same."""
+    monkeypatch.setenv("NVSHMEM_AMD_LDS_REDUCE_BYTES", "0")
+    monkeypatch.setenv("NVSHMEM_AMD_CACHEABLE_SOURCE_BYTES", "0")
+    monkeypatch.setenv("NVSHMEM_AMD_TWO_STEP_REDUCE_MEMBERS", "2")
+    monkeypatch.setenv("NVSHMEM_AMD_TWO_STEP_REDUCE_BYTES", "0")
+    _allreduce_battery(npes, np.random.default_rng(7100 + npes), "two-step")
+
+
+def _allreduce_battery(npes, rng, tag):
     with runtime(npes, 16 << 20) as rt:
         cap = 40000
         src = rt.malloc(cap * 8 + 1024); dst = rt.malloc(cap * 8 + 1024)
@@ -271,7 +288,7 @@ def test_lds_staged_allreduce_for_every_team_size_class(npes, monkeypatch):
             f = (rng.standard_normal((npes, n)) * 10.0 ** rng.integers(-3, 4, (npes, n))).astype(np.float32)
             rt.upload_all(src, f, off)
             rt.fill(dst, 0xCD, cap * 8 + 1024)
-            note("lds allreduce npes=%d float sum n=%d off=%d" % (npes, n, off))
+            note("%s allreduce npes=%d float sum n=%d off=%d" % (tag, npes, n, off))
             rt.reduce("float", "sum", dst + off, src + off, n)
             want = O.reduce("f32", "sum", f)
             got = rt.download_all(dst, ((off + n * 4 + 64) // 4,), np.uint32)
@@ -283,7 +300,7 @@ def test_lds_staged_allreduce_for_every_team_size_class(npes, monkeypatch):
         f[rng.integers(0, npes, 50), rng.integers(0, n, 50)] = np.nan
         f[rng.integers(0, npes, 50), rng.integers(0, n, 50)] = -0.0
         rt.upload_all(src, f)
-        note("lds allreduce npes=%d float max with NaN, in place" % npes)
+        note("%s allreduce npes=%d float max with NaN, in place" % (tag, npes))
         rt.reduce("float", "max", src, src, n)
         want = O.reduce("f32", "max", f)
         assert all(bits_equal(rt.download(src, pe, (n,), np.float32), want) for pe in (0, npes // 2, npes - 1))
@@ -300,7 +317,7 @@ def test_lds_staged_allreduce_for_every_team_size_class(npes, monkeypatch):
         xt, yt = rt.team_split_2d(N.TEAM_WORLD, xr)
         f = (rng.standard_normal((npes, n)) * 10.0 ** rng.integers(-3, 4, (npes, n))).astype(np.float32)
         rt.upload_all(src, f)
-        note("lds allreduce npes=%d rows of %d" % (npes, xr))
+        note("%s allreduce npes=%d rows of %d" % (tag, npes, xr))
         rt.reduce("float", "sum", dst, src, n, team=xt)
         for r0 in range(0, npes, xr):
             members = list(range(r0, min(r0 + xr, npes)))
