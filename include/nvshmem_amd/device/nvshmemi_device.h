@@ -186,12 +186,13 @@ typedef nvshmemi_v4u __attribute__((aligned(1))) nvshmemi_v4u_unaligned;
 /* Cache policy of the vector body.  Stores stream (non-temporal): a copy never reads its destination
  * back.  Loads stay cacheable for short and medium copies, because callers often push the same source
  * to several PEs (top-k token dispatch, all-push collectives) and the repeats then hit in L2 (measured
- * 1.4x on the MoE dispatch); a single copy of NVSHMEMI_AMD_COPY_NT_BYTES (8 MiB) or more streams its
- * loads too (measured +5 % on a 256 MiB put, +1.3 % on 16 MiB slices; 1 MiB as the threshold gains
- * nothing over 8).  NVSHMEMI_AMD_COPY_NT overrides the choice for a translation
- * unit: bit 0 set = always non-temporal loads, 0 = never; bit 1 = non-temporal stores. */
+ * 1.4x on the MoE dispatch); a single copy of NVSHMEMI_AMD_COPY_NT_BYTES (1 MiB) or more streams its
+ * loads too (measured +5 % on a 256 MiB put from 16 blocks per PE and +5.5 % on a 64 MiB one, whose blocks
+ * move 4 MiB each; 64 KiB as the threshold gains nothing over 1 MiB).  NVSHMEMI_AMD_COPY_NT overrides the
+ * choice for a translation unit: bit 0 set = always non-temporal loads, 0 = never; bit 1 = non-temporal
+ * stores. */
 #ifndef NVSHMEMI_AMD_COPY_NT_BYTES
-#define NVSHMEMI_AMD_COPY_NT_BYTES (8u << 20)
+#define NVSHMEMI_AMD_COPY_NT_BYTES (1u << 20)
 #endif
 
 /* A 16-byte store at agent scope (written through the L2).  The compiler has no such store, so it is
