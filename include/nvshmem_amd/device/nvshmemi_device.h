@@ -1078,6 +1078,37 @@ NVSHMEMI_DEVICE_INLINE T nvshmemi_amd_fold_step(int i, T acc, T x) {
     return (i == 1) ? nvshmemi_amd_reduce_op<T, OP>(acc, x) : nvshmemi_amd_reduce_op<T, OP>(x, acc);
 }
 
+/* The form an accumulator takes between the steps of a fold.  For most types it is the element itself.  A
+ * bf16 sum or product keeps it as the fp32 value of the rounded bf16 (the bf16's bits in the high half of the
+ * word), which v_cvt_pk_bf16_f32 writes directly when the value is its second operand: a step is then
+ * add + convert instead of add + convert + shift, with the same rounding, once per step. */
+template <typename T, int OP>
+struct nvshmemi_amd_fold_form {
+    typedef T acc_t;
+    static NVSHMEMI_DEVICE_INLINE acc_t lift(T x) { return x; }
+    static NVSHMEMI_DEVICE_INLINE acc_t step(int i, acc_t acc, T x) { return nvshmemi_amd_fold_step<T, OP>(i, acc, x); }
+    static NVSHMEMI_DEVICE_INLINE T lower(acc_t acc) { return acc; }
+};
+template <int OP>
+struct nvshmemi_amd_bf16_float_form {
+    typedef float acc_t;
+    static NVSHMEMI_DEVICE_INLINE acc_t lift(__hip_bfloat16 x) {
+        return __builtin_bit_cast(float, (unsigned)__builtin_bit_cast(unsigned short, x) << 16);
+    }
+    static NVSHMEMI_DEVICE_INLINE acc_t step(int i, acc_t acc, __hip_bfloat16 x) {
+        typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
+        typedef float floatx2 __attribute__((ext_vector_type(2)));
+        const float a = (i == 1) ? acc : lift(x), b = (i == 1) ? lift(x) : acc;
+        const floatx2 wide = {0.0f, OP == NVSHMEMI_OP_sum ? a + b : a * b};
+        return __builtin_bit_cast(float, __builtin_convertvector(wide, bf16x2));
+    }
+    static NVSHMEMI_DEVICE_INLINE __hip_bfloat16 lower(acc_t acc) {
+        return __builtin_bit_cast(__hip_bfloat16, (unsigned short)(__builtin_bit_cast(unsigned, acc) >> 16));
+    }
+};
+template <> struct nvshmemi_amd_fold_form<__hip_bfloat16, NVSHMEMI_OP_sum> : nvshmemi_amd_bf16_float_form<NVSHMEMI_OP_sum> {};
+template <> struct nvshmemi_amd_fold_form<__hip_bfloat16, NVSHMEMI_OP_prod> : nvshmemi_amd_bf16_float_form<NVSHMEMI_OP_prod> {};
+
 /* ------------------------------------------------------------------------------------------------
  * Low-latency packets for small collectives (the role of the reference's LL protocol,
  * non_abi/device/common/nvshmemi_common_device.cuh:981-1066 packLL / recvLL, used by

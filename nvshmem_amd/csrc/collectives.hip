@@ -323,13 +323,17 @@ __global__ __launch_bounds__(NPES ? NPES / MPW * 64 : 1024) void reduce_vector_k
         // narrower elements that share the word, each folded on its own in member order - so that a tile of
         // 1- or 2-byte elements costs as many LDS instructions as one of 4-byte elements
         for (unsigned w = threadIdx.x; w < tile_words; w += blockDim.x) {
-            word_t acc = stage_w[w];
+            typedef nvshmemi_amd_fold_form<T, OP> form;
+            const word_t first = stage_w[w];
+            typename form::acc_t acc[EPW];
+#pragma unroll
+            for (int j = 0; j < EPW; ++j) acc[j] = form::lift(first.e[j]);
             if (NPES) {
 #pragma unroll
                 for (int p = 1; p < NPES; ++p) {
                     const word_t x = stage_w[(size_t)p * tile_words + w];
 #pragma unroll
-                    for (int j = 0; j < EPW; ++j) acc.e[j] = nvshmemi_amd_fold_step<T, OP>(p, acc.e[j], x.e[j]);
+                    for (int j = 0; j < EPW; ++j) acc[j] = form::step(p, acc[j], x.e[j]);
                 }
             } else {
                 // eight members' values fetched from LDS before they are folded, in member order
@@ -341,15 +345,18 @@ __global__ __launch_bounds__(NPES ? NPES / MPW * 64 : 1024) void reduce_vector_k
 #pragma unroll
                     for (int k = 0; k < 8; ++k)
 #pragma unroll
-                        for (int j = 0; j < EPW; ++j) acc.e[j] = nvshmemi_amd_fold_step<T, OP>(p + k, acc.e[j], x[k].e[j]);
+                        for (int j = 0; j < EPW; ++j) acc[j] = form::step(p + k, acc[j], x[k].e[j]);
                 }
                 for (; p < npes; ++p) {
                     const word_t x = stage_w[(size_t)p * tile_words + w];
 #pragma unroll
-                    for (int j = 0; j < EPW; ++j) acc.e[j] = nvshmemi_amd_fold_step<T, OP>(p, acc.e[j], x.e[j]);
+                    for (int j = 0; j < EPW; ++j) acc[j] = form::step(p, acc[j], x.e[j]);
                 }
             }
-            result_w[w] = acc;
+            word_t out;
+#pragma unroll
+            for (int j = 0; j < EPW; ++j) out.e[j] = form::lower(acc[j]);
+            result_w[w] = out;
         }
         __syncthreads();
 #pragma unroll
