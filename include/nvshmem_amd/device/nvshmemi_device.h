@@ -611,6 +611,9 @@ NVSHMEMI_DEVICE_INLINE void nvshmemi_amd_record_timeout(const void *addr, uint64
     rec[2] = found;
     rec[3] = expected;
     __hip_atomic_store(rec, seq, __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_AGENT);
+    /* the host's copy of "something happened": any number of this period differs from what the host saw last */
+    if (nvshmemi_device_state_d.timeout_flag)
+        __hip_atomic_store(nvshmemi_device_state_d.timeout_flag, seq, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
 }
 
 /* Spin until `*ivar cmp value`; `ivar` is a local operand.  Returns the value that ended the wait.

@@ -248,6 +248,9 @@ typedef struct nvshmemi_device_state {
                                 word NVSHMEMI_AMD_TIMEOUT_COUNT_WORD counts the bounded waits that gave up */
     uint64_t heap_magic;     /* floor(2^40 / (heap_size >> 21)) + 1: the slice that holds heap offset d is
                                 ((d >> 21) * heap_magic) >> 40 (exact while the whole heap is at most 512 GiB) */
+    uint64_t *timeout_flag;  /* pinned host memory (or null): a bounded wait that gives up stores its timeout's
+                                number here too, so that the host's check after a synchronisation is one load and
+                                the count is fetched from the GPU only when something happened */
 } nvshmemi_device_state_t;
 
 #define NVSHMEMI_AMD_TIMEOUT_COUNT_WORD 0

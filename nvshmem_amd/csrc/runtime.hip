@@ -63,6 +63,12 @@ bool check_symmetric_range(Runtime &rt, const char *what, const void *p, uint64_
 
 uint64_t report_timeouts(Runtime &rt, const char *where) {
     if (!rt.initialized || !rt.dev.runtime_words) return 0;
+    // callers have synchronised with the device: what a kernel stored to the pinned word has arrived
+    if (rt.timeout_flag) {
+        const uint64_t flag = __atomic_load_n(rt.timeout_flag, __ATOMIC_ACQUIRE);
+        if (flag == rt.timeout_flag_seen) return 0;
+        rt.timeout_flag_seen = flag;
+    }
     uint64_t count = 0;
     if (hipMemcpy(&count, rt.dev.runtime_words + NVSHMEMI_AMD_TIMEOUT_COUNT_WORD, sizeof count,
                   hipMemcpyDeviceToHost) != hipSuccess) {
@@ -239,6 +245,16 @@ int nvshmemx_amd_init(int npes, size_t symmetric_size) {
     rt.dev.sync_epoch = (uint64_t *)(uintptr_t)epoch;
     rt.dev.timeout_record = (uint64_t *)(uintptr_t)trec;
     rt.dev.runtime_words = (uint64_t *)(uintptr_t)(trec + NVSHMEMI_MALLOC_ALIGNMENT);
+    void *flag = nullptr;
+    if (hipHostMalloc(&flag, sizeof(uint64_t), hipHostMallocDefault) == hipSuccess && flag) {
+        rt.timeout_flag = (uint64_t *)flag;
+        *rt.timeout_flag = 0;
+    } else {
+        (void)hipGetLastError();  // without the word every report fetches the count from the GPU
+        rt.timeout_flag = nullptr;
+    }
+    rt.timeout_flag_seen = 0;
+    rt.dev.timeout_flag = rt.timeout_flag;
     rt.dev.spin_limit = env_size("NVSHMEM_AMD_SPIN_LIMIT", 1ull << 22);
     rt.dev.options = 0;
     if (const char *order = getenv("NVSHMEM_AMD_PUT_SIGNAL_ORDER")) {
@@ -256,6 +272,8 @@ int nvshmemx_amd_init(int npes, size_t symmetric_size) {
     if (!teams_init(rt)) {
         teams_finalize(rt);
         (void)hipFree(rt.base);
+        if (rt.timeout_flag) (void)hipHostFree(rt.timeout_flag);
+        rt.timeout_flag = nullptr;
         rt.space.reset();
         rt.base = nullptr;
         rt.initialized = false;
@@ -290,6 +308,9 @@ void nvshmem_finalize(void) {
     rt.timeouts_seen = 0;
     teams_finalize(rt);
     (void)hipFree(rt.base);
+    if (rt.timeout_flag) (void)hipHostFree(rt.timeout_flag);
+    rt.timeout_flag = nullptr;
+    rt.timeout_flag_seen = 0;
     rt.space.reset();
     rt.base = nullptr;
     rt.initialized = false;

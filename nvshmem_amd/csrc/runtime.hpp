@@ -72,6 +72,10 @@ struct Runtime {
     unsigned two_step_reduce_members = 16;
     uint64_t two_step_reduce_bytes = (uint64_t)1 << 30;
     uint64_t timeouts_seen = 0;  // bounded waits that gave up, as far as the host has reported them
+    // pinned host word the GPU writes a timeout's number to (null if it could not be allocated), and the value
+    // the host found there at its last report: equal values mean nothing gave up since
+    uint64_t *timeout_flag = nullptr;
+    uint64_t timeout_flag_seen = 0;
 
     static Runtime &get();
 

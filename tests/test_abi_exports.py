@@ -46,7 +46,7 @@ def test_constants_have_the_reference_abi_values():
                     os.path.join(ROOT, "include"), "-o", exe], input=src.encode(), check=True)
     out = subprocess.run([exe], stdout=subprocess.PIPE, check=True).stdout.decode().split()
     assert out[:10] == ["0", "1", "2", "3", "4", "5", "9", "10", "0", "7"]
-    assert int(out[10]) == 104
+    assert int(out[10]) == 112
     # team ids: src/include/device_host/nvshmem_common.cuh:406-419; the config struct is 64 bytes
     # (src/include/device_host/nvshmem_types.h:301)
     assert out[11:] == ["-1", "1", "2", "3", "4", "5", "6", "64"]
