@@ -186,13 +186,19 @@ typedef nvshmemi_v4u __attribute__((aligned(1))) nvshmemi_v4u_unaligned;
 /* Cache policy of the vector body.  Stores stream (non-temporal): a copy never reads its destination
  * back.  Loads stay cacheable for short and medium copies, because callers often push the same source
  * to several PEs (top-k token dispatch, all-push collectives) and the repeats then hit in L2 (measured
- * 1.4x on the MoE dispatch); a single copy of NVSHMEMI_AMD_COPY_NT_BYTES (1 MiB) or more streams its
- * loads too (measured +5 % on a 256 MiB put from 16 blocks per PE and +5.5 % on a 64 MiB one, whose blocks
- * move 4 MiB each; 64 KiB as the threshold gains nothing over 1 MiB).  NVSHMEMI_AMD_COPY_NT overrides the
- * choice for a translation unit: bit 0 set = always non-temporal loads, 0 = never; bit 1 = non-temporal
- * stores. */
+ * 1.4x on the MoE dispatch).  A long copy streams its loads too when the source cannot be expected in the
+ * Infinity Cache: a put of NVSHMEMI_AMD_COPY_NT_BYTES (1 MiB) or more, or a long get, whose size times the
+ * number of thread groups of its scope in the grid - what the grid moves if every group copies as much -
+ * exceeds NVSHMEMI_AMD_COPY_CACHE_BYTES (256 MiB).  Measured on puts from 16 blocks per PE on 8 PEs:
+ * +5 % at 256 MiB and +5.5 % at 64 MiB per PE with streamed loads, but 45 -> 86 us at 16 MiB and
+ * 68 -> 118 us at 32 MiB per PE, sizes whose sources the cache holds from one put to the next.
+ * NVSHMEMI_AMD_COPY_NT overrides the choice for a translation unit: bit 0 set = always non-temporal
+ * loads, 0 = never; bit 1 = non-temporal stores. */
 #ifndef NVSHMEMI_AMD_COPY_NT_BYTES
 #define NVSHMEMI_AMD_COPY_NT_BYTES (1u << 20)
+#endif
+#ifndef NVSHMEMI_AMD_COPY_CACHE_BYTES
+#define NVSHMEMI_AMD_COPY_CACHE_BYTES (256ull << 20)
 #endif
 
 /* A 16-byte store at agent scope (written through the L2).  The compiler has no such store, so it is
@@ -340,10 +346,10 @@ NVSHMEMI_DEVICE_INLINE size_t nvshmemi_amd_copy_deep_rounds(char *__restrict__ d
     return rounds * per_round;
 }
 
-/* How a copy loads its source: by the size of the call (the policy above), or streamed whatever the size.
- * A get streams: its source is another PE's memory, which the caller reads once (the token combine, 2 KiB
- * per call from scattered rows: 5.73 -> 6.02 TB/s), whereas the source of a put is local data that is often
- * sent to several PEs. */
+/* How a copy loads its source: by the size of the call (the policy above), or streamed also when it is
+ * short.  A get streams: its source is another PE's memory, which the caller reads once (the token combine,
+ * 2 KiB per call from scattered rows: 5.73 -> 6.02 TB/s), whereas the source of a put is local data that is
+ * often sent to several PEs.  Long gets follow the policy above like long puts. */
 enum nvshmemi_amd_load_policy_t { NVSHMEMI_AMD_LOAD_BY_SIZE = 0, NVSHMEMI_AMD_LOAD_STREAM = 1 };
 
 template <bool SRC_ALIGNED, int STORE, int LOAD = NVSHMEMI_AMD_LOAD_BY_SIZE, bool BLOCK_WIDE = false>
@@ -379,7 +385,17 @@ NVSHMEMI_DEVICE_INLINE void nvshmemi_memcpy_threadgroup(void *__restrict__ dst_v
 #if defined(NVSHMEMI_AMD_COPY_NT)
     const bool stream_loads = (NVSHMEMI_AMD_COPY_NT & 1) != 0;
 #else
-    const bool stream_loads = LOAD == NVSHMEMI_AMD_LOAD_STREAM || len >= NVSHMEMI_AMD_COPY_NT_BYTES;
+    /* (decided for the deep rounds only - shorter copies of a get stream by their template argument - so
+     * that short copies do not read the launch dimensions) */
+    bool stream_loads = false;
+    if (len / 16 >= (size_t)NVSHMEMI_AMD_COPY_DEEP_MIN * nthr &&
+        (LOAD == NVSHMEMI_AMD_LOAD_STREAM || len >= NVSHMEMI_AMD_COPY_NT_BYTES)) {
+        const uint64_t per_block = SCOPE == NVSHMEMI_THREADGROUP_BLOCK ? 1
+                                   : (uint64_t)blockDim.x * blockDim.y * blockDim.z /
+                                         (SCOPE == NVSHMEMI_THREADGROUP_WARP ? NVSHMEMI_WARP_SIZE : 1);
+        const uint64_t groups = (uint64_t)gridDim.x * gridDim.y * gridDim.z * (per_block ? per_block : 1);
+        stream_loads = len > NVSHMEMI_AMD_COPY_CACHE_BYTES / groups;
+    }
 #endif
 
     size_t head = (size_t)(-(uintptr_t)dst & 15);
