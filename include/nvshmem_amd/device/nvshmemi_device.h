@@ -187,9 +187,10 @@ typedef nvshmemi_v4u __attribute__((aligned(1))) nvshmemi_v4u_unaligned;
  * back.  Loads stay cacheable for short and medium copies, because callers often push the same source
  * to several PEs (top-k token dispatch, all-push collectives) and the repeats then hit in L2 (measured
  * 1.4x on the MoE dispatch).  A long copy streams its loads too when the source cannot be expected in the
- * Infinity Cache: a put of NVSHMEMI_AMD_COPY_NT_BYTES (1 MiB) or more, or a long get, whose size times the
- * number of thread groups of its scope in the grid - what the grid moves if every group copies as much -
- * exceeds NVSHMEMI_AMD_COPY_CACHE_BYTES (256 MiB).  Measured on puts from 16 blocks per PE on 8 PEs:
+ * Infinity Cache: a put of NVSHMEMI_AMD_COPY_NT_BYTES (1 MiB) or more, or a get of NVSHMEMI_AMD_GET_NT_BYTES
+ * (64 KiB) or more, whose size times the number of thread groups of its scope in the grid - what the grid
+ * moves if every group copies as much - exceeds NVSHMEMI_AMD_COPY_CACHE_BYTES (256 MiB).  Shorter gets
+ * always stream.  Measured on puts from 16 blocks per PE on 8 PEs:
  * +5 % at 256 MiB and +5.5 % at 64 MiB per PE with streamed loads, but 45 -> 86 us at 16 MiB and
  * 68 -> 118 us at 32 MiB per PE, sizes whose sources the cache holds from one put to the next.
  * NVSHMEMI_AMD_COPY_NT overrides the choice for a translation unit: bit 0 set = always non-temporal
@@ -199,6 +200,9 @@ typedef nvshmemi_v4u __attribute__((aligned(1))) nvshmemi_v4u_unaligned;
 #endif
 #ifndef NVSHMEMI_AMD_COPY_CACHE_BYTES
 #define NVSHMEMI_AMD_COPY_CACHE_BYTES (256ull << 20)
+#endif
+#ifndef NVSHMEMI_AMD_GET_NT_BYTES /* gets shorter than this stream their loads without looking at the grid */
+#define NVSHMEMI_AMD_GET_NT_BYTES (64u << 10)
 #endif
 
 /* A 16-byte store at agent scope (written through the L2).  The compiler has no such store, so it is
@@ -349,7 +353,7 @@ NVSHMEMI_DEVICE_INLINE size_t nvshmemi_amd_copy_deep_rounds(char *__restrict__ d
 /* How a copy loads its source: by the size of the call (the policy above), or streamed also when it is
  * short.  A get streams: its source is another PE's memory, which the caller reads once (the token combine,
  * 2 KiB per call from scattered rows: 5.73 -> 6.02 TB/s), whereas the source of a put is local data that is
- * often sent to several PEs.  Long gets follow the policy above like long puts. */
+ * often sent to several PEs.  Gets of 64 KiB or more follow the policy above like long puts. */
 enum nvshmemi_amd_load_policy_t { NVSHMEMI_AMD_LOAD_BY_SIZE = 0, NVSHMEMI_AMD_LOAD_STREAM = 1 };
 
 template <bool SRC_ALIGNED, int STORE, int LOAD = NVSHMEMI_AMD_LOAD_BY_SIZE, bool BLOCK_WIDE = false>
@@ -371,8 +375,11 @@ NVSHMEMI_DEVICE_INLINE void nvshmemi_amd_copy_vectors(char *__restrict__ dst,
         nvec -= done;
     }
 #endif
-    nvshmemi_amd_copy_rounds<SRC_ALIGNED, NVSHMEMI_AMD_COPY_NT_ALWAYS || LOAD == NVSHMEMI_AMD_LOAD_STREAM, STORE,
-                             NVSHMEMI_AMD_COPY_UNROLL, true>(dst, src, nvec, tid, nthr);
+    if (LOAD == NVSHMEMI_AMD_LOAD_STREAM && !NVSHMEMI_AMD_COPY_NT_ALWAYS && !stream_loads)
+        nvshmemi_amd_copy_rounds<SRC_ALIGNED, false, STORE, NVSHMEMI_AMD_COPY_UNROLL, true>(dst, src, nvec, tid, nthr);
+    else
+        nvshmemi_amd_copy_rounds<SRC_ALIGNED, NVSHMEMI_AMD_COPY_NT_ALWAYS || LOAD == NVSHMEMI_AMD_LOAD_STREAM, STORE,
+                                 NVSHMEMI_AMD_COPY_UNROLL, true>(dst, src, nvec, tid, nthr);
 }
 
 template <int SCOPE, int STORE = NVSHMEMI_AMD_STORE_STREAM, int LOAD = NVSHMEMI_AMD_LOAD_BY_SIZE>
@@ -385,16 +392,17 @@ NVSHMEMI_DEVICE_INLINE void nvshmemi_memcpy_threadgroup(void *__restrict__ dst_v
 #if defined(NVSHMEMI_AMD_COPY_NT)
     const bool stream_loads = (NVSHMEMI_AMD_COPY_NT & 1) != 0;
 #else
-    /* (decided for the deep rounds only - shorter copies of a get stream by their template argument - so
-     * that short copies do not read the launch dimensions) */
-    bool stream_loads = false;
-    if (len / 16 >= (size_t)NVSHMEMI_AMD_COPY_DEEP_MIN * nthr &&
-        (LOAD == NVSHMEMI_AMD_LOAD_STREAM || len >= NVSHMEMI_AMD_COPY_NT_BYTES)) {
-        const uint64_t per_block = SCOPE == NVSHMEMI_THREADGROUP_BLOCK ? 1
-                                   : (uint64_t)blockDim.x * blockDim.y * blockDim.z /
-                                         (SCOPE == NVSHMEMI_THREADGROUP_WARP ? NVSHMEMI_WARP_SIZE : 1);
-        const uint64_t groups = (uint64_t)gridDim.x * gridDim.y * gridDim.z * (per_block ? per_block : 1);
-        stream_loads = len > NVSHMEMI_AMD_COPY_CACHE_BYTES / groups;
+    /* (short copies decide without reading the launch dimensions: puts keep their loads cacheable, gets
+     * stream) */
+    bool stream_loads = LOAD == NVSHMEMI_AMD_LOAD_STREAM;
+    if (len >= (LOAD == NVSHMEMI_AMD_LOAD_STREAM ? NVSHMEMI_AMD_GET_NT_BYTES : NVSHMEMI_AMD_COPY_NT_BYTES)) {
+        const float per_block = SCOPE == NVSHMEMI_THREADGROUP_BLOCK ? 1.0f
+                                : (float)(blockDim.x * blockDim.y * blockDim.z) /
+                                      (SCOPE == NVSHMEMI_THREADGROUP_WARP ? (float)NVSHMEMI_WARP_SIZE : 1.0f);
+        const float groups = (float)gridDim.x * (float)gridDim.y * (float)gridDim.z * per_block;
+        stream_loads = (float)len * groups > (float)NVSHMEMI_AMD_COPY_CACHE_BYTES;
+    } else if (LOAD == NVSHMEMI_AMD_LOAD_BY_SIZE) {
+        stream_loads = false;
     }
 #endif
 
@@ -413,8 +421,8 @@ NVSHMEMI_DEVICE_INLINE void nvshmemi_memcpy_threadgroup(void *__restrict__ dst_v
         size_t pre = 0;
         if (nvec >= 256) {
             pre = (size_t)((-(uintptr_t)dst >> 4) & 63);
-            if (((uintptr_t)src & 15) == 0) nvshmemi_amd_copy_vectors<true, STORE, LOAD>(dst, src, pre, tid, nthr, false);
-            else nvshmemi_amd_copy_vectors<false, STORE, LOAD>(dst, src, pre, tid, nthr, false);
+            if (((uintptr_t)src & 15) == 0) nvshmemi_amd_copy_vectors<true, STORE, LOAD>(dst, src, pre, tid, nthr, stream_loads);
+            else nvshmemi_amd_copy_vectors<false, STORE, LOAD>(dst, src, pre, tid, nthr, stream_loads);
         }
         constexpr bool block_wide = SCOPE == NVSHMEMI_THREADGROUP_BLOCK;   // every wavefront of the block is here
         if (((uintptr_t)src & 15) == 0)
