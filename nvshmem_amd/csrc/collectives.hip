@@ -92,12 +92,6 @@ enum { kStoreStream = 0 /* nt */, kStoreThrough = 1 /* sc1 */, kStoreThroughStre
 #ifndef NVSHMEM_AMD_STORE_REPLICATE /* fcollect and broadcast, one wavefront storing to every member */
 #define NVSHMEM_AMD_STORE_REPLICATE kStoreThroughStream
 #endif
-#ifndef NVSHMEM_AMD_STORE_REPLICATE_SPLIT /* the same with the members split over neighbouring blocks */
-#define NVSHMEM_AMD_STORE_REPLICATE_SPLIT kStoreStream
-#endif
-#ifndef NVSHMEM_AMD_STORE_WAVE_SPLIT
-#define NVSHMEM_AMD_STORE_WAVE_SPLIT kStoreThroughStream
-#endif
 #ifndef NVSHMEM_AMD_STORE_REDUCE
 #define NVSHMEM_AMD_STORE_REDUCE kStoreThroughStream
 #endif
@@ -140,7 +134,7 @@ __device__ __forceinline__ void copy_tile(char *__restrict__ dst, const char *__
     nvshmemi_v4u v[kCopyUnroll];
 #pragma unroll
     for (int u = 0; u < kCopyUnroll; ++u) {
-        const uint64_t i = v0 + (threadIdx.x & (kCopyThreads - 1)) + (uint64_t)u * kCopyThreads;
+        const uint64_t i = v0 + threadIdx.x + (uint64_t)u * kCopyThreads;
         if (i < nvec) v[u] = SRC_ALIGNED ? stream_load<NTL>(src + 16 * i) : nvshmemi_amd_load16<false>(src + 16 * i);
     }
     if (REPLICATE) {
@@ -148,24 +142,21 @@ __device__ __forceinline__ void copy_tile(char *__restrict__ dst, const char *__
             char *d = dst + (uint64_t)r * rep_stride;
 #pragma unroll
             for (int u = 0; u < kCopyUnroll; ++u) {
-                const uint64_t i = v0 + (threadIdx.x & (kCopyThreads - 1)) + (uint64_t)u * kCopyThreads;
+                const uint64_t i = v0 + threadIdx.x + (uint64_t)u * kCopyThreads;
                 if (i < nvec) stream_store<STORE>(d + 16 * i, v[u]);
             }
         }
     } else {
 #pragma unroll
         for (int u = 0; u < kCopyUnroll; ++u) {
-            const uint64_t i = v0 + (threadIdx.x & (kCopyThreads - 1)) + (uint64_t)u * kCopyThreads;
+            const uint64_t i = v0 + threadIdx.x + (uint64_t)u * kCopyThreads;
             if (i < nvec) stream_store<STORE>(dst + 16 * i, v[u]);
         }
     }
 }
 
-// WAVE_SPLIT: the blocks that share a piece (fcollect / broadcast with part_shift > 0) are the wavefronts of
-// ONE block instead of neighbouring blocks, so the piece crosses the fabric once and the other wavefronts'
-// loads are served by the compute unit's own L1.
-template <int MODE, int kCopyUnroll, bool NTL, int STORE, bool WAVE_SPLIT = false>
-__global__ __launch_bounds__(WAVE_SPLIT ? 1024 : kCopyThreads) void segment_copy_kernel(char *base, uint64_t slice_bytes,
+template <int MODE, int kCopyUnroll, bool NTL, int STORE>
+__global__ __launch_bounds__(kCopyThreads) void segment_copy_kernel(char *base, uint64_t slice_bytes,
                                                                 const nvshmemi_amd_team_view_t *groups,
                                                                 int max_size, uint64_t dst_off,
                                                                 uint64_t src_off, uint64_t seg_bytes,
@@ -204,7 +195,7 @@ __global__ __launch_bounds__(WAVE_SPLIT ? 1024 : kCopyThreads) void segment_copy
     const uint64_t nvec_total = (seg_bytes - head) / 16;
     const uint64_t tail_start = head + nvec_total * 16;
 
-    if (blockIdx.x == 0 && threadIdx.x < kCopyThreads) {
+    if (blockIdx.x == 0) {
         // at most 15 + 15 bytes per replica
         const uint64_t edge = head + (seg_bytes - tail_start);
         for (uint64_t e = threadIdx.x; e < edge * (uint64_t)nrep; e += kCopyThreads) {
@@ -217,14 +208,14 @@ __global__ __launch_bounds__(WAVE_SPLIT ? 1024 : kCopyThreads) void segment_copy
     // lie in front of the segment
     const uint64_t lead = ((uint64_t)(uintptr_t)(dst + head) >> 4) & 63;
     constexpr uint64_t kTileVectors = (uint64_t)kCopyThreads * kCopyUnroll;
-    // fcollect / broadcast: 2^part_shift consecutive blocks share a tile and split its destinations
-    // With chunk_shift > 0 the sharers of a tile are 2^chunk_shift blocks apart instead of neighbours: the grid walks a
-    // chunk of 2^chunk_shift tiles once per group of destinations, so the blocks in flight write to few destinations
-    // at a time, each a run of consecutive pieces, and re-read the chunk from the L2 of the XCD that fetched it
-    // (sharers are a multiple of 8 blocks apart).
-    uint64_t tile_index = WAVE_SPLIT ? blockIdx.x : blockIdx.x >> part_shift;
-    unsigned part_index = WAVE_SPLIT ? threadIdx.x / kCopyThreads : blockIdx.x & ((1u << part_shift) - 1);
-    if (!WAVE_SPLIT && chunk_shift) {
+    // fcollect / broadcast with part_shift > 0: 2^part_shift blocks share a tile and split its destinations.  The
+    // sharers of a tile are 2^chunk_shift blocks apart: the grid walks a chunk of 2^chunk_shift tiles once per
+    // group of destinations, so the blocks in flight write to few destinations at a time, each a run of
+    // consecutive pieces, and re-read the chunk from the L2 of the XCD that fetched it (sharers are a multiple of
+    // 8 blocks apart).  The host passes both shifts as zero or both as non-zero.
+    uint64_t tile_index = blockIdx.x;
+    unsigned part_index = 0;
+    if (chunk_shift) {
         part_index = (blockIdx.x >> chunk_shift) & ((1u << part_shift) - 1);
         tile_index = (blockIdx.x & ((1u << chunk_shift) - 1)) +
                      (((uint64_t)blockIdx.x >> (chunk_shift + part_shift)) << chunk_shift);
@@ -522,32 +513,12 @@ __global__ __launch_bounds__(kThreads) void reduce_scalar_kernel(char *base, uin
     }
 }
 
-// fcollect / broadcast of sources too large to stay in the Infinity Cache split the destinations of a piece
-// over several wavefronts.  Earlier forms, kept selectable (NVSHMEM_AMD_*_SPLIT 1 and 2): at most four
-// destinations per wavefront, the sharers being neighbouring blocks (they run on different XCDs, so the piece
-// is fetched once per sharer from the Infinity Cache) or the wavefronts of one block: broadcast of 512 MiB to
-// 8 PEs 5.05 -> 6.03 TB/s, fcollect of 16 x 32 MiB 5.25 -> 5.85.  The default is the chunked form below.
-// Cache-resident sources keep one wavefront per piece: a split costs them up to 9 %.
-#ifndef NVSHMEM_AMD_REPLICAS_PER_WAVE
-#define NVSHMEM_AMD_REPLICAS_PER_WAVE 4
-#endif
-#ifndef NVSHMEM_AMD_FCOLLECT_SPLIT /* 0: one wavefront stores to all members; 1: neighbouring blocks share; 2: the wavefronts of one block; 3: chunked */
-#define NVSHMEM_AMD_FCOLLECT_SPLIT 3
-#endif
-#ifndef NVSHMEM_AMD_BROADCAST_SPLIT /* 0, 1 or 3, as above */
-#define NVSHMEM_AMD_BROADCAST_SPLIT 3
-#endif
 #ifndef NVSHMEM_AMD_STORE_FCOLLECT_CHUNKED
 #define NVSHMEM_AMD_STORE_FCOLLECT_CHUNKED kStoreThroughStream /* +2 % over nt */
 #endif
 #ifndef NVSHMEM_AMD_STORE_BROADCAST_CHUNKED
 #define NVSHMEM_AMD_STORE_BROADCAST_CHUNKED kStoreStream /* +2.5 % over sc1 nt */
 #endif
-static uint32_t replica_part_shift(int max_size, int per_wave = NVSHMEM_AMD_REPLICAS_PER_WAVE) {
-    uint32_t shift = 0;
-    while (((max_size + (1 << shift) - 1) >> shift) > per_wave) ++shift;
-    return shift;
-}
 
 // Chunked sharing, the form fcollect and broadcast of sources beyond the Infinity Cache take: a wavefront stores
 // its piece to two destinations, and the grid walks a chunk of tiles once per pair of destinations before it moves
@@ -558,6 +529,9 @@ static uint32_t replica_part_shift(int max_size, int per_wave = NVSHMEM_AMD_REPL
 // 32 MiB fcollect / 512 MiB broadcast to 8): fcollect 5.85 -> 6.30 TB/s, broadcast 6.07 -> 6.48; the chunk that
 // measured best makes chunk x groups = 16384 blocks, twice what the GPU holds at a time (fcollect: 2^11 tiles x
 // 8 pairs; broadcast: 2^12 x 4; half or double that chunk loses 1-12 %), one destination per wavefront 20 %.
+// Forms with at most four destinations per wavefront whose sharers are neighbouring blocks, or the wavefronts of
+// one block, measured 5.85 / 6.03 TB/s on the same two workloads.  Cache-resident sources keep one wavefront per
+// piece storing to every member: a split costs them up to 9 %.
 #ifndef NVSHMEM_AMD_CHUNKED_REPLICAS_PER_WAVE
 #define NVSHMEM_AMD_CHUNKED_REPLICAS_PER_WAVE 2
 #endif
@@ -586,12 +560,11 @@ static uint64_t total_members(const TeamLaunch &tl) {
 // Launches the broadcast kernel: member `root`'s [soff, +bytes) to every member's [doff, +bytes).
 static int launch_broadcast(Runtime &rt, const TeamLaunch &tl, uint64_t doff, uint64_t soff, uint64_t bytes, int root,
                             hipStream_t stream, bool force_chunked = false) {
-    // a source that cannot stay in the Infinity Cache: split the destinations (see replica_part_shift)
+    // a source that cannot stay in the Infinity Cache: the chunked form (teams of fewer than four members have
+    // one group of destinations and keep the plain form)
     const bool big_source = force_chunked || bytes * (uint64_t)tl.ngroups > rt.cacheable_source_bytes;
-    const bool chunked = big_source && NVSHMEM_AMD_BROADCAST_SPLIT == 3;
-    const uint32_t part_shift = chunked ? chunked_part_shift(tl.max_size)
-                                : big_source && NVSHMEM_AMD_BROADCAST_SPLIT ? replica_part_shift(tl.max_size) : 0;
-    const uint32_t chunk_shift = chunked && part_shift ? chunk_shift_for(part_shift) : 0;
+    const uint32_t part_shift = big_source ? chunked_part_shift(tl.max_size) : 0;
+    const uint32_t chunk_shift = part_shift ? chunk_shift_for(part_shift) : 0;
     uint64_t tiles = (bytes / 16 + 64 + kCopyThreads - 1) / kCopyThreads + 1;
     tiles = ((tiles + (1ull << chunk_shift) - 1) >> chunk_shift << chunk_shift) << part_shift;  // whole chunks
     if (tiles > 0x7fffffffull) {
@@ -605,7 +578,6 @@ static int launch_broadcast(Runtime &rt, const TeamLaunch &tl, uint64_t doff, ui
                        rt.base, rt.heap_size, tl.groups, tl.max_size, doff, soff, (uint64_t)bytes, root, \
                        part_shift, chunk_shift)
     if (chunk_shift != 0) NVSHMEM_AMD_LAUNCH_BROADCAST(false, NVSHMEM_AMD_STORE_BROADCAST_CHUNKED);
-    else if (part_shift != 0) NVSHMEM_AMD_LAUNCH_BROADCAST(false, NVSHMEM_AMD_STORE_REPLICATE_SPLIT);
     else if (big_source) NVSHMEM_AMD_LAUNCH_BROADCAST(true, NVSHMEM_AMD_STORE_REPLICATE);
     else NVSHMEM_AMD_LAUNCH_BROADCAST(false, NVSHMEM_AMD_STORE_REPLICATE);
 #undef NVSHMEM_AMD_LAUNCH_BROADCAST
@@ -949,15 +921,11 @@ static int segment_collective(int mode, const char *what, nvshmem_team_t team, v
     const uint64_t tile_vectors = (uint64_t)kCopyThreads * (mode == kModeFcollect ? NVSHMEM_AMD_FCOLLECT_UNROLL
                                                                               : NVSHMEM_AMD_ALLTOALL_UNROLL);
     const bool big_source = src_bytes * total_members(tl) > rt.cacheable_source_bytes;
-    const bool chunked = mode == kModeFcollect && big_source && NVSHMEM_AMD_FCOLLECT_SPLIT == 3;
-    const uint32_t part_shift =
-        chunked ? chunked_part_shift(tl.max_size)
-        : mode == kModeFcollect && big_source && NVSHMEM_AMD_FCOLLECT_SPLIT ? replica_part_shift(tl.max_size) : 0;
-    const uint32_t chunk_shift = chunked && part_shift ? chunk_shift_for(part_shift) : 0;
-    // (NVSHMEM_AMD_FCOLLECT_SPLIT 2: the wavefronts of one block share the piece)
-    const bool wave_split = part_shift != 0 && NVSHMEM_AMD_FCOLLECT_SPLIT == 2 && (kCopyThreads << part_shift) <= 1024;
+    // an fcollect whose sources cannot stay in the Infinity Cache takes the chunked form
+    const uint32_t part_shift = mode == kModeFcollect && big_source ? chunked_part_shift(tl.max_size) : 0;
+    const uint32_t chunk_shift = part_shift ? chunk_shift_for(part_shift) : 0;
     uint64_t tiles = (seg_bytes / 16 + 64 + tile_vectors - 1) / tile_vectors + 1;
-    tiles = ((tiles + (1ull << chunk_shift) - 1) >> chunk_shift << chunk_shift) << (wave_split ? 0 : part_shift);  // whole chunks
+    tiles = ((tiles + (1ull << chunk_shift) - 1) >> chunk_shift << chunk_shift) << part_shift;  // whole chunks
     const unsigned segs = mode == kModeFcollect ? (unsigned)n : (unsigned)(n * n);
     if (tiles > 0x7fffffffull) {
         set_error("%s: message too large", what);
@@ -965,20 +933,14 @@ static int segment_collective(int mode, const char *what, nvshmem_team_t team, v
     }
     // blocks that share a piece re-read it from the cache, so the loads stay cacheable then
     const bool stream_source = part_shift == 0 && big_source;
-    const dim3 grid((unsigned)tiles, segs, (unsigned)tl.ngroups), block(wave_split ? kCopyThreads << part_shift : kCopyThreads);
+    const dim3 grid((unsigned)tiles, segs, (unsigned)tl.ngroups), block(kCopyThreads);
 #define NVSHMEM_AMD_LAUNCH_SEGCOPY(MODE, U, NTL, STORE)                                            \
     hipLaunchKernelGGL((segment_copy_kernel<MODE, U, NTL, STORE>), grid, block, 0, stream, rt.base, \
                        rt.heap_size, tl.groups, tl.max_size, doff, soff, (uint64_t)seg_bytes, 0,   \
                        part_shift, chunk_shift)
     if (mode == kModeFcollect) {
-        if (wave_split)
-            hipLaunchKernelGGL((segment_copy_kernel<kModeFcollect, NVSHMEM_AMD_FCOLLECT_UNROLL, true, NVSHMEM_AMD_STORE_WAVE_SPLIT, true>),
-                               grid, block, 0, stream, rt.base, rt.heap_size, tl.groups, tl.max_size, doff, soff,
-                               (uint64_t)seg_bytes, 0, part_shift, chunk_shift);
-        else if (chunk_shift != 0)
+        if (chunk_shift != 0)
             NVSHMEM_AMD_LAUNCH_SEGCOPY(kModeFcollect, NVSHMEM_AMD_FCOLLECT_UNROLL, false, NVSHMEM_AMD_STORE_FCOLLECT_CHUNKED);
-        else if (part_shift != 0)
-            NVSHMEM_AMD_LAUNCH_SEGCOPY(kModeFcollect, NVSHMEM_AMD_FCOLLECT_UNROLL, false, NVSHMEM_AMD_STORE_REPLICATE_SPLIT);
         else if (stream_source)
             NVSHMEM_AMD_LAUNCH_SEGCOPY(kModeFcollect, NVSHMEM_AMD_FCOLLECT_UNROLL, true, NVSHMEM_AMD_STORE_REPLICATE);
         else
