@@ -594,15 +594,18 @@ void launch_reduce(Runtime &rt, const TeamLaunch &tl, uint64_t dst_off, uint64_t
                    uint64_t nelems, hipStream_t stream) {
     const bool vector_ok = ((dst_off | src_off) & 15) == 0;
     const unsigned ngroups = (unsigned)tl.ngroups;
-    // Which vector kernel.  Once the sources no longer fit the Infinity Cache - more than
-    // Runtime::lds_reduce_bytes (256 MiB, counted as 4-byte elements) in all - the LDS-staged kernel wins
-    // for every team of 3 to 64 members; below that, and for 2 members, the gather kernel does.
-    // Measured with random fp32 data and write-through stores, LDS-staged against gather, TB/s at
+    // Which vector kernel.  From Runtime::lds_reduce_bytes of sources in all (64 MiB, counted as 4-byte
+    // elements; a quarter of that for teams of 17 to 32 members, four times for larger ones) the LDS-staged
+    // kernel wins for every team of 3 to 64 members; below that, and for 2 members, the gather kernel does.
+    // fp32 sum on a stream, LDS-staged / gather in TB/s, sources of 32 MiB | 64 MiB | 128 MiB in all: 4 members
+    // 7.3 / 8.4 | 7.6 / 7.4 | 8.3 / 8.1, 8 members 7.8 / 8.3 | 7.8 / 6.9 | 8.5 / 7.7, 16 members 7.0 / 8.3 |
+    // 7.6 / 6.6 | 8.3 / 7.6; 32 members lead with the LDS kernel from 16 MiB on (7.3 / 5.3), 48 and 64 members
+    // with the gather kernel up to 128-192 MiB (5.9 / 6.8).  Beyond the cache,
+    // measured with random fp32 data and write-through stores, LDS-staged against gather, TB/s at
     // 512 MiB / 2 GiB of sources: 4 members 6.54 / 6.55 against 6.19 / 6.24, 6 members 6.37 / 6.44
     // against 5.89 / 5.58, 8 members 6.46 / 6.53 against 6.03 / 6.09, 12 members 6.28 / 6.28 against
     // 5.73 / 5.83, 16 members 6.21 / 6.12 against 5.44 / 5.57, 32 members 6.17 / 6.10 against 5.22 / 5.49,
-    // 64 members 5.64 / 5.64 against 5.15 / 5.26; at 128 MiB the two are level, at 32 MiB the gather
-    // kernel leads by up to 20 % for up to 16 members.  A wavefront of the LDS kernel serves one member
+    // 64 members 5.64 / 5.64 against 5.15 / 5.26.  A wavefront of the LDS kernel serves one member
     // for the compile-time sizes 8 and 16, two members up to 32 and four beyond: one load and one store
     // per lane measured best where the block stays within 16 wavefronts, and wavefronts of fewer than
     // 64 lanes per member (512- or 256-byte accesses) lost 7-22 % against the gather kernel.  The
@@ -610,6 +613,9 @@ void launch_reduce(Runtime &rt, const TeamLaunch &tl, uint64_t dst_off, uint64_t
     const uint64_t total_bytes = total_members(tl) * nelems * sizeof(T);
     const int fixed_size = tl.min_size == tl.max_size ? tl.max_size : 0;
     const bool stream_source = total_bytes > rt.cacheable_source_bytes;
+    const uint64_t lds_from_elements = (tl.max_size > 32   ? rt.lds_reduce_bytes * 4
+                                        : tl.max_size > 16 ? rt.lds_reduce_bytes / 4
+                                                           : rt.lds_reduce_bytes) / 4;
     // The threshold counts elements (as 4-byte ones): narrow types fold more elements per byte.
     // mpw: members per wavefront of the LDS-staged kernel; ct_size: a compile-time team size, if any
     int mpw = 0, ct_size = 0;
@@ -628,7 +634,7 @@ void launch_reduce(Runtime &rt, const TeamLaunch &tl, uint64_t dst_off, uint64_t
     // and from three times that many members whatever the size.
     if (vector_ok && rt.two_step_reduce_members && tl.min_size >= (int)rt.two_step_reduce_members &&
         (total_bytes >= rt.two_step_reduce_bytes || tl.min_size >= 3 * (int)rt.two_step_reduce_members) &&
-        total_members(tl) * nelems > rt.lds_reduce_bytes / 4) {
+        total_members(tl) * nelems >= lds_from_elements) {
         const uint64_t nvec = nelems / (16 / sizeof(T));
         uint64_t blocks = (nvec + 63 + 63) / 64;
         if (blocks <= 0x7fffffffull) {
@@ -643,7 +649,7 @@ void launch_reduce(Runtime &rt, const TeamLaunch &tl, uint64_t dst_off, uint64_t
             return;
         }
     }
-    if (vector_ok && mpw && total_members(tl) * nelems > rt.lds_reduce_bytes / 4) {
+    if (vector_ok && mpw && total_members(tl) * nelems >= lds_from_elements) {
         const uint32_t lane_shift = 6;
         const unsigned threads = (unsigned)((tl.max_size + mpw - 1) / mpw) << lane_shift;
         const uint64_t nvec = nelems / (16 / sizeof(T));

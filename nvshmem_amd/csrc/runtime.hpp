@@ -61,10 +61,10 @@ struct Runtime {
     // Host-launched collectives treat sources of more bytes than this (all PEs together) as too
     // large to stay in the Infinity Cache: NVSHMEM_AMD_CACHEABLE_SOURCE_BYTES, read at init
     uint64_t cacheable_source_bytes = (uint64_t)256 << 20;
-    // Allreduce on teams of exactly 8 or 16 members takes the LDS-staged kernel when the sources of
-    // all PEs together hold more than this many bytes' worth of 4-byte elements:
-    // NVSHMEM_AMD_LDS_REDUCE_BYTES, read at init
-    uint64_t lds_reduce_bytes = (uint64_t)256 << 20;
+    // Allreduce on teams of 3 to 64 members takes the LDS-staged kernel when the sources of all PEs
+    // together hold at least this many bytes' worth of 4-byte elements (a quarter of it for teams of 17
+    // to 32 members, four times for larger ones): NVSHMEM_AMD_LDS_REDUCE_BYTES, read at init
+    uint64_t lds_reduce_bytes = (uint64_t)64 << 20;
     // An allreduce beyond the cache takes two steps - fold into member 0, chunked broadcast - instead of the fused
     // kernel from this team size on (NVSHMEM_AMD_TWO_STEP_REDUCE_MEMBERS, read at init; 0 = never) when the
     // sources of all members together hold at least two_step_reduce_bytes (NVSHMEM_AMD_TWO_STEP_REDUCE_BYTES), and
