@@ -560,10 +560,12 @@ static uint64_t total_members(const TeamLaunch &tl) {
 // Launches the broadcast kernel: member `root`'s [soff, +bytes) to every member's [doff, +bytes).
 static int launch_broadcast(Runtime &rt, const TeamLaunch &tl, uint64_t doff, uint64_t soff, uint64_t bytes, int root,
                             hipStream_t stream, bool force_chunked = false) {
-    // a source that cannot stay in the Infinity Cache: the chunked form (teams of fewer than four members have
-    // one group of destinations and keep the plain form)
-    const bool big_source = force_chunked || bytes * (uint64_t)tl.ngroups > rt.cacheable_source_bytes;
-    const uint32_t part_shift = big_source ? chunked_part_shift(tl.max_size) : 0;
+    // The chunked form from Runtime::chunked_copy_bytes (128 MiB) on: measured level with the plain form at
+    // 64 MiB and 3-5 % ahead from 128 MiB for 4 and 8 members (teams of fewer than four members have one group
+    // of destinations and keep the plain form).  A source that cannot stay in the Infinity Cache is streamed.
+    const bool big_source = bytes * (uint64_t)tl.ngroups > rt.cacheable_source_bytes;
+    const bool chunked = force_chunked || bytes * (uint64_t)tl.ngroups >= rt.chunked_copy_bytes;
+    const uint32_t part_shift = chunked ? chunked_part_shift(tl.max_size) : 0;
     const uint32_t chunk_shift = part_shift ? chunk_shift_for(part_shift) : 0;
     uint64_t tiles = (bytes / 16 + 64 + kCopyThreads - 1) / kCopyThreads + 1;
     tiles = ((tiles + (1ull << chunk_shift) - 1) >> chunk_shift << chunk_shift) << part_shift;  // whole chunks
@@ -927,8 +929,14 @@ static int segment_collective(int mode, const char *what, nvshmem_team_t team, v
     const uint64_t tile_vectors = (uint64_t)kCopyThreads * (mode == kModeFcollect ? NVSHMEM_AMD_FCOLLECT_UNROLL
                                                                               : NVSHMEM_AMD_ALLTOALL_UNROLL);
     const bool big_source = src_bytes * total_members(tl) > rt.cacheable_source_bytes;
-    // an fcollect whose sources cannot stay in the Infinity Cache takes the chunked form
-    const uint32_t part_shift = mode == kModeFcollect && big_source ? chunked_part_shift(tl.max_size) : 0;
+    // An fcollect takes the chunked form when its sources hold Runtime::chunked_copy_bytes (128 MiB) or more and
+    // its destinations eight times that: with the sources still in the Infinity Cache it is the n-fold larger
+    // destinations that decide.  Chunked / plain in TB/s at 64 | 128 | 256 MiB of sources: 16 members 6.3 / 6.5 |
+    // 7.2 / 6.6 | 7.7 / 6.5, 8 members 6.4 / 6.9 | 7.3 / 6.9 | 7.9 / 6.9, 4 members 6.7 / 7.7 | 7.7 / 8.0 | 8.4 / 8.1.
+    const uint64_t all_sources = src_bytes * total_members(tl);
+    const bool chunked = mode == kModeFcollect && all_sources >= rt.chunked_copy_bytes &&
+                         all_sources * n >= 8 * rt.chunked_copy_bytes;
+    const uint32_t part_shift = chunked ? chunked_part_shift(tl.max_size) : 0;
     const uint32_t chunk_shift = part_shift ? chunk_shift_for(part_shift) : 0;
     uint64_t tiles = (seg_bytes / 16 + 64 + tile_vectors - 1) / tile_vectors + 1;
     tiles = ((tiles + (1ull << chunk_shift) - 1) >> chunk_shift << chunk_shift) << part_shift;  // whole chunks

@@ -266,6 +266,7 @@ int nvshmemx_amd_init(int npes, size_t symmetric_size) {
     rt.dev.heap_magic = (1ull << 40) / (rt.heap_size >> 21) + 1;
     rt.plain_collective_launch = env_size("NVSHMEM_AMD_PLAIN_COLLECTIVE_LAUNCH", 0) != 0;
     rt.cacheable_source_bytes = env_size("NVSHMEM_AMD_CACHEABLE_SOURCE_BYTES", (size_t)256 << 20);
+    rt.chunked_copy_bytes = env_size("NVSHMEM_AMD_CHUNKED_COPY_BYTES", (size_t)128 << 20);
     rt.lds_reduce_bytes = env_size("NVSHMEM_AMD_LDS_REDUCE_BYTES", (size_t)64 << 20);
     rt.two_step_reduce_members = (unsigned)env_size("NVSHMEM_AMD_TWO_STEP_REDUCE_MEMBERS", 16);
     rt.two_step_reduce_bytes = env_size("NVSHMEM_AMD_TWO_STEP_REDUCE_BYTES", (size_t)1 << 30);

@@ -61,6 +61,9 @@ struct Runtime {
     // Host-launched collectives treat sources of more bytes than this (all PEs together) as too
     // large to stay in the Infinity Cache: NVSHMEM_AMD_CACHEABLE_SOURCE_BYTES, read at init
     uint64_t cacheable_source_bytes = (uint64_t)256 << 20;
+    // fcollect and broadcast take the chunked form from this many bytes of sources (all PEs together) on:
+    // NVSHMEM_AMD_CHUNKED_COPY_BYTES, read at init
+    uint64_t chunked_copy_bytes = (uint64_t)128 << 20;
     // Allreduce on teams of 3 to 64 members takes the LDS-staged kernel when the sources of all PEs
     // together hold at least this many bytes' worth of 4-byte elements (a quarter of it for teams of 17
     // to 32 members, four times for larger ones): NVSHMEM_AMD_LDS_REDUCE_BYTES, read at init

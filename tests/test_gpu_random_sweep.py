@@ -3,7 +3,8 @@ element types, operators, counts and byte offsets, each compared with the CPU or
 (integers, copies) or bit for bit with the fixed PE order (floating point).  The cases are drawn from
 a fixed seed, so a failure names a reproducible case.  NVSHMEM_AMD_TEST_SEED_OFFSET shifts the seeds for a longer
 run over other cases; the kernel-selection thresholds can be lowered from the environment as for any program
-(NVSHMEM_AMD_LDS_REDUCE_BYTES=0 NVSHMEM_AMD_CACHEABLE_SOURCE_BYTES=0 sends these small messages through the
+(NVSHMEM_AMD_LDS_REDUCE_BYTES=0 NVSHMEM_AMD_CACHEABLE_SOURCE_BYTES=0 NVSHMEM_AMD_CHUNKED_COPY_BYTES=0 sends these
+small messages through the
 kernels meant for large ones)."""
 import os
 

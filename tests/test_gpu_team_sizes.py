@@ -182,11 +182,13 @@ def test_small_in_kernel_collectives_with_and_without_packets(disable, plain, mo
 
 @pytest.mark.parametrize("npes", [3, 8, 13, 16, 33, 64])
 def test_large_source_policy_of_fcollect_and_broadcast(npes, monkeypatch):
-    """Sources beyond NVSHMEM_AMD_CACHEABLE_SOURCE_BYTES (read at init) are streamed, and fcollect /
-    broadcast then split the destinations of a piece over several wavefronts (two per wavefront, the
-    grid walking a chunk of the message once per pair).  With the threshold at zero every size takes that path: ragged, misaligned messages
-    must come out the same, bytes outside the destination untouched."""
+    """Sources beyond NVSHMEM_AMD_CACHEABLE_SOURCE_BYTES (read at init) are streamed, and from
+    NVSHMEM_AMD_CHUNKED_COPY_BYTES on fcollect / broadcast split the destinations of a piece over several
+    wavefronts (two per wavefront, the grid walking a chunk of the message once per pair).  With the
+    thresholds at zero every size takes that path: ragged, misaligned messages must come out the same, bytes
+    outside the destination untouched."""
     monkeypatch.setenv("NVSHMEM_AMD_CACHEABLE_SOURCE_BYTES", "0")
+    monkeypatch.setenv("NVSHMEM_AMD_CHUNKED_COPY_BYTES", "0")
     monkeypatch.setenv("NVSHMEM_AMD_LDS_REDUCE_BYTES", "0")      # 8 and 16 members: the LDS-staged allreduce
     rng = np.random.default_rng(100 + npes)
     with runtime(npes, 1 << 24) as rt:
@@ -231,6 +233,7 @@ def test_large_source_fcollect_and_broadcast_across_several_chunks(npes, monkeyp
     group of destinations: a message of several chunks plus a ragged rest, misaligned at both ends, must
     arrive whole on every member, with the bytes around the destination untouched."""
     monkeypatch.setenv("NVSHMEM_AMD_CACHEABLE_SOURCE_BYTES", "0")
+    monkeypatch.setenv("NVSHMEM_AMD_CHUNKED_COPY_BYTES", "0")
     rng = np.random.default_rng(4100 + npes)
     nbytes = (9 << 20) + 1234
     with runtime(npes, (npes + 1) * (10 << 20) + (8 << 20)) as rt:
@@ -275,6 +278,7 @@ def test_two_step_allreduce(npes, monkeypatch):
     NaN-carrying max, bf16, int64, families of ragged teams - must come out bit for bit the same."""
     monkeypatch.setenv("NVSHMEM_AMD_LDS_REDUCE_BYTES", "0")
     monkeypatch.setenv("NVSHMEM_AMD_CACHEABLE_SOURCE_BYTES", "0")
+    monkeypatch.setenv("NVSHMEM_AMD_CHUNKED_COPY_BYTES", "0")
     monkeypatch.setenv("NVSHMEM_AMD_TWO_STEP_REDUCE_MEMBERS", "2")
     monkeypatch.setenv("NVSHMEM_AMD_TWO_STEP_REDUCE_BYTES", "0")
     _allreduce_battery(npes, np.random.default_rng(7100 + npes), "two-step")
