@@ -596,8 +596,8 @@ void launch_reduce(Runtime &rt, const TeamLaunch &tl, uint64_t dst_off, uint64_t
                    uint64_t nelems, hipStream_t stream) {
     const bool vector_ok = ((dst_off | src_off) & 15) == 0;
     const unsigned ngroups = (unsigned)tl.ngroups;
-    // Which vector kernel.  From Runtime::lds_reduce_bytes of sources in all (64 MiB, counted as 4-byte
-    // elements; a quarter of that for teams of 17 to 32 members, four times for larger ones) the LDS-staged
+    // Which vector kernel.  From Runtime::lds_reduce_bytes of sources in all (64 MiB; a quarter
+    // of that for teams of 17 to 32 members, four times for larger ones) the LDS-staged
     // kernel wins for every team of 3 to 64 members; below that, and for 2 members, the gather kernel does.
     // fp32 sum on a stream, LDS-staged / gather in TB/s, sources of 32 MiB | 64 MiB | 128 MiB in all: 4 members
     // 7.3 / 8.4 | 7.6 / 7.4 | 8.3 / 8.1, 8 members 7.8 / 8.3 | 7.8 / 6.9 | 8.5 / 7.7, 16 members 7.0 / 8.3 |
@@ -615,10 +615,10 @@ void launch_reduce(Runtime &rt, const TeamLaunch &tl, uint64_t dst_off, uint64_t
     const uint64_t total_bytes = total_members(tl) * nelems * sizeof(T);
     const int fixed_size = tl.min_size == tl.max_size ? tl.max_size : 0;
     const bool stream_source = total_bytes > rt.cacheable_source_bytes;
-    const uint64_t lds_from_elements = (tl.max_size > 32   ? rt.lds_reduce_bytes * 4
-                                        : tl.max_size > 16 ? rt.lds_reduce_bytes / 4
-                                                           : rt.lds_reduce_bytes) / 4;
-    // The threshold counts elements (as 4-byte ones): narrow types fold more elements per byte.
+    // (in bytes whatever the element type: fp32, bf16 and int64 cross over at the same 64 MiB on 8 and 16 members)
+    const uint64_t lds_from_bytes = tl.max_size > 32   ? rt.lds_reduce_bytes * 4
+                                    : tl.max_size > 16 ? rt.lds_reduce_bytes / 4
+                                                       : rt.lds_reduce_bytes;
     // mpw: members per wavefront of the LDS-staged kernel; ct_size: a compile-time team size, if any
     int mpw = 0, ct_size = 0;
     constexpr int kNarrowMpw = sizeof(T) <= 2 ? NVSHMEM_AMD_REDUCE_NARROW_MPW : NVSHMEM_AMD_REDUCE_WIDE_MPW;
@@ -632,11 +632,11 @@ void launch_reduce(Runtime &rt, const TeamLaunch &tl, uint64_t dst_off, uint64_t
     // serialises n steps between two barriers.  fp32 sum, TB/s, fused / two-step at 512 MiB and 2 GiB of sources in
     // all: 12 members 6.41 / 6.18 and 6.28 / 6.29, 16: 6.26 / 6.19 and 6.02 / 6.41, 24: 5.84 / 5.71 and 5.69 / 6.23,
     // 32: 6.09 / 6.09 and 6.09 / 6.51, 48: 5.68 / 5.78 and 5.57 / 6.25, 64: 5.55 / 5.97 and 5.59 / 6.56.  So: from
-    // Runtime::two_step_reduce_members (16) members on when the sources hold two_step_reduce_bytes (1 GiB) or more,
+    // Runtime::two_step_reduce_members (16) members on when the sources hold two_step_reduce_bytes (512 MiB: 16 members 6.2 against 6.0 TB/s fused there, 32 members 6.3 against 5.8) or more,
     // and from three times that many members whatever the size.
     if (vector_ok && rt.two_step_reduce_members && tl.min_size >= (int)rt.two_step_reduce_members &&
         (total_bytes >= rt.two_step_reduce_bytes || tl.min_size >= 3 * (int)rt.two_step_reduce_members) &&
-        total_members(tl) * nelems >= lds_from_elements) {
+        total_bytes >= lds_from_bytes) {
         const uint64_t nvec = nelems / (16 / sizeof(T));
         uint64_t blocks = (nvec + 63 + 63) / 64;
         if (blocks <= 0x7fffffffull) {
@@ -651,7 +651,7 @@ void launch_reduce(Runtime &rt, const TeamLaunch &tl, uint64_t dst_off, uint64_t
             return;
         }
     }
-    if (vector_ok && mpw && total_members(tl) * nelems >= lds_from_elements) {
+    if (vector_ok && mpw && total_bytes >= lds_from_bytes) {
         const uint32_t lane_shift = 6;
         const unsigned threads = (unsigned)((tl.max_size + mpw - 1) / mpw) << lane_shift;
         const uint64_t nvec = nelems / (16 / sizeof(T));

@@ -269,7 +269,7 @@ int nvshmemx_amd_init(int npes, size_t symmetric_size) {
     rt.chunked_copy_bytes = env_size("NVSHMEM_AMD_CHUNKED_COPY_BYTES", (size_t)128 << 20);
     rt.lds_reduce_bytes = env_size("NVSHMEM_AMD_LDS_REDUCE_BYTES", (size_t)64 << 20);
     rt.two_step_reduce_members = (unsigned)env_size("NVSHMEM_AMD_TWO_STEP_REDUCE_MEMBERS", 16);
-    rt.two_step_reduce_bytes = env_size("NVSHMEM_AMD_TWO_STEP_REDUCE_BYTES", (size_t)1 << 30);
+    rt.two_step_reduce_bytes = env_size("NVSHMEM_AMD_TWO_STEP_REDUCE_BYTES", (size_t)512 << 20);
     if (!teams_init(rt)) {
         teams_finalize(rt);
         (void)hipFree(rt.base);

@@ -65,7 +65,7 @@ struct Runtime {
     // NVSHMEM_AMD_CHUNKED_COPY_BYTES, read at init
     uint64_t chunked_copy_bytes = (uint64_t)128 << 20;
     // Allreduce on teams of 3 to 64 members takes the LDS-staged kernel when the sources of all PEs
-    // together hold at least this many bytes' worth of 4-byte elements (a quarter of it for teams of 17
+    // together hold at least this many bytes (a quarter of it for teams of 17
     // to 32 members, four times for larger ones): NVSHMEM_AMD_LDS_REDUCE_BYTES, read at init
     uint64_t lds_reduce_bytes = (uint64_t)64 << 20;
     // An allreduce beyond the cache takes two steps - fold into member 0, chunked broadcast - instead of the fused
@@ -73,7 +73,7 @@ struct Runtime {
     // sources of all members together hold at least two_step_reduce_bytes (NVSHMEM_AMD_TWO_STEP_REDUCE_BYTES), and
     // from three times the team size at any size
     unsigned two_step_reduce_members = 16;
-    uint64_t two_step_reduce_bytes = (uint64_t)1 << 30;
+    uint64_t two_step_reduce_bytes = (uint64_t)512 << 20;
     uint64_t timeouts_seen = 0;  // bounded waits that gave up, as far as the host has reported them
     // pinned host word the GPU writes a timeout's number to (null if it could not be allocated), and the value
     // the host found there at its last report: equal values mean nothing gave up since
