@@ -32,6 +32,13 @@ def test_driver_table_rows():
     assert perftest_tables.rows_of(text) == [(8, 0.002), (268435456, 382.40)]
 
 
+def test_collective_table_rows_are_the_bandwidth_table_only():
+    text = ("#reduction_on_stream\nsize(B)     scope     latency (us)\n1024        stream    3.24\n"
+            "#reduction_on_stream\nsize(B)     scope     algorithmic BW (GB/s)\n1024        stream    5.05\n"
+            "2048        stream    11.2\n")
+    assert perftest_tables.bandwidth_rows(text) == [(1024, 5.05), (2048, 11.2)]
+
+
 def test_fingerprint_covers_the_kernel_sources_and_is_stable():
     files = fingerprint.kernel_sources()
     assert "include/nvshmem_amd/device/nvshmemi_device.h" in files
